@@ -1,0 +1,694 @@
+/*
+ * CPU oracle for the per-rank compute half of five CATCCOS fused operators.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only tests, the smoke check
+ * and the benchmark's cpu_baseline leg may load it.  It restates, in plain C,
+ * the arithmetic of the reference's Python golden generators (paths relative to
+ * the reference tree):
+ *
+ *   formats / MX block quantiser  examples/utils/gen_mx_quant_allgather_data.py
+ *                                 :41-73 (emax, max), :79-128 (FP8 tables),
+ *                                 :168-189 (E8M0 exponent), :198-247 (table
+ *                                 rounding), :255-313 (FP8 rows), :352-449
+ *                                 (FP4 table, nibble packing, FP4 rows),
+ *                                 :497-503 (bf16 rounding)
+ *   int8 GEMM + dequant           examples/utils/gen_quant_data_mmdqrs.py:76-79
+ *   grouped int8 + SwiGLU         examples/utils/gen_data_dispatch_gmm_dequant_swiglu.py
+ *                                 :269-273 (swiglu), :298-320 (grouped GEMM,
+ *                                 per-channel, fp16 step, per-token, swiglu)
+ *   MX GEMM / grouped MX GEMM     examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/
+ *                                 gen_data_mxfp8_mmrs.py:299-356 and
+ *                                 examples/utils/gen_data_fp4_mx_alltoallv_gmm.py
+ *                                 :522-545 (nibbles), :586-620 (B scale layout),
+ *                                 :724-734 (grouped matmul)
+ *   token prefix sums             include/catccos/comm/block/comm_block_scheduler_alltoallv_gmm.hpp
+ *                                 :92-159
+ *   grouped tile order            include/catccos/dgemm/block/block_scheduler_alltoallv_allgather.hpp
+ *                                 :122-168 and include/catccos/catccos.hpp:141-163
+ *
+ * Parity status of each function is recorded next to it ("pinned by ...").
+ * Functions never pinned by an independent check would say "parity unpinned";
+ * none do at present except where marked.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_FMT_E4M3 0
+#define ORC_FMT_E5M2 1
+#define ORC_FMT_E2M1 2
+/* rounding rule of the payload cast */
+#define ORC_ROUND_RNE 0 /* nearest, ties to even code, sign of zero kept      */
+#define ORC_ROUND_LUT 1 /* nearest, ties to the smaller magnitude, zero is +0 */
+
+/* ------------------------------------------------------------------ bf16 */
+
+/* pinned by: torch.bfloat16 casts over random and special values */
+float orc_bf16_to_f32(uint16_t h)
+{
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* gen_mx_quant_allgather_data.py:497-503; NaN kept quiet as utils.py:68-87 */
+uint16_t orc_f32_to_bf16(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu)) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+/* ------------------------------------------------------- format decoders */
+
+/* Value of a small-float code with `eb` exponent bits, `mb` mantissa bits. */
+static float small_decode(uint32_t mag, int eb, int mb, int bias)
+{
+    uint32_t e = (mag >> mb) & ((1u << eb) - 1u);
+    uint32_t m = mag & ((1u << mb) - 1u);
+    if (e == 0) return ldexpf((float)m, 1 - bias - mb);
+    return ldexpf((float)((1u << mb) + m), (int)e - bias - mb);
+}
+
+/* E4M3 "fn": 0x7F / 0xFF are NaN, no infinities.
+ * pinned by: torch.float8_e4m3fn over all 256 codes */
+float orc_e4m3_decode(uint8_t c)
+{
+    uint32_t mag = c & 0x7Fu;
+    float v = (mag == 0x7Fu) ? NAN : small_decode(mag, 4, 3, 7);
+    return (c & 0x80u) ? -v : v;
+}
+
+/* E5M2: IEEE-like, exponent 31 is Inf/NaN.
+ * pinned by: torch.float8_e5m2 over all 256 codes */
+float orc_e5m2_decode(uint8_t c)
+{
+    uint32_t mag = c & 0x7Fu;
+    float v;
+    if (mag == 0x7Cu) v = INFINITY;
+    else if (mag > 0x7Cu) v = NAN;
+    else v = small_decode(mag, 5, 2, 15);
+    return (c & 0x80u) ? -v : v;
+}
+
+/* E2M1 nibble: magnitudes {0,.5,1,1.5,2,3,4,6}.
+ * pinned by: the closed list in gen_data_fp4_mx_alltoallv_gmm.py:99-129 */
+float orc_e2m1_decode(uint8_t nib)
+{
+    float v = small_decode(nib & 7u, 2, 1, 1);
+    return (nib & 8u) ? -v : v;
+}
+
+/* E8M0: 2^(b-127); 0xFF is NaN.  pinned by: torch.float8_e8m0fnu, 256 codes */
+float orc_e8m0_decode(uint8_t b)
+{
+    if (b == 0xFFu) return NAN;
+    return ldexpf(1.0f, (int)b - 127);
+}
+
+/* ------------------------------------------------------- format encoders */
+
+typedef struct {
+    int ncodes;        /* number of finite non-negative codes             */
+    float val[128];    /* val[i] = magnitude of code i, ascending          */
+    float maxv;
+    int emax;
+    uint32_t signbit;
+    uint8_t nan_code;
+} fmt_table;
+
+static fmt_table g_tab[3];
+static int g_tab_ready = 0;
+
+static void build_tables(void)
+{
+    if (g_tab_ready) return;
+    fmt_table *t = &g_tab[ORC_FMT_E4M3];
+    t->ncodes = 127; /* 0x00..0x7E */
+    for (int i = 0; i < 127; i++) t->val[i] = small_decode((uint32_t)i, 4, 3, 7);
+    t->maxv = 448.0f; t->emax = 8; t->signbit = 0x80u; t->nan_code = 0x7Fu;
+    t = &g_tab[ORC_FMT_E5M2];
+    t->ncodes = 124; /* 0x00..0x7B */
+    for (int i = 0; i < 124; i++) t->val[i] = small_decode((uint32_t)i, 5, 2, 15);
+    t->maxv = 57344.0f; t->emax = 15; t->signbit = 0x80u; t->nan_code = 0x7Fu;
+    t = &g_tab[ORC_FMT_E2M1];
+    t->ncodes = 8;
+    for (int i = 0; i < 8; i++) t->val[i] = small_decode((uint32_t)i, 2, 1, 1);
+    t->maxv = 6.0f; t->emax = 2; t->signbit = 0x8u; t->nan_code = 0x7u; /* E2M1 has no NaN */
+#pragma omp flush
+    g_tab_ready = 1;
+}
+
+/*
+ * Round an already-scaled value to the nearest code of the format.
+ *   clamp to +-max first (gen_mx_quant_allgather_data.py:284-285, :389),
+ *   nearest table entry (:214-233); on a tie RNE takes the even code,
+ *   the table rule takes the smaller magnitude (`<=`, :231);
+ *   the table rule writes +0 for every zero result (:236-243), RNE keeps the sign.
+ * NaN input gives the format's NaN code (E2M1: the maximum).
+ * pinned by: torch float8 casts (RNE) on dense sweeps incl. all midpoints;
+ *            brute-force argmin over the full table (table rule); idempotence
+ *            encode(decode(c)) == c for every code.
+ */
+uint8_t orc_encode(float y, int fmt, int rounding)
+{
+    build_tables();
+    const fmt_table *t = &g_tab[fmt];
+    uint32_t u;
+    memcpy(&u, &y, 4);
+    uint32_t neg = u >> 31;
+    if (y != y) return (uint8_t)((neg ? t->signbit : 0u) | t->nan_code);
+    float mag = fabsf(y);
+    if (mag > t->maxv) mag = t->maxv;
+    /* first index with val >= mag */
+    int lo = 0, hi = t->ncodes - 1;
+    while (lo < hi) {
+        int mid = (lo + hi) >> 1;
+        if (t->val[mid] < mag) lo = mid + 1; else hi = mid;
+    }
+    int up = lo, dn = up > 0 ? up - 1 : 0;
+    float du = t->val[up] - mag, dd = mag - t->val[dn];
+    int code;
+    if (dd < du) code = dn;
+    else if (du < dd) code = up;
+    else if (rounding == ORC_ROUND_LUT) code = dn;
+    else code = (dn & 1) ? up : dn;
+    if (code == 0 && rounding == ORC_ROUND_LUT) return 0;
+    return (uint8_t)(code | (neg ? t->signbit : 0u));
+}
+
+float orc_decode(uint8_t c, int fmt)
+{
+    if (fmt == ORC_FMT_E4M3) return orc_e4m3_decode(c);
+    if (fmt == ORC_FMT_E5M2) return orc_e5m2_decode(c);
+    return orc_e2m1_decode(c);
+}
+
+/* --------------------------------------------------------- E8M0 exponent */
+
+/*
+ * Shared exponent of one block from its absolute maximum
+ * (gen_mx_quant_allgather_data.py:168-189):
+ *   amax < 1e-12 -> 0 ; else clamp(floor(log2 amax) - emax, -128, 127),
+ * with floor(log2) read from the biased exponent field.  The byte is e+127;
+ * e = -128 cannot be written as E8M0 and is stored as byte 0 (2^-127).
+ * Inf/NaN maxima give byte 0xFF (comm_block_mx_quant.hpp:505).
+ * pinned by: 2^e <= amax/2^emax < 2^(e+1) over all positive bf16 maxima.
+ */
+int orc_shared_exp(float amax, int emax, int *is_nan)
+{
+    uint32_t u;
+    *is_nan = 0;
+    if (amax != amax || isinf(amax)) { *is_nan = 1; return 0; }
+    if (amax < 1e-12f) return 0;
+    memcpy(&u, &amax, 4);
+    int e = (int)((u >> 23) & 0xFFu) - 127 - emax;
+    if (e < -128) e = -128;
+    if (e > 127) e = 127;
+    return e;
+}
+
+static int fmt_emax(int fmt) { build_tables(); return g_tab[fmt].emax; }
+
+/*
+ * MX quantisation of a bf16 matrix [M,K] along its last axis, block 32
+ * (gen_mx_quant_allgather_data.py:255-313 for FP8, :385-449 for FP4).
+ *   payload  FP8: [M,K] bytes.  FP4: [M,ceil(K/2)] bytes, element 2j in the
+ *            low nibble, 2j+1 in the high nibble (:400-411).
+ *   scales   [M, 2*ceil(nblk/2)] E8M0 bytes; padding entries are 1.0 = 127
+ *            (:307-311).
+ * A ragged last block is zero padded (:267-273).
+ * pinned by: closed forms of its parts (above), scale-shift invariance,
+ *            idempotence on dequantised data (the check the reference's own
+ *            run.sh performs), torch-cast cross-check on random data.
+ */
+int orc_mx_quant_rows(const uint16_t *x, int64_t M, int64_t K, int fmt, int rounding,
+                      uint8_t *payload, uint8_t *scales)
+{
+    build_tables();
+    const int64_t nblk = (K + 31) / 32;
+    const int64_t sld = ((nblk + 1) / 2) * 2;
+    const int64_t pld = (fmt == ORC_FMT_E2M1) ? (K + 1) / 2 : K;
+    const int emax = fmt_emax(fmt);
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; m++) {
+        const uint16_t *xr = x + m * K;
+        uint8_t *pr = payload + m * pld;
+        uint8_t *sr = scales + m * sld;
+        if (fmt == ORC_FMT_E2M1) memset(pr, 0, (size_t)pld);
+        for (int64_t b = 0; b < sld; b++) {
+            if (b >= nblk) { sr[b] = 127; continue; }
+            int64_t k0 = b * 32, k1 = k0 + 32 < K ? k0 + 32 : K;
+            float amax = 0.0f;
+            int bad = 0;
+            for (int64_t k = k0; k < k1; k++) {
+                float v = fabsf(orc_bf16_to_f32(xr[k]));
+                if (v != v) bad = 1;
+                if (v > amax) amax = v;
+            }
+            int is_nan;
+            int e = orc_shared_exp(bad ? NAN : amax, emax, &is_nan);
+            if (is_nan) {
+                sr[b] = 0xFF;
+            } else {
+                sr[b] = (uint8_t)(e + 127 < 0 ? 0 : e + 127);
+            }
+            if (e < -127) e = -127;
+            for (int64_t k = k0; k < k1; k++) {
+                float v = orc_bf16_to_f32(xr[k]);
+                /* division by 2^e is exact in fp32 unless the quotient is subnormal */
+                float y = is_nan ? NAN : ldexpf(v, -e);
+                uint8_t q = orc_encode(y, fmt, rounding);
+                if (fmt == ORC_FMT_E2M1) pr[k >> 1] |= (uint8_t)(q << ((k & 1) * 4));
+                else pr[k] = q;
+            }
+        }
+    }
+    return 0;
+}
+
+/*
+ * MX quantisation of a bf16 matrix B [K,N] (row-major) along axis 0, as the
+ * reference prepares the right-hand GEMM operand
+ * (gen_data_mxfp8_mmrs.py:202-217 = quantise the transpose by rows;
+ * gen_data_fp4_mx_alltoallv_gmm.py:586-620).
+ *   trans_b = 0: payload [K,N] (FP4: [K,N/2], adjacent columns share a byte),
+ *                scales physical [ceil(K/64), N, 2]
+ *   trans_b = 1: payload [N,K] (FP4: [N,K/2]), scales [N, 2*ceil(K/64)]
+ * pinned by: equality with orc_mx_quant_rows on the explicit transpose.
+ */
+int orc_mx_quant_b(const uint16_t *b, int64_t K, int64_t N, int fmt, int rounding, int trans_b,
+                   uint8_t *payload, uint8_t *scales)
+{
+    const int64_t nblk = (K + 31) / 32;
+    const int64_t sld = ((nblk + 1) / 2) * 2;
+    const int fp4 = fmt == ORC_FMT_E2M1;
+    const int64_t pldT = fp4 ? (K + 1) / 2 : K;
+    uint16_t *bt = (uint16_t *)malloc((size_t)(N * K) * 2);
+    uint8_t *pt = (uint8_t *)malloc((size_t)(N * pldT));
+    uint8_t *st = (uint8_t *)malloc((size_t)(N * sld));
+    if (!bt || !pt || !st) { free(bt); free(pt); free(st); return -1; }
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; n++)
+        for (int64_t k = 0; k < K; k++) bt[n * K + k] = b[k * N + n];
+    orc_mx_quant_rows(bt, N, K, fmt, rounding, pt, st);
+    if (trans_b) {
+        memcpy(payload, pt, (size_t)(N * pldT));
+        memcpy(scales, st, (size_t)(N * sld));
+    } else {
+        const int64_t pld = fp4 ? (N + 1) / 2 : N;
+        if (fp4) memset(payload, 0, (size_t)(K * pld));
+#pragma omp parallel for schedule(static)
+        for (int64_t k = 0; k < K; k++)
+            for (int64_t n = 0; n < N; n++) {
+                if (fp4) {
+                    uint8_t q = (pt[n * pldT + (k >> 1)] >> ((k & 1) * 4)) & 0xF;
+                    payload[k * pld + (n >> 1)] |= (uint8_t)(q << ((n & 1) * 4));
+                } else {
+                    payload[k * N + n] = pt[n * K + k];
+                }
+            }
+        for (int64_t kb = 0; kb < sld; kb++)
+            for (int64_t n = 0; n < N; n++)
+                scales[((kb >> 1) * N + n) * 2 + (kb & 1)] = st[n * sld + kb];
+    }
+    free(bt); free(pt); free(st);
+    return 0;
+}
+
+/* Dequantise an MX row-quantised matrix back to fp32 [M,K]
+ * (gen_mx_quant_allgather_data.py:293; exact: small float times power of two).
+ * pinned by: round trip with orc_mx_quant_rows. */
+void orc_mx_dequant_rows(const uint8_t *payload, const uint8_t *scales, int64_t M, int64_t K, int fmt,
+                         float *out)
+{
+    const int64_t nblk = (K + 31) / 32;
+    const int64_t sld = ((nblk + 1) / 2) * 2;
+    const int64_t pld = (fmt == ORC_FMT_E2M1) ? (K + 1) / 2 : K;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; m++)
+        for (int64_t k = 0; k < K; k++) {
+            uint8_t q = (fmt == ORC_FMT_E2M1) ? (payload[m * pld + (k >> 1)] >> ((k & 1) * 4)) & 0xF
+                                              : payload[m * pld + k];
+            out[m * K + k] = orc_decode(q, fmt) * orc_e8m0_decode(scales[m * sld + k / 32]);
+        }
+}
+
+/* ------------------------------------------------------- int8 GEMM paths */
+
+static float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+/*
+ * out[m,n] = float(sum_k a[m,k]*b[k,n] as int32) * per_tok[m] * per_ch[n]
+ * (gen_quant_data_mmdqrs.py:76-79), stored as fp32 and, if out_bf16 != NULL,
+ * rounded to bf16.  `rows` (may be NULL = all) lists the output rows to
+ * compute; out row i holds rows[i].  B is [K,N] (trans_b=0) or [N,K].
+ * pinned by: int64 numpy matmul on small shapes (int32 sums are exact).
+ */
+void orc_gemm_i8_dequant(const int8_t *a, const int8_t *b, const float *per_tok, const float *per_ch,
+                         int64_t M, int64_t N, int64_t K, int trans_b, const int64_t *rows, int64_t nrows,
+                         float *out_f32, uint16_t *out_bf16)
+{
+    if (!rows) nrows = M;
+#pragma omp parallel
+    {
+        int32_t *acc = (int32_t *)malloc((size_t)N * 4);
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t i = 0; i < nrows; i++) {
+            int64_t m = rows ? rows[i] : i;
+            const int8_t *ar = a + m * K;
+            memset(acc, 0, (size_t)N * 4);
+            if (!trans_b) {
+                for (int64_t k = 0; k < K; k++) {
+                    int32_t av = ar[k];
+                    const int8_t *br = b + k * N;
+                    for (int64_t n = 0; n < N; n++) acc[n] += av * (int32_t)br[n];
+                }
+            } else {
+                for (int64_t n = 0; n < N; n++) {
+                    const int8_t *bc = b + n * K;
+                    int32_t s = 0;
+                    for (int64_t k = 0; k < K; k++) s += (int32_t)ar[k] * (int32_t)bc[k];
+                    acc[n] = s;
+                }
+            }
+            for (int64_t n = 0; n < N; n++) {
+                float v = (float)acc[n] * per_tok[m] * per_ch[n];
+                if (out_f32) out_f32[i * N + n] = v;
+                if (out_bf16) out_bf16[i * N + n] = orc_f32_to_bf16(v);
+            }
+        }
+        free(acc);
+    }
+}
+
+/* Round an fp32 value to the nearest IEEE half (ties to even) and widen it
+ * back.  pinned by: torch.float16 casts. */
+float orc_round_through_f16(float v)
+{
+    if (v != v) return v;
+    float a = fabsf(v);
+    if (a >= 65520.0f) return v < 0 ? -INFINITY : INFINITY;
+    int e;
+    (void)frexpf(a, &e);               /* a = f * 2^e, f in [0.5,1) */
+    int q = (e - 1 < -14 ? -14 : e - 1) - 10; /* spacing of halves near a is 2^q */
+    float r = ldexpf(rintf(ldexpf(a, -q)), q); /* rintf: ties to even in the default mode */
+    return v < 0 ? -r : r;
+}
+static float f32_to_f16_to_f32(float v) { return orc_round_through_f16(v); }
+
+/*
+ * Grouped int8 GEMM + per-channel dequant + per-token dequant + SwiGLU
+ * (gen_data_dispatch_gmm_dequant_swiglu.py:298-320, swiglu :269-273).
+ *   x [T,K] int8, rows of expert e are contiguous, group_sizes[e] rows each;
+ *   w [E,K,N] int8; per_ch [E,N]; per_tok [T];
+ *   c = float(acc) * per_ch[e,n]           (optionally rounded through fp16,
+ *                                           as the reference's :309-310)
+ *   c = c * per_tok[r]
+ *   out[r,j] = c[j] * sigmoid(c[j]) * c[j + N/2],  j < N/2  (first half = gate)
+ * Rows past sum(group_sizes) are zero (:319-320).
+ * pinned by: torch.nn.functional.silu on the fp32 intermediate + the pinned
+ *            int8 GEMM; per-group equality with the dense routine.
+ */
+void orc_gmm_i8_dequant_swiglu(const int8_t *x, const int8_t *w, const int32_t *group_sizes, int64_t E,
+                               int64_t T, int64_t K, int64_t N, const float *per_tok, const float *per_ch,
+                               int fp16_step, const int64_t *rows, int64_t nrows, float *out_f32,
+                               uint16_t *out_bf16)
+{
+    const int64_t H = N / 2;
+    int64_t *row_expert = (int64_t *)malloc((size_t)(T > 0 ? T : 1) * 8);
+    int64_t r = 0;
+    for (int64_t e = 0; e < E; e++)
+        for (int32_t i = 0; i < group_sizes[e] && r < T; i++) row_expert[r++] = e;
+    for (; r < T; r++) row_expert[r] = -1;
+    if (!rows) nrows = T;
+#pragma omp parallel
+    {
+        int32_t *acc = (int32_t *)malloc((size_t)N * 4);
+        float *c = (float *)malloc((size_t)N * 4);
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t i = 0; i < nrows; i++) {
+            int64_t m = rows ? rows[i] : i;
+            int64_t e = row_expert[m];
+            if (e < 0) {
+                for (int64_t j = 0; j < H; j++) {
+                    if (out_f32) out_f32[i * H + j] = 0.0f;
+                    if (out_bf16) out_bf16[i * H + j] = 0;
+                }
+                continue;
+            }
+            const int8_t *ar = x + m * K;
+            const int8_t *we = w + e * K * N;
+            memset(acc, 0, (size_t)N * 4);
+            for (int64_t k = 0; k < K; k++) {
+                int32_t av = ar[k];
+                const int8_t *br = we + k * N;
+                for (int64_t n = 0; n < N; n++) acc[n] += av * (int32_t)br[n];
+            }
+            for (int64_t n = 0; n < N; n++) {
+                float v = (float)acc[n] * per_ch[e * N + n];
+                if (fp16_step) v = f32_to_f16_to_f32(v);
+                c[n] = v * per_tok[m];
+            }
+            for (int64_t j = 0; j < H; j++) {
+                float g = c[j];
+                float v = g * sigmoidf_(g) * c[j + H];
+                if (out_f32) out_f32[i * H + j] = v;
+                if (out_bf16) out_bf16[i * H + j] = orc_f32_to_bf16(v);
+            }
+        }
+        free(acc);
+        free(c);
+    }
+    free(row_expert);
+}
+
+/* --------------------------------------------------------- MX GEMM paths */
+
+static inline uint8_t payload_at(const uint8_t *p, int64_t ld_elems, int64_t r, int64_t c, int fp4)
+{
+    if (fp4) {
+        int64_t ldb = (ld_elems + 1) / 2;
+        return (p[r * ldb + (c >> 1)] >> ((c & 1) * 4)) & 0xF;
+    }
+    return p[r * ld_elems + c];
+}
+
+/*
+ * Grouped (E >= 1) MX GEMM golden: C = deq(A) @ deq(B_e), fp32 accumulate
+ * (gen_data_mxfp8_mmrs.py:345-355; gen_data_fp4_mx_alltoallv_gmm.py:724-734),
+ *   deq(x)[m,k] = decode(q[m,k]) * 2^(s[m,k/32]-127).
+ *   a  payload [T,K] (FP4 [T,K/2]); sa [T, 2*ceil(K/64)]
+ *   b  per expert: trans_b=0 payload [K,N] (FP4 [K,N/2]), sb [ceil(K/64),N,2]
+ *                  trans_b=1 payload [N,K] (FP4 [N,K/2]), sb [N,2*ceil(K/64)]
+ *   group_sizes NULL means one dense problem (E must be 1).
+ * Rows past sum(group_sizes) are zero (:788-790).
+ * Accumulation runs over k in ascending order in fp32; `out_f64` (optional)
+ * receives the same sums accumulated in double for tolerance studies.
+ * pinned by: fp64 numpy matmul of independently dequantised operands on small
+ *            shapes; scales == 127 reduces to a plain FP8 GEMM; one-hot rows.
+ */
+void orc_mx_gmm(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb,
+                const int32_t *group_sizes, int64_t E, int64_t T, int64_t N, int64_t K, int fmt, int trans_b,
+                const int64_t *rows, int64_t nrows, float *out_f32, uint16_t *out_bf16, double *out_f64)
+{
+    const int fp4 = fmt == ORC_FMT_E2M1;
+    const int64_t nblk = (K + 31) / 32;
+    const int64_t sld = ((nblk + 1) / 2) * 2;
+    const int64_t b_bytes = fp4 ? (trans_b ? N * ((K + 1) / 2) : K * ((N + 1) / 2)) : K * N;
+    const int64_t sb_bytes = sld * N;
+    int64_t *row_expert = (int64_t *)malloc((size_t)(T > 0 ? T : 1) * 8);
+    if (group_sizes) {
+        int64_t r = 0;
+        for (int64_t e = 0; e < E; e++)
+            for (int32_t i = 0; i < group_sizes[e] && r < T; i++) row_expert[r++] = e;
+        for (; r < T; r++) row_expert[r] = -1;
+    } else {
+        for (int64_t r = 0; r < T; r++) row_expert[r] = 0;
+    }
+    if (!rows) nrows = T;
+#pragma omp parallel
+    {
+        float *arow = (float *)malloc((size_t)K * 4);
+        float *acc = (float *)malloc((size_t)N * 4);
+        double *acc64 = out_f64 ? (double *)malloc((size_t)N * 8) : NULL;
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t i = 0; i < nrows; i++) {
+            int64_t m = rows ? rows[i] : i;
+            int64_t e = row_expert[m];
+            for (int64_t n = 0; n < N; n++) { acc[n] = 0.0f; if (acc64) acc64[n] = 0.0; }
+            if (e >= 0) {
+                const uint8_t *be = b + e * b_bytes;
+                const uint8_t *sbe = sb + e * sb_bytes;
+                for (int64_t k = 0; k < K; k++)
+                    arow[k] = orc_decode(payload_at(a, K, m, k, fp4), fmt) * orc_e8m0_decode(sa[m * sld + k / 32]);
+                if (!trans_b) {
+                    for (int64_t k = 0; k < K; k++) {
+                        float av = arow[k];
+                        int64_t kb = k / 32;
+                        const uint8_t *srow = sbe + (kb >> 1) * N * 2 + (kb & 1);
+                        for (int64_t n = 0; n < N; n++) {
+                            float bv = orc_decode(payload_at(be, N, k, n, fp4), fmt) * orc_e8m0_decode(srow[n * 2]);
+                            acc[n] += av * bv;
+                            if (acc64) acc64[n] += (double)av * (double)bv;
+                        }
+                    }
+                } else {
+                    for (int64_t n = 0; n < N; n++) {
+                        float s = 0.0f;
+                        double s64 = 0.0;
+                        for (int64_t k = 0; k < K; k++) {
+                            float bv = orc_decode(payload_at(be, K, n, k, fp4), fmt) *
+                                       orc_e8m0_decode(sbe[n * sld + k / 32]);
+                            s += arow[k] * bv;
+                            s64 += (double)arow[k] * (double)bv;
+                        }
+                        acc[n] = s;
+                        if (acc64) acc64[n] = s64;
+                    }
+                }
+            }
+            for (int64_t n = 0; n < N; n++) {
+                if (out_f32) out_f32[i * N + n] = acc[n];
+                if (out_bf16) out_bf16[i * N + n] = orc_f32_to_bf16(acc[n]);
+                if (out_f64) out_f64[i * N + n] = acc64[n];
+            }
+        }
+        free(arow); free(acc); free(acc64);
+    }
+    free(row_expert);
+}
+
+/* ---------------------------------------------- token-count prefix sums */
+
+/* comm_block_scheduler_alltoallv_gmm.hpp:113-121: rows that source core
+ * `core_idx` has already sent to ranks below `rank`.
+ * pinned by: the reference's unit-test vector (test_comm_block_scheduler_alltoallv_gmm.cpp:96-102) */
+int32_t orc_sched_src_prev_sum(const int32_t *token_per_expert, int32_t rank, int32_t ep,
+                               int32_t expert_per_rank, uint32_t core_idx)
+{
+    int32_t s = 0;
+    if ((int64_t)core_idx < ep)
+        for (int32_t i = 0; i < rank * expert_per_rank; i++)
+            s += token_per_expert[(int64_t)core_idx * ep * expert_per_rank + i];
+    return s;
+}
+
+/* :92-105.  pinned by: the same unit-test vector */
+uint32_t orc_sched_comm_loops(int32_t ep, uint32_t core_idx, uint32_t core_num)
+{
+    if (core_num == 0) return 1;
+    uint32_t res = (uint32_t)ep / core_num;
+    if (core_idx < ((uint32_t)ep % core_num)) res++;
+    return res;
+}
+
+/* :123-128.  pinned by: the same unit-test vector */
+uint32_t orc_sched_block_offset_row(uint32_t core_idx, uint32_t core_num, uint32_t comm_idx)
+{
+    return core_idx + comm_idx * core_num;
+}
+
+/* :130-159: cumsum_mm[r][e] = sum_{r'<=r} token_per_expert[r'][rank*E_loc + e];
+ * the last row holds each local expert's total row count.
+ * pinned by: numpy cumsum (closed form) */
+void orc_sched_cumsum_mm(const int32_t *token_per_expert, int32_t rank, int32_t ep, int32_t expert_per_rank,
+                         int32_t *cumsum_mm)
+{
+    for (int32_t e = 0; e < expert_per_rank; e++) {
+        int32_t s = 0;
+        for (int32_t r = 0; r < ep; r++) {
+            s += token_per_expert[(int64_t)r * ep * expert_per_rank + rank * expert_per_rank + e];
+            cumsum_mm[r * expert_per_rank + e] = s;
+        }
+    }
+}
+
+/*
+ * Grouped-GEMM tile order on one device (source-rank dimension collapsed):
+ * groups are visited in expert order; group g has ceil(m_g/BM) x ceil(N/BN)
+ * tiles numbered row-major with every odd tile-row reversed
+ * (MatrixSwizzle<1,0>, catccos.hpp:141-163); tiles are dealt to `nblocks`
+ * workers round-robin with the remainder carried into the next group
+ * (block_scheduler_alltoallv_allgather.hpp:132-153), i.e. the global tile
+ * index modulo nblocks picks the worker.  Output rows of group g start at the
+ * exclusive prefix sum of the sizes (:66-73).
+ * Writes up to `cap` records {worker, group, row0, col0, rows, cols} and
+ * returns the total number of tiles.
+ * pinned by: partition invariants (every output element covered once, empty
+ *            groups give no tile) and hand-worked small cases.
+ */
+int64_t orc_grouped_tile_order(const int32_t *group_sizes, int64_t E, int64_t N, int32_t bm, int32_t bn,
+                               int32_t nblocks, int64_t cap, int64_t *rec)
+{
+    int64_t total = 0, row_base = 0;
+    int64_t gn = (N + bn - 1) / bn;
+    for (int64_t g = 0; g < E; g++) {
+        int64_t mg = group_sizes[g];
+        int64_t gm = (mg + bm - 1) / bm;
+        for (int64_t t = 0; t < gm * gn; t++) {
+            int64_t tr = t / gn, tc = t % gn;
+            if (tr & 1) tc = gn - 1 - tc;
+            if (total < cap) {
+                int64_t *q = rec + total * 6;
+                q[0] = total % nblocks;
+                q[1] = g;
+                q[2] = row_base + tr * bm;
+                q[3] = tc * bn;
+                q[4] = (mg - tr * bm) < bm ? (mg - tr * bm) : bm;
+                q[5] = (N - tc * bn) < bn ? (N - tc * bn) : bn;
+            }
+            total++;
+        }
+        row_base += mg;
+    }
+    return total;
+}
+
+/* ----------------------------------------------------- comparison metrics */
+
+/*
+ * Error metrics of verify_result.py:154-196 and the 1e-2 gate of the task:
+ *   m[0] = max |d-g| / max(|g|, 1)        (the reference's floor, :172)
+ *   m[1] = max |d-g| / max(|g|, rms(g))   (floor that is not vacuous for small g)
+ *   m[2] = mean((d-g)/max(1,|g|))         (the reference's "eb", :52-61)
+ *   m[3] = rms(g)
+ *   m[4] = fraction of elements with |d-g| > rtol*max(1,|g|)
+ * pinned by: numpy restatement on random data.
+ */
+void orc_compare(const float *d, const float *g, int64_t n, float rtol, double *m)
+{
+    double ss = 0.0;
+    for (int64_t i = 0; i < n; i++) ss += (double)g[i] * (double)g[i];
+    double rms = n ? sqrt(ss / (double)n) : 0.0;
+    double m0 = 0.0, m1 = 0.0, eb = 0.0;
+    int64_t bad = 0;
+    for (int64_t i = 0; i < n; i++) {
+        double dv = d[i], gv = g[i];
+        if (dv != dv || isinf(dv)) dv = 0.0;
+        if (gv != gv || isinf(gv)) gv = 0.0;
+        double diff = fabs(dv - gv), ag = fabs(gv);
+        double f1 = ag > 1.0 ? ag : 1.0, f2 = ag > rms ? ag : rms;
+        if (diff / f1 > m0) m0 = diff / f1;
+        if (f2 > 0.0 && diff / f2 > m1) m1 = diff / f2;
+        eb += (dv - gv) / f1;
+        if (diff > (double)rtol * f1) bad++;
+    }
+    m[0] = m0; m[1] = m1; m[2] = n ? eb / (double)n : 0.0; m[3] = rms; m[4] = n ? (double)bad / (double)n : 0.0;
+}
+
+int orc_num_threads(void)
+{
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}

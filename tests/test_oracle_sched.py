@@ -1,0 +1,56 @@
+"""Scheduler arithmetic: the reference's only numeric known-answer test, plus partition invariants."""
+import numpy as np
+
+import oracle as orc
+
+
+def test_reference_unit_test_vector():
+    """tests/comm_block_scheduler_alltoallv_gmm/test_comm_block_scheduler_alltoallv_gmm.cpp:37-102:
+    rank=2, EP=4, expertPerRank=2, tokenData[i]=i+1; expected 16 ints (entries 2,3 are the
+    freshly reset context)."""
+    tok = np.arange(1, 33, dtype=np.int32)
+    rank, ep, epr = 2, 4, 2
+    got = []
+    core, num = 1, 3
+    got += [core, num, 0, 0, orc.sched_src_prev_sum(tok, rank, ep, epr, core), orc.sched_comm_loops(ep, core, num),
+            orc.sched_block_offset_row(core, num, 0), orc.sched_block_offset_row(core, num, 1)]
+    core, num = 4, 6
+    got += [core, orc.sched_src_prev_sum(tok, rank, ep, epr, core), orc.sched_comm_loops(ep, core, num),
+            orc.sched_block_offset_row(core, num, 0)]
+    core, num = 0, 3
+    got += [core, orc.sched_src_prev_sum(tok, rank, ep, epr, core), orc.sched_comm_loops(ep, core, num),
+            orc.sched_block_offset_row(core, num, 1)]
+    assert got == [1, 3, 0, 0, 42, 1, 1, 4, 4, 0, 0, 4, 0, 10, 2, 3]
+
+
+def test_cumsum_mm_is_column_cumsum():
+    rng = np.random.default_rng(0)
+    ep, epr, rank = 4, 3, 1
+    tok = rng.integers(0, 50, ep * ep * epr).astype(np.int32)
+    got = orc.sched_cumsum_mm(tok, rank, ep, epr)
+    want = np.cumsum(tok.reshape(ep, ep * epr)[:, rank * epr:(rank + 1) * epr], axis=0)
+    assert np.array_equal(got, want)
+
+
+def test_tile_order_partitions_output_once():
+    gs = np.array([300, 0, 1, 128, 129, 0, 77], np.int32)
+    n, bm, bn, nb = 600, 128, 256, 5
+    rec = orc.grouped_tile_order(gs, n, bm, bn, nb)
+    cover = np.zeros((int(gs.sum()), n), np.int32)
+    starts = np.concatenate([[0], np.cumsum(gs)])
+    for i, (w, g, r0, c0, rows, cols) in enumerate(rec):
+        assert w == i % nb
+        assert starts[g] <= r0 and r0 + rows <= starts[g + 1] and rows > 0 and cols > 0
+        cover[r0:r0 + rows, c0:c0 + cols] += 1
+    assert np.all(cover == 1)
+    assert len(rec) == sum(-(-int(m) // bm) * -(-n // bn) for m in gs)
+    assert not np.any(np.isin(rec[:, 1], [1, 5]))  # empty groups yield no tile
+
+
+def test_tile_order_serpentine_small_case():
+    rec = orc.grouped_tile_order(np.array([3, 2], np.int32), 3, 1, 1, 2)
+    # group 0: 3x3 tiles, odd tile-rows reversed; group 1: 2x3
+    want_cols = [0, 1, 2, 2, 1, 0, 0, 1, 2, 0, 1, 2, 2, 1, 0]
+    want_rows = [0, 0, 0, 1, 1, 1, 2, 2, 2, 3, 3, 3, 4, 4, 4]
+    assert list(rec[:, 3]) == want_cols and list(rec[:, 2]) == want_rows
+    assert list(rec[:, 0]) == [i % 2 for i in range(15)]
