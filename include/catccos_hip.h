@@ -1,0 +1,89 @@
+/*
+ * catccos_hip.h -- C ABI of the MI355X (gfx950) compute library.
+ *
+ * One shared library (libcatccos_hip.so) exports the per-rank compute half of
+ * five CATCCOS fused operators.  All arguments are plain pointers and sizes;
+ * device pointers are HIP device addresses, `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream).  Every call returns 0 on success or a
+ * negative CCH_E* code; cch_last_error() then gives a message for the calling
+ * thread.  Kernel entry points only enqueue work; they never synchronise.
+ *
+ * Reference interfaces these entry points stand in for (paths relative to the
+ * reference tree) are cited on each declaration.
+ */
+#ifndef CATCCOS_HIP_H
+#define CATCCOS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* status codes */
+#define CCH_OK 0
+#define CCH_EINVAL (-1)   /* bad argument (shape, alignment, enum)          */
+#define CCH_EHIP (-2)     /* a HIP runtime call failed                      */
+#define CCH_ENODEV (-3)   /* no gfx950 device visible                       */
+#define CCH_ENOSUP (-4)   /* valid request this build does not implement    */
+
+/* payload formats (MX_QUANT_DTYPE of examples/ascend950_mx_quant_allgather/CMakeLists.txt:11-36) */
+#define CCH_FMT_E4M3 0
+#define CCH_FMT_E5M2 1
+#define CCH_FMT_E2M1 2
+
+/* payload rounding: 0 = round to nearest even, sign of zero kept (the device
+ * cast, include/catccos/comm/block/comm_block_mx_quant.hpp:596-642);
+ * 1 = the golden generator's table rule: ties to the smaller magnitude, zero
+ * always +0 (examples/utils/gen_mx_quant_allgather_data.py:198-247). */
+#define CCH_ROUND_RNE 0
+#define CCH_ROUND_LUT 1
+
+/* ---- runtime shims: what the host operator layer needs in place of acl.h ----
+ * Replace aclInit/aclrtSetDevice, aclrtMalloc/aclrtFree, aclrtMallocHost/
+ * aclrtFreeHost, aclrtMemcpy, aclrtMemset, aclrtCreateStream/
+ * aclrtSynchronizeStream/aclrtDestroyStream as used by utils/info.h:135-193 and
+ * examples/<op>/<op>_host.h. */
+int cch_init(int device);
+const char *cch_last_error(void);
+int cch_device_info(char *name, size_t name_len, int *compute_units, int *clock_mhz, uint64_t *hbm_bytes);
+int cch_malloc(void **ptr, size_t bytes);
+int cch_free(void *ptr);
+int cch_malloc_host(void **ptr, size_t bytes);
+int cch_free_host(void *ptr);
+int cch_memcpy_h2d(void *dst, const void *src, size_t bytes);
+int cch_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int cch_memset(void *dst, int value, size_t bytes);
+int cch_stream_create(void **stream);
+int cch_stream_sync(void *stream);
+int cch_stream_destroy(void *stream);
+
+/* ---- MX block quantisation (config 1) --------------------------------------
+ * Replaces the quantising half of Comm::Kernel::MxQuantAllGather
+ * (include/catccos/comm/kernel/mx_quant_allgather.hpp:165-212) and
+ * CommBlockMxQuant::ComputeMxQuant (include/catccos/comm/block/
+ * comm_block_mx_quant.hpp:414-663), launched in the reference by
+ * LaunchAscend950BF16QuantAllGatherFP8E4M3FN
+ * (tests/dynamic_tiling/impl/kernel_mxfp_ascend950.cpp:19).
+ *   x        bf16 [m,k] row-major
+ *   payload  FP8: [m,k] bytes; FP4: [m,ceil(k/2)], element 2j in the low nibble
+ *   scales   E8M0 [m, 2*ceil(k/64)]; entries past ceil(k/32) are 127 (=1.0)
+ * One scale per 32 consecutive elements of a row; a ragged last block is
+ * treated as zero padded. */
+int cch_mx_quant_rows(const void *x, void *payload, void *scales, int64_t m, int64_t k, int fmt, int rounding,
+                      void *stream);
+
+/* Same quantiser for a right-hand GEMM operand b [k,n] (row-major bf16) with
+ * blocks running down the k axis, i.e. what the reference's generators do for B
+ * (examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/gen_data_mxfp8_mmrs.py:202-217).
+ *   trans_b = 0: payload [k,n] (FP4 [k,n/2]), scales physical [ceil(k/64), n, 2]
+ *   trans_b = 1: payload [n,k] (FP4 [n,k/2]), scales [n, 2*ceil(k/64)]
+ * Requires k % 64 == 0 and n % 2 == 0. */
+int cch_mx_quant_b(const void *b, void *payload, void *scales, int64_t k, int64_t n, int fmt, int rounding,
+                   int trans_b, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CATCCOS_HIP_H */
