@@ -1,0 +1,139 @@
+// C ABI of the GEMM family: argument checks, problem description, kernel choice.
+#include <atomic>
+#include <cstring>
+
+#include "common.h"
+#include "gemm_common.h"
+
+namespace cch {
+int launch_gemm_naive(const GemmProblem &p, int kind, int epi, hipStream_t stream);
+int launch_gemm_tile(const GemmProblem &p, int kind, int epi, hipStream_t stream);
+bool gemm_tile_supports(const GemmProblem &p, int kind);
+
+static std::atomic<int> g_force_generic{0};
+
+static int run(const GemmProblem &p, int kind, int epi, hipStream_t stream)
+{
+    if (p.T == 0 || p.n_out == 0) return CCH_OK;
+    if (!g_force_generic.load() && gemm_tile_supports(p, kind)) return launch_gemm_tile(p, kind, epi, stream);
+    return launch_gemm_naive(p, kind, epi, stream);
+}
+
+static int check_shape(const char *who, int64_t t, int64_t n, int64_t k)
+{
+    CCH_REQUIRE(t >= 0 && n >= 0 && k >= 0, "%s: negative shape", who);
+    CCH_REQUIRE(t < ((int64_t)1 << 31) && n < ((int64_t)1 << 31) && k < ((int64_t)1 << 31), "%s: shape too large", who);
+    return CCH_OK;
+}
+}  // namespace cch
+
+using namespace cch;
+
+extern "C" {
+
+int cch_set_option(const char *name, int value)
+{
+    CCH_REQUIRE(name != nullptr, "cch_set_option: null name");
+    if (strcmp(name, "force_generic_gemm") == 0) {
+        g_force_generic.store(value);
+        return CCH_OK;
+    }
+    return fail(CCH_EINVAL, "cch_set_option: unknown option %s", name);
+}
+
+int cch_gemm_i8_dequant(const void *a, const void *b, const float *per_tok, const float *per_ch, void *out, int64_t m,
+                        int64_t n, int64_t k, int trans_b, void *stream)
+{
+    int rc = check_shape("cch_gemm_i8_dequant", m, n, k);
+    if (rc) return rc;
+    CCH_REQUIRE(trans_b == 0 || trans_b == 1, "cch_gemm_i8_dequant: trans_b %d", trans_b);
+    if (m == 0 || n == 0) return CCH_OK;
+    CCH_REQUIRE(out && per_tok && per_ch && (k == 0 || (a && b)), "cch_gemm_i8_dequant: null pointer");
+    GemmProblem p{};
+    p.a = static_cast<const uint8_t *>(a);
+    p.b = static_cast<const uint8_t *>(b);
+    p.per_tok = per_tok;
+    p.per_ch = per_ch;
+    p.out = static_cast<uint16_t *>(out);
+    p.num_groups = 1;
+    p.T = (int)m; p.N = (int)n; p.K = (int)k; p.n_out = (int)n;
+    p.trans_b = trans_b;
+    return run(p, KIND_I8, EPI_DEQUANT, static_cast<hipStream_t>(stream));
+}
+
+int cch_gmm_i8_dequant_swiglu(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok,
+                              const float *per_ch, void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k,
+                              int trans_b, void *stream)
+{
+    int rc = check_shape("cch_gmm_i8_dequant_swiglu", t, n, k);
+    if (rc) return rc;
+    CCH_REQUIRE(trans_b == 0 || trans_b == 1, "cch_gmm_i8_dequant_swiglu: trans_b %d", trans_b);
+    CCH_REQUIRE(n % 2 == 0, "cch_gmm_i8_dequant_swiglu: n=%lld must be even (gate | up halves)", (long long)n);
+    CCH_REQUIRE(num_experts >= 1 && num_experts <= 65535, "cch_gmm_i8_dequant_swiglu: num_experts=%lld", (long long)num_experts);
+    if (t == 0 || n == 0) return CCH_OK;
+    CCH_REQUIRE(out && per_tok && per_ch && group_sizes && (k == 0 || (x && w)), "cch_gmm_i8_dequant_swiglu: null pointer");
+    GemmProblem p{};
+    p.a = static_cast<const uint8_t *>(x);
+    p.b = static_cast<const uint8_t *>(w);
+    p.per_tok = per_tok;
+    p.per_ch = per_ch;
+    p.out = static_cast<uint16_t *>(out);
+    p.group_sizes = group_sizes;
+    p.num_groups = (int)num_experts;
+    p.T = (int)t; p.N = (int)n; p.K = (int)k; p.n_out = (int)(n / 2);
+    p.trans_b = trans_b;
+    p.b_stride = n * k;
+    return run(p, KIND_I8, EPI_DEQUANT_SWIGLU, static_cast<hipStream_t>(stream));
+}
+
+static int mx_problem(const char *who, GemmProblem &p, const void *a, const void *sa, const void *b, const void *sb,
+                      const int32_t *group_sizes, void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k,
+                      int fmt, int trans_b, int *kind)
+{
+    int rc = check_shape(who, t, n, k);
+    if (rc) return rc;
+    CCH_REQUIRE(trans_b == 0 || trans_b == 1, "%s: trans_b %d", who, trans_b);
+    CCH_REQUIRE(fmt == CCH_FMT_E4M3 || fmt == CCH_FMT_E5M2 || fmt == CCH_FMT_E2M1, "%s: unknown format %d", who, fmt);
+    CCH_REQUIRE(num_experts >= 1 && num_experts <= 65535, "%s: num_experts=%lld", who, (long long)num_experts);
+    CCH_REQUIRE(t == 0 || n == 0 || (a && sa && b && sb && out) || k == 0, "%s: null pointer", who);
+    const bool fp4 = fmt == CCH_FMT_E2M1;
+    CCH_REQUIRE(!fp4 || (k % 2 == 0 && n % 2 == 0), "%s: FP4 needs even k and n", who);
+    p.a = static_cast<const uint8_t *>(a);
+    p.sa = static_cast<const uint8_t *>(sa);
+    p.b = static_cast<const uint8_t *>(b);
+    p.sb = static_cast<const uint8_t *>(sb);
+    p.out = static_cast<uint16_t *>(out);
+    p.group_sizes = group_sizes;
+    p.num_groups = (int)num_experts;
+    p.T = (int)t; p.N = (int)n; p.K = (int)k; p.n_out = (int)n;
+    p.fmt = fmt;
+    p.trans_b = trans_b;
+    p.sld = (int)(2 * ((k + 63) / 64));
+    p.b_stride = fp4 ? n * k / 2 : n * k;
+    p.sb_stride = (int64_t)p.sld * n;
+    *kind = fp4 ? KIND_F4 : KIND_F8;
+    return CCH_OK;
+}
+
+int cch_mx_gemm(const void *a, const void *sa, const void *b, const void *sb, void *out, int64_t m, int64_t n, int64_t k,
+                int fmt, int trans_b, void *stream)
+{
+    GemmProblem p{};
+    int kind = 0;
+    int rc = mx_problem("cch_mx_gemm", p, a, sa, b, sb, nullptr, out, 1, m, n, k, fmt, trans_b, &kind);
+    if (rc) return rc;
+    return run(p, kind, EPI_PLAIN, static_cast<hipStream_t>(stream));
+}
+
+int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes, void *out,
+               int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, void *stream)
+{
+    GemmProblem p{};
+    int kind = 0;
+    CCH_REQUIRE(group_sizes != nullptr || t == 0, "cch_mx_gmm: null group_sizes");
+    int rc = mx_problem("cch_mx_gmm", p, a, sa, b, sb, group_sizes, out, num_experts, t, n, k, fmt, trans_b, &kind);
+    if (rc) return rc;
+    return run(p, kind, EPI_PLAIN, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

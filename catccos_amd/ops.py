@@ -82,3 +82,108 @@ def mx_quant_b(b, fmt="e4m3", rounding=ROUND_RNE, trans_b=0):
         scales = torch.empty((k // 64, n, 2), dtype=torch.uint8, device=b.device)
     check(_abi.lib().cch_mx_quant_b(_ptr(b), _ptr(payload), _ptr(scales), k, n, fmt, rounding, int(trans_b), _stream()))
     return payload, scales
+
+
+def set_option(name, value):
+    """Library switch (see cch_set_option in include/catccos_hip.h)."""
+    check(_abi.lib().cch_set_option(name.encode(), int(value)))
+
+
+def _check_2d(name, t, dtype):
+    if t.dim() != 2 or t.dtype != dtype:
+        raise ValueError("%s must be a 2-D %s tensor" % (name, dtype))
+
+
+def w8a8_matmul_dequant(a, b, per_tok, per_ch, trans_b=0):
+    """int8 [M,K] x int8 [K,N] (or [N,K] with trans_b=1) -> bf16 [M,N], scaled per token and per channel."""
+    _require_gpu(a, b, per_tok, per_ch)
+    _check_2d("a", a, torch.int8)
+    _check_2d("b", b, torch.int8)
+    a, b = a.contiguous(), b.contiguous()
+    m, k = a.shape
+    n = b.shape[0] if trans_b else b.shape[1]
+    if (b.shape[1] if trans_b else b.shape[0]) != k:
+        raise ValueError("inner dimensions differ: a %s, b %s, trans_b=%d" % (tuple(a.shape), tuple(b.shape), trans_b))
+    per_tok = per_tok.contiguous().float()
+    per_ch = per_ch.contiguous().float()
+    if per_tok.numel() != m or per_ch.numel() != n:
+        raise ValueError("per_tok must have M entries and per_ch N entries")
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    check(_abi.lib().cch_gemm_i8_dequant(_ptr(a), _ptr(b), _ptr(per_tok), _ptr(per_ch), _ptr(out), m, n, k,
+                                         int(trans_b), _stream()))
+    return out
+
+
+def gmm_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, trans_b=0):
+    """Grouped int8 matmul + dequant + SwiGLU: x int8 [T,K] grouped by expert, w int8 [E,K,N]
+    (or [E,N,K]), group_sizes int32 [E] on the device; returns bf16 [T, N/2]."""
+    _require_gpu(x, w, group_sizes, per_tok, per_ch)
+    _check_2d("x", x, torch.int8)
+    if w.dim() != 3 or w.dtype != torch.int8:
+        raise ValueError("w must be a 3-D int8 tensor")
+    if group_sizes.dtype != torch.int32 or group_sizes.dim() != 1:
+        raise ValueError("group_sizes must be a 1-D int32 tensor")
+    x, w, group_sizes = x.contiguous(), w.contiguous(), group_sizes.contiguous()
+    t, k = x.shape
+    e = w.shape[0]
+    n = w.shape[1] if trans_b else w.shape[2]
+    if (w.shape[2] if trans_b else w.shape[1]) != k or group_sizes.numel() != e:
+        raise ValueError("shape mismatch between x, w and group_sizes")
+    per_tok = per_tok.contiguous().float()
+    per_ch = per_ch.contiguous().float()
+    if per_tok.numel() != t or tuple(per_ch.shape) != (e, n):
+        raise ValueError("per_tok must be [T] and per_ch [E,N]")
+    out = torch.empty((t, n // 2), dtype=torch.bfloat16, device=x.device)
+    check(_abi.lib().cch_gmm_i8_dequant_swiglu(_ptr(x), _ptr(w), _ptr(group_sizes), _ptr(per_tok), _ptr(per_ch),
+                                               _ptr(out), e, t, n, k, int(trans_b), _stream()))
+    return out
+
+
+def _mx_shapes(a, sa, b, sb, fmt, trans_b, grouped):
+    fmt = _fmt(fmt)
+    fp4 = fmt == FMT_E2M1
+    _check_2d("a", a, torch.uint8)
+    _check_2d("sa", sa, torch.uint8)
+    t = a.shape[0]
+    k = a.shape[1] * (2 if fp4 else 1)
+    bs = b.shape[1:] if grouped else b.shape
+    if len(bs) != 2 or b.dtype != torch.uint8 or sb.dtype != torch.uint8:
+        raise ValueError("b / sb must be uint8 tensors of rank %d" % (3 if grouped else 2))
+    if trans_b:
+        n, kb = bs[0], bs[1] * (2 if fp4 else 1)
+    else:
+        kb, n = bs[0], bs[1] * (2 if fp4 else 1)
+    if kb != k:
+        raise ValueError("inner dimensions differ: a gives K=%d, b gives K=%d" % (k, kb))
+    if tuple(sa.shape) != (t, scale_cols(k)):
+        raise ValueError("sa must be [%d,%d]" % (t, scale_cols(k)))
+    e = b.shape[0] if grouped else 1
+    if sb.numel() != e * scale_cols(k) * n:
+        raise ValueError("sb has %d entries, expected %d" % (sb.numel(), e * scale_cols(k) * n))
+    return fmt, t, n, k, e
+
+
+def mx_matmul(a, sa, b, sb, fmt="e4m3", trans_b=0):
+    """MX dense GEMM: payload/scales as produced by mx_quant (a) and mx_quant_b (b); bf16 [M,N]."""
+    _require_gpu(a, sa, b, sb)
+    a, sa, b, sb = a.contiguous(), sa.contiguous(), b.contiguous(), sb.contiguous()
+    fmt, m, n, k, _ = _mx_shapes(a, sa, b, sb, fmt, trans_b, False)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    check(_abi.lib().cch_mx_gemm(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(out), m, n, k, fmt, int(trans_b), _stream()))
+    return out
+
+
+def mx_grouped_matmul(a, sa, b, sb, group_sizes, fmt="e4m3", trans_b=0):
+    """MX grouped GEMM: rows of a grouped by expert (group_sizes int32 [E] on the device),
+    b [E,...] / sb [E,...] one operand per expert; bf16 [T,N]."""
+    _require_gpu(a, sa, b, sb, group_sizes)
+    if group_sizes.dtype != torch.int32 or group_sizes.dim() != 1:
+        raise ValueError("group_sizes must be a 1-D int32 tensor")
+    a, sa, b, sb, group_sizes = a.contiguous(), sa.contiguous(), b.contiguous(), sb.contiguous(), group_sizes.contiguous()
+    fmt, t, n, k, e = _mx_shapes(a, sa, b, sb, fmt, trans_b, True)
+    if group_sizes.numel() != e:
+        raise ValueError("group_sizes must have one entry per expert")
+    out = torch.empty((t, n), dtype=torch.bfloat16, device=a.device)
+    check(_abi.lib().cch_mx_gmm(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(group_sizes), _ptr(out), e, t, n, k, fmt,
+                                int(trans_b), _stream()))
+    return out

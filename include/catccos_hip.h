@@ -83,6 +83,54 @@ int cch_mx_quant_rows(const void *x, void *payload, void *scales, int64_t m, int
 int cch_mx_quant_b(const void *b, void *payload, void *scales, int64_t k, int64_t n, int fmt, int rounding,
                    int trans_b, void *stream);
 
+/* ---- int8 W8A8 matmul + per-token x per-channel dequant (config 2) ----------
+ * Replaces LaunchAllGatherMatmulDequantINT8 (tests/dynamic_tiling/impl/kernel_int8.cpp:113-130)
+ * minus its allgather, i.e. FixpipeBlockMmad::operator()
+ * (include/catccos/dgemm/block/block_mmad_preload_fixpipe.hpp:151-379) followed by the
+ * per-token epilogue (include/catccos/epilogue/block/block_epilogue_per_token_dequant.hpp:247-266):
+ *   out[m,n] = bf16( float(sum_k a[m,k]*b[k,n]) * per_tok[m] * per_ch[n] )
+ *   a int8 [m,k]; b int8 [k,n] (trans_b=0) or [n,k] (trans_b=1); per_tok fp32 [m];
+ *   per_ch fp32 [n]; out bf16 [m,n]. */
+int cch_gemm_i8_dequant(const void *a, const void *b, const float *per_tok, const float *per_ch, void *out, int64_t m,
+                        int64_t n, int64_t k, int trans_b, void *stream);
+
+/* ---- MoE grouped W8A8 matmul + dequant + SwiGLU (config 4) -------------------
+ * Replaces the grouped GEMM of AlltoallvGmmDequantKernel::operator()<AIC>
+ * (include/catccos/dgemm/kernel/alltoallv_gmm_dequant_v2.hpp:164-244) and DequantSwigluKernel
+ * (examples/aux_ops/group_dequant_swiglu.h:91-168), fused:
+ *   rows of x are grouped by expert in expert order, group_sizes[e] rows each (device int32);
+ *   c = float(acc) * per_ch[e,n] * per_tok[r];  out[r,j] = silu(c[j]) * c[j+n/2], j < n/2
+ *   x int8 [t,k]; w int8 [E,k,n] (trans_b=0) or [E,n,k] (trans_b=1); per_ch fp32 [E,n];
+ *   out bf16 [t,n/2].  Rows past sum(group_sizes) are written as zeros. */
+int cch_gmm_i8_dequant_swiglu(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok,
+                              const float *per_ch, void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k,
+                              int trans_b, void *stream);
+
+/* ---- MX (FP8 / FP4 payload, E8M0 scales) dense GEMM (config 3) ---------------
+ * Replaces the compute half of MatmulReduceScatterMxTla::operator()<AIC>
+ * (include/catccos/dgemm/kernel/matmul_reduce_scatter_mx_tla.hpp:277-322), whose block MMAD
+ * lives in the absent catlass submodule:
+ *   out[m,n] = bf16( sum_k deq(a)[m,k] * deq(b)[k,n] ),  fp32 accumulation
+ *   a payload [m,k] (FP4 [m,k/2]); sa [m, 2*ceil(k/64)];
+ *   trans_b=0: b [k,n] (FP4 [k,n/2]), sb [ceil(k/64), n, 2]
+ *   trans_b=1: b [n,k] (FP4 [n,k/2]), sb [n, 2*ceil(k/64)] */
+int cch_mx_gemm(const void *a, const void *sa, const void *b, const void *sb, void *out, int64_t m, int64_t n, int64_t k,
+                int fmt, int trans_b, void *stream);
+
+/* ---- MX grouped matmul over variable-size expert groups (config 5) -----------
+ * Replaces the compute half of MxAllToAllVGroupedMatmulTla::operator()<AIC>
+ * (include/catccos/dgemm/kernel/mx_alltoallv_group_matmul.hpp:265-316) and its tile scheduler
+ * (include/catccos/dgemm/block/block_scheduler_alltoallv_allgather.hpp:27-233) with the
+ * source-rank dimension collapsed: rows of a are grouped by expert, group_sizes[e] rows each
+ * (device int32), b / sb hold num_experts operands back to back in the cch_mx_gemm layouts.
+ * Rows past sum(group_sizes) are written as zeros. */
+int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes, void *out,
+               int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, void *stream);
+
+/* Library switches for tests: "force_generic_gemm" = 1 routes every GEMM entry point through
+ * the shape-agnostic one-thread-per-element kernels instead of the tiled MFMA kernels. */
+int cch_set_option(const char *name, int value);
+
 #ifdef __cplusplus
 }
 #endif
