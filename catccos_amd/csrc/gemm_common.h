@@ -11,7 +11,7 @@ namespace cch {
 enum GemmKind { KIND_I8 = 0, KIND_F8 = 1, KIND_F4 = 2 };
 enum GemmEpilogue { EPI_PLAIN = 0, EPI_DEQUANT = 1, EPI_DEQUANT_SWIGLU = 2 };
 
-constexpr int MAX_GROUPS = 512;
+constexpr int MAX_GROUPS = 256;
 
 // One (dense or grouped) problem: out[T, n_out] = epilogue(A[T,K] x B_e[K,N]).
 struct GemmProblem {
