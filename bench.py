@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Headline benchmark: MXFP8 grouped GEMM (the MoE expert matmul of the
+ascend950_fp8_mx_alltoallv_grouped_matmul operator, one rank's share) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the grouped GEMM over one batch of synthetic input that is already
+resident in HBM: 16384 received tokens, 32 local experts with Zipf(1.1)-skewed group sizes
+(at least one empty), K = 7168, N = 4096, E4M3 payload with one E8M0 scale per 32 elements,
+fp32 accumulation, bf16 output.  Input quantisation is data preparation and is not timed.
+
+Prints ONE JSON line.  `value` is TFLOP/s of the whole job; `roofline` prices the GEMM kernel
+against the dense FP8 MFMA peak from HIP-event timing of the launches themselves;
+`cpu_baseline` is the CPU oracle (test infrastructure, used here only as the timed baseline)
+on a bounded sample of output rows of the same workload; `extra` carries the MX-quantiser
+line (HBM-bound) and the other configurations measured with the same library.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP8_PEAK_TFLOPS = 5000.0   # MI355X dense FP8 / INT8 MFMA, published
+FP4_PEAK_TFLOPS = 10100.0  # MI355X dense FP4 MFMA, published
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+
+
+def zipf_groups(rng, t, e):
+    """multinomial(t, p_e ~ (e+1)^-1.1) over permuted expert ids, with at least one empty group."""
+    import numpy as np
+    p = (np.arange(e) + 1.0) ** -1.1
+    p = p[rng.permutation(e)]
+    gs = rng.multinomial(t, p / p.sum()).astype(np.int32)
+    if gs.min() > 0:
+        i, j = int(gs.argmin()), int(gs.argmax())
+        gs[j] += gs[i]
+        gs[i] = 0
+    return gs
+
+
+def event_time_ms(fn, steps, warmup):
+    """Mean and per-launch durations of fn() on the current stream, by HIP events."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    per = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    return wall, per
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU's share of the grouped GEMM; this build has no multi-GPU path "
+                 "(the reference's communication stages are out of scope). Run with --gpus 1.")
+
+    import numpy as np
+    import torch
+    import catccos_amd as cc
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (MI355X); none is visible")
+    dev = "cuda"
+    torch.manual_seed(5)
+    rng = np.random.default_rng(5)
+
+    # ------------------------------------------------------------ workload (config 5 shapes, E4M3 payload)
+    E, T, K, N = 32, 16384, 7168, 4096
+    TRANS_B = 1   # W stored [E, N, K] (K-contiguous), the layout the reference's MXFP8 run uses (transB=1)
+    gs_host = zipf_groups(rng, T, E)
+    gs = torch.from_numpy(gs_host).to(dev)
+    x0 = (torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16)
+    a, sa = cc.mx_quant(x0, "e4m3")
+    b = torch.empty((E, N, K), dtype=torch.uint8, device=dev)
+    sb = torch.empty((E, N, K // 32), dtype=torch.uint8, device=dev)
+    for e in range(E):
+        w0 = (torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16)
+        b[e], sb[e] = cc.mx_quant_b(w0, "e4m3", trans_b=TRANS_B)
+    del x0, w0
+    torch.cuda.synchronize()
+
+    out = [None]
+
+    def step():
+        out[0] = cc.mx_grouped_matmul(a, sa, b, sb, gs, "e4m3", TRANS_B)
+
+    wall_ms, per_ms = event_time_ms(step, args.steps, args.warmup)
+    kernel_ms = float(np.mean(per_ms))
+    flop = 2.0 * T * N * K
+    value = flop / (wall_ms * 1e-3) / 1e12
+    achieved = flop / (kernel_ms * 1e-3) / 1e12
+
+    # size-independent sanity of the timed result: sampled rows against the oracle happen in the CPU leg below
+    result = {
+        "metric": "MXFP8 GMM TFLOP/s (% MFMA peak); MX-quant HBM GB/s (% of peak)",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "mxfp8 (e4m3 x e4m3, e8m0 scales, f32 accumulate, bf16 out)",
+        "data": "synthetic",
+        "config": {"workload": "MXFP8 grouped matmul, config-5 shapes with E4M3 payload", "experts": E, "tokens": T, "k": K,
+                   "n": N, "trans_b": TRANS_B, "group_sizes": gs_host.tolist()},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / FP8_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "gemm_tile_kernel<KIND_F8, EPI_PLAIN, E4M3>", "algorithmic_flop_per_launch": flop,
+                     "kernel_ms_min": round(float(np.min(per_ms)), 4), "kernel_ms_mean": round(kernel_ms, 4)},
+    }
+
+    # ------------------------------------------------------------ CPU baseline on a bounded sample of rows
+    if not args.no_cpu_baseline:
+        import oracle as orc
+        a_h, sa_h = a.cpu().numpy(), sa.cpu().numpy()
+        b_h, sb_h = b.cpu().numpy(), sb.cpu().numpy()
+        out_h = out[0].float().cpu().numpy()
+        used = int(gs_host.sum())
+        probe = np.sort(rng.choice(used, 8, replace=False)).astype(np.int64)
+        t0 = time.perf_counter()
+        orc.mx_gmm(a_h, sa_h, b_h, sb_h, N, K, orc.E4M3, TRANS_B, group_sizes=gs_host, rows=probe)
+        per_row = (time.perf_counter() - t0) / probe.size
+        nrows = int(min(used, max(16, 15.0 / max(per_row, 1e-6))))
+        rows = np.sort(rng.choice(used, nrows, replace=False)).astype(np.int64)
+        t0 = time.perf_counter()
+        gold = orc.mx_gmm(a_h, sa_h, b_h, sb_h, N, K, orc.E4M3, TRANS_B, group_sizes=gs_host, rows=rows)
+        dt = time.perf_counter() - t0
+        m = orc.compare(out_h[rows], gold)
+        result["cpu_baseline"] = {
+            "value": round(2.0 * nrows * N * K / dt / 1e12, 5), "unit": "TFLOP/s", "cores": orc.num_threads(), "kind": "port",
+            "sample": "%d of %d output rows (all %d columns, full K) of the same workload, %.1f s" % (nrows, T, N, dt),
+            "parity_on_sample": {"max_rel_err_floor1": m["max_rel_floor1"], "max_rel_err_floor_rms": m["max_rel_floor_rms"]},
+        }
+
+    # ------------------------------------------------------------ the other configurations, same library
+    if not args.no_extra:
+        extra = {}
+        # config 1: MX quantiser, rotating buffer sets larger than the 256 MB Infinity Cache
+        M1, K1 = 4096, 7168
+        sets = [torch.randn(M1, K1, device=dev).to(torch.bfloat16) for _ in range(6)]
+        idx = [0]
+
+        def qstep():
+            cc.mx_quant(sets[idx[0] % len(sets)], "e4m3")
+            idx[0] += 1
+
+        _, q_ms = event_time_ms(qstep, 60, 12)
+        qbytes = M1 * K1 * 2 + M1 * K1 + M1 * K1 // 32
+        q_gbs = qbytes / (float(np.mean(q_ms)) * 1e-3) / 1e9
+        extra["mx_quant_cfg1"] = {"gb_per_s": round(q_gbs, 1), "frac_of_hbm_peak": round(q_gbs / HBM_PEAK_GBS, 4),
+                                  "us": round(float(np.mean(q_ms)) * 1e3, 2), "bytes": qbytes, "buffers": "6 rotating sets (534 MB)"}
+        del sets
+        # config 2: int8 W8A8 + dequant
+        m2, k2, n2 = 8192, 4096, 8192
+        a2 = torch.randint(-127, 128, (m2, k2), dtype=torch.int8, device=dev)
+        b2 = torch.randint(-127, 128, (n2, k2), dtype=torch.int8, device=dev)
+        pt2 = torch.rand(m2, device=dev) * 0.019 + 0.001
+        pc2 = torch.rand(n2, device=dev) * 0.019 + 0.001
+        _, t2 = event_time_ms(lambda: cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, 1), 10, 3)
+        extra["w8a8_dequant_cfg2"] = {"tops": round(2.0 * m2 * n2 * k2 / (np.mean(t2) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t2)) * 1e3, 1)}
+        extra["w8a8_dequant_cfg2"]["frac_of_int8_peak"] = round(extra["w8a8_dequant_cfg2"]["tops"] / FP8_PEAK_TFLOPS, 4)
+        del a2, b2
+        # config 3: MXFP8 dense
+        m3, k3, n3 = 4096, 2048, 7168
+        a3, sa3 = cc.mx_quant(torch.randn(m3, k3, device=dev).to(torch.bfloat16), "e4m3")
+        b3, sb3 = cc.mx_quant_b(torch.randn(k3, n3, device=dev).to(torch.bfloat16), "e4m3", trans_b=1)
+        _, t3 = event_time_ms(lambda: cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", 1), 20, 5)
+        extra["mxfp8_dense_cfg3"] = {"tflops": round(2.0 * m3 * n3 * k3 / (np.mean(t3) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t3)) * 1e3, 1)}
+        extra["mxfp8_dense_cfg3"]["frac_of_fp8_peak"] = round(extra["mxfp8_dense_cfg3"]["tflops"] / FP8_PEAK_TFLOPS, 4)
+        # config 4: MoE W8A8 grouped + dequant + SwiGLU
+        e4, t4, k4, n4 = 16, 8192, 7168, 4096
+        gs4 = torch.from_numpy(zipf_groups(rng, t4, e4)).to(dev)
+        x4 = torch.randint(-127, 128, (t4, k4), dtype=torch.int8, device=dev)
+        w4 = torch.randint(-127, 128, (e4, n4, k4), dtype=torch.int8, device=dev)
+        pt4 = torch.rand(t4, device=dev) * 0.019 + 0.001
+        pc4 = torch.rand(e4, n4, device=dev) * 0.019 + 0.001
+        _, tt4 = event_time_ms(lambda: cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, 1), 10, 3)
+        extra["moe_w8a8_swiglu_cfg4"] = {"tops": round(2.0 * t4 * n4 * k4 / (np.mean(tt4) * 1e-3) / 1e12, 1), "us": round(float(np.mean(tt4)) * 1e3, 1)}
+        extra["moe_w8a8_swiglu_cfg4"]["frac_of_int8_peak"] = round(extra["moe_w8a8_swiglu_cfg4"]["tops"] / FP8_PEAK_TFLOPS, 4)
+        del x4, w4
+        # config 5: MXFP4 grouped (same groups as the headline)
+        a5, sa5 = cc.mx_quant((torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16), "e2m1")
+        b5 = torch.empty((E, N, K // 2), dtype=torch.uint8, device=dev)
+        sb5 = torch.empty((E, N, K // 32), dtype=torch.uint8, device=dev)
+        for e in range(E):
+            b5[e], sb5[e] = cc.mx_quant_b((torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16), "e2m1", trans_b=1)
+        _, t5 = event_time_ms(lambda: cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", 1), 10, 3)
+        extra["mxfp4_grouped_cfg5"] = {"tflops": round(flop / (np.mean(t5) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t5)) * 1e3, 1)}
+        extra["mxfp4_grouped_cfg5"]["frac_of_fp4_peak"] = round(extra["mxfp4_grouped_cfg5"]["tflops"] / FP4_PEAK_TFLOPS, 4)
+        result["extra"] = extra
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

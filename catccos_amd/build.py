@@ -65,8 +65,10 @@ def build_host():
     common = ["g++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-I" + os.path.join(ROOT, "include"), "-I" + host_dir]
     rpath = ["-L" + PKG, "-Wl,-rpath,$ORIGIN"]
     _run(common + ["-shared", "-o", HOST_LIB] + lib_srcs + rpath + ["-lcatccos_hip"])
+    # the operators and launchers register themselves from static initialisers of the host library,
+    # so the driver must keep the dependency although it names none of its symbols
     _run(common + ["-o", DRIVER, os.path.join(host_dir, "catccos_run.cpp")] + rpath +
-         ["-lcatccos_host", "-lcatccos_hip"])
+         ["-Wl,--no-as-needed", "-lcatccos_host", "-lcatccos_hip"])
     return HOST_LIB
 
 

@@ -1,0 +1,71 @@
+// Launch<Op><DType> functions with the reference's KernelFuncPtr signature
+// (tests/dynamic_tiling/include/launch_map.h:15-16; bodies there: impl/kernel_int8.cpp:113-130,
+// impl/kernel_mxfp_ascend950.cpp:19, impl/kernel_fp16_ascend950.cpp:592-612).  Each one maps the
+// KernelParams pointer roles of its operator onto one C-ABI call and, like DeviceDGemm::Run
+// (include/catccos/dgemm/device/device_dgemm.hpp:89-120), synchronises the stream before returning.
+#include "launch_map.h"
+
+namespace {
+void Finish(int rc, void *stream, const char *what)
+{
+    if (rc != CCH_OK) fprintf(stderr, "%s: cchError:%d %s\n", what, rc, cch_last_error());
+    CCH_CHECK(cch_stream_sync(stream));
+}
+struct AutoRegister {
+    AutoRegister(CocCommType type, CocDataType dtype, KernelFuncPtr fn) { KernelDispatcher::RegisterKernelFunc(type, dtype, fn); }
+};
+}  // namespace
+
+void LaunchAscend950BF16QuantAllGatherFP8E4M3FN(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
+                                                CocTilingParams &t, uint32_t, uint32_t)
+{
+    Finish(cch_mx_quant_rows(p.ptrA, p.ptrC, p.ptrB, t.m, t.n, CCH_FMT_E4M3, CCH_ROUND_RNE, stream), stream, "MxQuantAllGather");
+}
+
+void LaunchAllGatherMatmulDequantINT8(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
+                                      CocTilingParams &t, uint32_t, uint32_t transB)
+{
+    Finish(cch_gemm_i8_dequant(p.ptrA, p.ptrB, reinterpret_cast<const float *>(p.customPtrs[1]),
+                               reinterpret_cast<const float *>(p.customPtrs[0]), p.ptrC, t.m, t.n, t.k, (int)transB, stream),
+           stream, "AllGatherMatmulDequant");
+}
+
+void LaunchAscend950MxFp8MatmulReduceScatterFP8E4M3FN(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
+                                                      CocTilingParams &t, uint32_t, uint32_t transB)
+{
+    Finish(cch_mx_gemm(p.ptrA, p.customPtrs[0], p.ptrB, p.customPtrs[1], p.ptrC, t.m, t.n, t.k, CCH_FMT_E4M3, (int)transB, stream),
+           stream, "Ascend950MxFp8MatmulReduceScatter");
+}
+
+void LaunchDispatchGmmDequantSwigluINT8(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
+                                        CocTilingParams &t, uint32_t, uint32_t transB)
+{
+    Finish(cch_gmm_i8_dequant_swiglu(p.ptrA, p.ptrB, reinterpret_cast<const int32_t *>(p.customPtrs[1]),
+                                     reinterpret_cast<const float *>(p.customPtrs[2]),
+                                     reinterpret_cast<const float *>(p.customPtrs[0]), p.ptrC, t.expertNum, t.m, t.n, t.k,
+                                     (int)transB, stream),
+           stream, "DispatchGmmDequantSwiglu");
+}
+
+void LaunchAscend950Fp4MxAllToAllVGroupedMatmulBF16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
+                                                    CocTilingParams &t, uint32_t, uint32_t transB)
+{
+    Finish(cch_mx_gmm(p.ptrA, p.customPtrs[0], p.ptrB, p.customPtrs[1], reinterpret_cast<const int32_t *>(p.customPtrs[3]),
+                      p.ptrC, t.expertNum, t.m, t.n, t.k, CCH_FMT_E2M1, (int)transB, stream),
+           stream, "Ascend950Fp4MxAllToAllVGroupedMatmul");
+}
+
+void LaunchAscend950Fp8MxAllToAllVGroupedMatmulBF16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
+                                                    CocTilingParams &t, uint32_t, uint32_t transB)
+{
+    Finish(cch_mx_gmm(p.ptrA, p.customPtrs[0], p.ptrB, p.customPtrs[1], reinterpret_cast<const int32_t *>(p.customPtrs[3]),
+                      p.ptrC, t.expertNum, t.m, t.n, t.k, CCH_FMT_E4M3, (int)transB, stream),
+           stream, "Ascend950Fp8MxAllToAllVGroupedMatmul");
+}
+
+static AutoRegister s_reg0(MX_QUANT_ALLGATHER, FP8E4M3FN, &LaunchAscend950BF16QuantAllGatherFP8E4M3FN);
+static AutoRegister s_reg1(ALLGATHER_MATMUL_DEQUANT, INT8, &LaunchAllGatherMatmulDequantINT8);
+static AutoRegister s_reg2(ASCEND950_MXFP8_MATMUL_REDUCE_SCATTER, FP8E4M3FN, &LaunchAscend950MxFp8MatmulReduceScatterFP8E4M3FN);
+static AutoRegister s_reg3(DISPATCH_GMM_DEQUANT_SWIGLU, INT8, &LaunchDispatchGmmDequantSwigluINT8);
+static AutoRegister s_reg4(ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL, BF16, &LaunchAscend950Fp4MxAllToAllVGroupedMatmulBF16);
+static AutoRegister s_reg5(ASCEND950_FP8_MX_ALLTOALLV_GROUPED_MATMUL, BF16, &LaunchAscend950Fp8MxAllToAllVGroupedMatmulBF16);

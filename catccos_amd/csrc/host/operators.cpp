@@ -1,0 +1,249 @@
+// The host-side operators of the hot path, registered under the reference's registry names.
+// Each one knows its buffer sizes and data files for ONE rank's already-landed slice: the
+// communication stage of the reference operator is dropped, so rankSize only selects file names
+// and output offsets.  File names follow the reference's <op>_host.h files (cited per class);
+// all files are raw little-endian arrays without header.
+#include <cstdlib>
+#include <vector>
+
+#include "operator_registry.h"
+
+namespace {
+
+// Device buffer of `bytes`, filled from `path` (if `dataDir` is non-empty) or with `fillByte`.
+// `minFileBytes` > 0 accepts a shorter file (the rest keeps the fill value).
+uint8_t *LoadOrFill(size_t bytes, const std::string &dataDir, const std::string &name, int fillByte,
+                    size_t *fileBytes = nullptr)
+{
+    void *dev = nullptr;
+    CCH_CHECK(cch_malloc(&dev, bytes));
+    if (bytes == 0 || dev == nullptr) return static_cast<uint8_t *>(dev);
+    if (dataDir.empty()) {
+        CCH_CHECK(cch_memset(dev, fillByte, bytes));
+        return static_cast<uint8_t *>(dev);
+    }
+    void *host = nullptr;
+    CCH_CHECK(cch_malloc_host(&host, bytes));
+    if (host == nullptr) return static_cast<uint8_t *>(dev);
+    memset(host, fillByte, bytes);
+    size_t got = 0;
+    ReadFile(dataDir + "/" + name, host, bytes, &got);
+    if (fileBytes) *fileBytes = got;
+    CCH_CHECK(cch_memcpy_h2d(dev, host, bytes));
+    CCH_CHECK(cch_free_host(host));
+    return static_cast<uint8_t *>(dev);
+}
+
+uint8_t *DeviceAlloc(size_t bytes)
+{
+    void *dev = nullptr;
+    CCH_CHECK(cch_malloc(&dev, bytes));
+    return static_cast<uint8_t *>(dev);
+}
+
+void DumpDevice(const uint8_t *dev, size_t bytes, const std::string &path, size_t offset = 0)
+{
+    if (bytes == 0) return;
+    void *host = nullptr;
+    CCH_CHECK(cch_malloc_host(&host, bytes));
+    if (host == nullptr) return;
+    CCH_CHECK(cch_memcpy_d2h(host, dev, bytes));
+    WriteFile(path, host, bytes, offset);
+    CCH_CHECK(cch_free_host(host));
+}
+
+std::string R(uint32_t rank) { return std::to_string(rank); }
+size_t ScaleCols(size_t k) { return 2 * ((k + 63) / 64); }  // E8M0 bytes per row: block count padded to even
+
+// ---------------------------------------------------------------------------------------------
+// MX quantisation, bf16 -> FP8 E4M3 + E8M0 (reference examples/ascend950_mx_quant_allgather/
+// mx_quant_allgather_host.h:7-119).  ptrA = input, ptrB = scales, ptrC = payload.
+// Here `n` is the quantised (row) length, as in the reference.
+class MxQuantAllGatherOperator : public CatccosOperator {
+public:
+    void AllocateDeviceSpace(KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        const size_t m = t.m, n = t.n;
+        // constant fill: bf16 1.0 = 0x3F80 cannot be made by memset, 0x3C3C (~0.0115) can
+        uint8_t *in = LoadOrFill(m * n * 2, dataFile, "rank_" + R(rankId) + "_input.bin", 0x3C);
+        uint8_t *out = DeviceAlloc(m * n);
+        uint8_t *scale = DeviceAlloc(m * ScaleCols(n));
+        params.SetKernelParams(in, scale, out);
+    }
+    void WriteResultFile(const KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        const size_t m = t.m, n = t.n;
+        DumpDevice(params.ptrC, m * n, dataFile + "/rank_" + R(rankId) + "_output.bin");
+        DumpDevice(params.ptrB, m * ScaleCols(n), dataFile + "/rank_" + R(rankId) + "_mxscale.bin");
+    }
+    size_t GetWorkspaceSize(const CocTilingParams &) override { return 0; }
+    CocCommType GetActualKernelType(const CocTilingParams &) override { return MX_QUANT_ALLGATHER; }
+    bool CheckCocTilingParams(uint32_t, const CocTilingParams &t) override { return t.m > 0 && t.n > 0 && t.n % MX_BLOCK_SIZE == 0; }
+};
+
+// ---------------------------------------------------------------------------------------------
+// int8 matmul + dequant (reference examples/allgather_matmul_dequant/allgather_matmul_dequant_host.h:16-128).
+// ptrA = A int8 [m,k], ptrB = B int8 ([k,n] or, with transB, [n,k]), ptrC = out bf16 [m,n],
+// custom[0] = per-channel fp32 [n], custom[1] = per-token fp32 [m].
+// scale_gm.bin may hold fp32[n] or the reference's 64-bit fix-pipe words (low 32 bits = the fp32
+// scale, examples/utils/gen_allgather_fixpipe_quant_data.py:57-60); pertoken_scale_gm_rank<r>.bin
+// is this build's addition (fp32[m]; absent = all ones).
+class AllGatherMatmulDequantOperator : public CatccosOperator {
+public:
+    void AllocateDeviceSpace(KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        const size_t m = t.m, k = t.k, n = t.n;
+        uint8_t *a = LoadOrFill(m * k, dataFile, "a_gm_rank" + R(rankId) + ".bin", 1);
+        uint8_t *b = LoadOrFill(k * n, dataFile, "b_gm_rank" + R(rankId) + ".bin", 1);
+        uint8_t *d = DeviceAlloc(m * n * 2);
+        std::vector<float> perCh(n, 1.0f), perTok(m, 1.0f);
+        if (!dataFile.empty()) {
+            std::vector<uint64_t> raw(n, 0);
+            size_t got = 0;
+            if (ReadFile(dataFile + "/scale_gm.bin", raw.data(), n * 8, &got)) {
+                if (got == n * 8) {
+                    for (size_t i = 0; i < n; i++) {
+                        const uint32_t lo = static_cast<uint32_t>(raw[i]);
+                        memcpy(&perCh[i], &lo, 4);
+                    }
+                } else if (got == n * 4) {
+                    memcpy(perCh.data(), raw.data(), n * 4);
+                } else {
+                    ERROR_LOG("scale_gm.bin has %zu bytes, expected %zu or %zu", got, n * 4, n * 8);
+                }
+            }
+            struct stat st;
+            const std::string tokFile = dataFile + "/pertoken_scale_gm_rank" + R(rankId) + ".bin";
+            if (stat(tokFile.c_str(), &st) == 0) ReadFile(tokFile, perTok.data(), m * 4);
+        }
+        uint8_t *chDev = DeviceAlloc(n * 4), *tokDev = DeviceAlloc(m * 4);
+        CCH_CHECK(cch_memcpy_h2d(chDev, perCh.data(), n * 4));
+        CCH_CHECK(cch_memcpy_h2d(tokDev, perTok.data(), m * 4));
+        params.SetKernelParams(a, b, d, chDev, tokDev);
+    }
+    void WriteResultFile(const KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        DumpDevice(params.ptrC, static_cast<size_t>(t.m) * t.n * 2, dataFile + "/output_rank" + R(rankId) + ".bin");
+    }
+    size_t GetWorkspaceSize(const CocTilingParams &) override { return 0; }  // no B padding pass on this path
+    CocCommType GetActualKernelType(const CocTilingParams &) override { return ALLGATHER_MATMUL_DEQUANT; }
+    bool CheckCocTilingParams(uint32_t, const CocTilingParams &t) override { return t.m > 0 && t.n > 0 && t.k > 0; }
+};
+
+// ---------------------------------------------------------------------------------------------
+// MXFP8 dense GEMM (reference examples/ascend950_mxfp8_matmul_reduce_scatter/
+// ascend950_mxfp8_matmul_reduce_scatter_host.h:28-142).  ptrA/ptrB payloads, ptrC = out bf16,
+// custom[0] = scaleA [m, 2*ceil(k/64)], custom[1] = scaleB (layout by transB).
+// The result goes to output.bin at offset rank * bytes, as every rank of the reference does.
+class Ascend950MxFp8MatmulReduceScatterOperator : public CatccosOperator {
+public:
+    void AllocateDeviceSpace(KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        const size_t m = t.m, k = t.k, n = t.n, sc = ScaleCols(k);
+        const std::string p = "rank_" + R(rankId) + "_";
+        uint8_t *a = LoadOrFill(m * k, dataFile, p + "a.bin", 0x38);  // E4M3 1.0
+        uint8_t *b = LoadOrFill(k * n, dataFile, p + "b.bin", 0x38);
+        uint8_t *sa = LoadOrFill(m * sc, dataFile, p + "a_scale.bin", 127);
+        uint8_t *sb = LoadOrFill(n * sc, dataFile, p + "b_scale.bin", 127);
+        uint8_t *d = DeviceAlloc(m * n * 2);
+        params.SetKernelParams(a, b, d, sa, sb);
+    }
+    void WriteResultFile(const KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        const size_t bytes = static_cast<size_t>(t.m) * t.n * 2;
+        DumpDevice(params.ptrC, bytes, dataFile + "/output.bin", rankId * bytes);
+    }
+    size_t GetWorkspaceSize(const CocTilingParams &) override { return 0; }
+    CocCommType GetActualKernelType(const CocTilingParams &) override { return ASCEND950_MXFP8_MATMUL_REDUCE_SCATTER; }
+    bool CheckCocTilingParams(uint32_t, const CocTilingParams &t) override { return t.m > 0 && t.n > 0 && t.k > 0 && t.k % MX_BLOCK_SIZE == 0; }
+};
+
+// ---------------------------------------------------------------------------------------------
+// MoE grouped int8 matmul + dequant + SwiGLU (reference examples/dispatch_gmm_dequant_swiglu/
+// dispatch_gmm_dequant_swiglu_host.h:15-119).  The routing / dispatch stage is dropped: a_gm_<r>.bin
+// holds the int8 tokens this rank received, grouped by local expert ([m,k], m = rows received);
+// group_list_<r>.bin int32[expertNum] their counts; pertoken_scale_<r>.bin fp32[m].
+// ptrA = tokens, ptrB = W int8 [E,k,n] (transB: [E,n,k]), ptrC = out bf16 [m,n/2],
+// custom[0] = per-channel fp32 [E,n], custom[1] = group list, custom[2] = per-token fp32 [m].
+class DispatchGmmDequantSwigluOperator : public CatccosOperator {
+public:
+    void AllocateDeviceSpace(KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        const size_t m = t.m, k = t.k, n = t.n, e = t.expertNum;
+        uint8_t *a = LoadOrFill(m * k, dataFile, "a_gm_" + R(rankId) + ".bin", 1);
+        uint8_t *b = LoadOrFill(e * k * n, dataFile, "b_gm_" + R(rankId) + ".bin", 1);
+        uint8_t *d = DeviceAlloc(m * (n / 2) * 2);
+        std::vector<float> perCh(e * n, 1.0f), perTok(m, 1.0f);
+        std::vector<int32_t> groups(e, 0);
+        for (size_t i = 0; i < e; i++) groups[i] = static_cast<int32_t>(m / e + (i < m % e ? 1 : 0));
+        if (!dataFile.empty()) {
+            ReadFile(dataFile + "/scale_gm_" + R(rankId) + ".bin", perCh.data(), e * n * 4);
+            ReadFile(dataFile + "/pertoken_scale_" + R(rankId) + ".bin", perTok.data(), m * 4);
+            ReadFile(dataFile + "/group_list_" + R(rankId) + ".bin", groups.data(), e * 4);
+        }
+        uint8_t *chDev = DeviceAlloc(e * n * 4), *tokDev = DeviceAlloc(m * 4), *grpDev = DeviceAlloc(e * 4);
+        CCH_CHECK(cch_memcpy_h2d(chDev, perCh.data(), e * n * 4));
+        CCH_CHECK(cch_memcpy_h2d(tokDev, perTok.data(), m * 4));
+        CCH_CHECK(cch_memcpy_h2d(grpDev, groups.data(), e * 4));
+        params.SetKernelParams(a, b, d, chDev, grpDev, tokDev);
+    }
+    void WriteResultFile(const KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        DumpDevice(params.ptrC, static_cast<size_t>(t.m) * (t.n / 2) * 2, dataFile + "/output_" + R(rankId) + ".bin");
+    }
+    size_t GetWorkspaceSize(const CocTilingParams &) override { return 0; }
+    CocCommType GetActualKernelType(const CocTilingParams &) override { return DISPATCH_GMM_DEQUANT_SWIGLU; }
+    bool CheckCocTilingParams(uint32_t, const CocTilingParams &t) override
+    {
+        return t.m > 0 && t.k > 0 && t.n > 0 && t.n % 2 == 0 && t.expertNum > 0;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// MX grouped matmul, FP4 and FP8 payload (reference examples/ascend950_fp4_mx_alltoallv_grouped_matmul/
+// ascend950_fp4_mx_alltoallv_grouped_matmul_host.h:7-165 and its fp8 twin).  ptrA = tokens received
+// (grouped by local expert, m rows), ptrB = W [E,...], ptrC = out bf16 [m,n], custom[0] = scaleA,
+// custom[1] = scaleB, custom[2] = local_tokens_per_expert (unused on one rank),
+// custom[3] = global_tokens_per_local_expert int32 [rankSize, E_loc]; with the source-rank
+// dimension collapsed its first row is the group list.
+template <bool FP4, CocCommType KIND> class MxAllToAllVGroupedMatmulOperator : public CatccosOperator {
+public:
+    void AllocateDeviceSpace(KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        const size_t m = t.m, k = t.k, n = t.n, e = t.expertNum, sc = ScaleCols(k), pack = FP4 ? 2 : 1;
+        const int one = FP4 ? 0x22 : 0x38;  // payload 1.0 in either format
+        uint8_t *a = LoadOrFill(m * k / pack, dataFile, "input_a_" + R(rankId) + ".bin", one);
+        uint8_t *b = LoadOrFill(e * k * n / pack, dataFile, "input_b_" + R(rankId) + ".bin", one);
+        uint8_t *sa = LoadOrFill(m * sc, dataFile, "input_a_scale_" + R(rankId) + ".bin", 127);
+        uint8_t *sb = LoadOrFill(e * n * sc, dataFile, "input_b_scale_" + R(rankId) + ".bin", 127);
+        uint8_t *d = DeviceAlloc(m * n * 2);
+        std::vector<int32_t> groups(e, 0);
+        for (size_t i = 0; i < e; i++) groups[i] = static_cast<int32_t>(m / e + (i < m % e ? 1 : 0));
+        if (!dataFile.empty()) ReadFile(dataFile + "/global_tokens_per_local_expert_" + R(rankId) + ".bin", groups.data(), e * 4);
+        uint8_t *localDev = DeviceAlloc(e * 4), *grpDev = DeviceAlloc(e * 4);
+        CCH_CHECK(cch_memcpy_h2d(localDev, groups.data(), e * 4));
+        CCH_CHECK(cch_memcpy_h2d(grpDev, groups.data(), e * 4));
+        params.SetKernelParams(a, b, d, sa, sb, localDev, grpDev);
+    }
+    void WriteResultFile(const KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        DumpDevice(params.ptrC, static_cast<size_t>(t.m) * t.n * 2, dataFile + "/output_" + R(rankId) + ".bin");
+    }
+    size_t GetWorkspaceSize(const CocTilingParams &) override { return 0; }
+    CocCommType GetActualKernelType(const CocTilingParams &) override { return KIND; }
+    bool CheckCocTilingParams(uint32_t, const CocTilingParams &t) override
+    {
+        return t.m > 0 && t.k > 0 && t.n > 0 && t.k % 64 == 0 && t.expertNum > 0 && (!FP4 || t.n % 2 == 0);
+    }
+};
+using Ascend950Fp4MxAllToAllVGroupedMatmulOperator = MxAllToAllVGroupedMatmulOperator<true, ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL>;
+using Ascend950Fp8MxAllToAllVGroupedMatmulOperator = MxAllToAllVGroupedMatmulOperator<false, ASCEND950_FP8_MX_ALLTOALLV_GROUPED_MATMUL>;
+
+}  // namespace
+
+REGISTER_OPERATOR("MxQuantAllGather", MxQuantAllGatherOperator)
+REGISTER_OPERATOR("AllGatherMatmulDequant", AllGatherMatmulDequantOperator)
+REGISTER_OPERATOR("Ascend950MxFp8MatmulReduceScatter", Ascend950MxFp8MatmulReduceScatterOperator)
+REGISTER_OPERATOR("DispatchGmmDequantSwiglu", DispatchGmmDequantSwigluOperator)
+REGISTER_OPERATOR("Ascend950Fp4MxAllToAllVGroupedMatmul", Ascend950Fp4MxAllToAllVGroupedMatmulOperator)
+REGISTER_OPERATOR("Ascend950Fp8MxAllToAllVGroupedMatmul", Ascend950Fp8MxAllToAllVGroupedMatmulOperator)

@@ -1,0 +1,104 @@
+"""End-to-end through the C++ operator surface, the way the reference's run.sh scripts test an
+operator: write input .bin files, run the driver binary, compare the output files with the golden
+(here: the CPU oracle)."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from test_gpu_gemm import assert_close, rand_bf16, zipf_groups
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DRIVER = os.path.join(ROOT, "catccos_amd", "catccos_run")
+
+
+def drive(tmp_path, *args):
+    r = subprocess.run([DRIVER, *map(str, args)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "error num: 0" in r.stdout and "[ERROR]" not in r.stdout, r.stdout
+    assert "[PERF] Avg latency" in r.stdout
+
+
+def bf16_file(path, shape):
+    return orc.bf16_to_f32(np.fromfile(path, dtype=np.uint16)).reshape(shape)
+
+
+def test_mx_quant_files_byte_exact(tmp_path):
+    """Shapes of the reference's own list (ascend950_mx_quant_allgather/scripts/test_shapes.csv), shrunk in M."""
+    for m, n in ((512, 1024), (510, 1024)):
+        d = tmp_path / str(m)   # result files are written in place (no truncation), so one directory per shape
+        d.mkdir()
+        rng = np.random.default_rng(m)
+        x = rand_bf16(rng, (m, n))
+        x.tofile(d / "rank_0_input.bin")
+        drive(d, "mxqtag", m, 0, n, d, "--iters", 1, "--warmup", 1)
+        q, s = orc.mx_quant_rows(x, orc.E4M3)
+        assert np.array_equal(np.fromfile(d / "rank_0_output.bin", dtype=np.uint8).reshape(m, n), q)
+        assert np.array_equal(np.fromfile(d / "rank_0_mxscale.bin", dtype=np.uint8).reshape(m, n // 32), s)
+
+
+@pytest.mark.parametrize("fixpipe_words", [False, True])
+def test_int8_dequant_files(tmp_path, fixpipe_words):
+    m, k, n = 384, 512, 640
+    rng = np.random.default_rng(1)
+    a = rng.integers(-16, 16, (m, k)).astype(np.int8)      # the reference's data range
+    b = rng.integers(-16, 16, (k, n)).astype(np.int8)
+    pc = rng.uniform(0.001, 0.02, n).astype(np.float32)
+    pt = rng.uniform(0.001, 0.02, m).astype(np.float32)
+    a.tofile(tmp_path / "a_gm_rank0.bin")
+    b.tofile(tmp_path / "b_gm_rank0.bin")
+    if fixpipe_words:   # 64-bit words, low half = fp32 scale with 13 mantissa bits cleared
+        pc = (pc.view(np.uint32) & 0xFFFFE000).view(np.float32)
+        pc.view(np.uint32).astype(np.uint64).tofile(tmp_path / "scale_gm.bin")
+        pt[:] = 1.0
+    else:
+        pc.tofile(tmp_path / "scale_gm.bin")
+        pt.tofile(tmp_path / "pertoken_scale_gm_rank0.bin")
+    drive(tmp_path, "agmmdq", m, k, n, tmp_path, "--iters", 1, "--warmup", 0)
+    assert_close(bf16_file(tmp_path / "output_rank0.bin", (m, n)), orc.gemm_i8_dequant(a, b, pt, pc))
+
+
+def test_mxfp8_dense_files_rank_offset(tmp_path):
+    m, k, n = 256, 256, 384
+    rng = np.random.default_rng(2)
+    pa, sa = orc.mx_quant_rows(rand_bf16(rng, (m, k)), orc.E4M3)
+    pb, sb = orc.mx_quant_b(rand_bf16(rng, (k, n)), orc.E4M3, orc.RNE, 1)   # the reference's run uses transB=1
+    for name, arr in (("a", pa), ("b", pb), ("a_scale", sa), ("b_scale", sb)):
+        arr.tofile(tmp_path / f"rank_1_{name}.bin")
+    drive(tmp_path, "a5mxfp8mmrs", m, k, n, tmp_path, "--transB", 1, "--rank", 1, "--iters", 1, "--warmup", 0)
+    out = orc.bf16_to_f32(np.fromfile(tmp_path / "output.bin", dtype=np.uint16))
+    assert out.size == 2 * m * n                      # rank 1 wrote the second slice
+    assert_close(out[m * n:].reshape(m, n), orc.mx_gmm(pa, sa, pb, sb, n, k, orc.E4M3, 1))
+
+
+def test_dispatch_gmm_swiglu_files(tmp_path):
+    e, t, k, n = 4, 700, 256, 512
+    rng = np.random.default_rng(3)
+    gs = zipf_groups(rng, t, e)
+    x = rng.integers(-127, 128, (t, k)).astype(np.int8)
+    w = rng.integers(-16, 16, (e, k, n)).astype(np.int8)
+    pt = rng.uniform(0.001, 0.02, t).astype(np.float32)
+    pc = rng.uniform(0.001, 0.02, (e, n)).astype(np.float32)
+    x.tofile(tmp_path / "a_gm_0.bin"); w.tofile(tmp_path / "b_gm_0.bin"); pc.tofile(tmp_path / "scale_gm_0.bin")
+    pt.tofile(tmp_path / "pertoken_scale_0.bin"); gs.tofile(tmp_path / "group_list_0.bin")
+    drive(tmp_path, "dgds", t, k, n, tmp_path, "--experts", e, "--iters", 1, "--warmup", 0)
+    assert_close(bf16_file(tmp_path / "output_0.bin", (t, n // 2)), orc.gmm_i8_dequant_swiglu(x, w, gs, pt, pc))
+
+
+@pytest.mark.parametrize("kernel,fmt", [("a5fp4mxatavgmm", orc.E2M1), ("a5fp8mxatavgmm", orc.E4M3)])
+def test_mx_grouped_files(tmp_path, kernel, fmt):
+    """The reference's own shape for this operator: 1024 x 256 x 256, 4 experts (test_shapes.csv)."""
+    e, t, k, n = 4, 1024, 256, 256
+    rng = np.random.default_rng(4)
+    gs = zipf_groups(rng, t, e)
+    pa, sa = orc.mx_quant_rows(rand_bf16(rng, (t, k), 0.5), fmt)
+    pbs, sbs = zip(*[orc.mx_quant_b(rand_bf16(rng, (k, n), 0.5), fmt, orc.RNE, 0) for _ in range(e)])
+    pb, sb = np.stack(pbs), np.stack(sbs)
+    pa.tofile(tmp_path / "input_a_0.bin"); pb.tofile(tmp_path / "input_b_0.bin")
+    sa.tofile(tmp_path / "input_a_scale_0.bin"); sb.tofile(tmp_path / "input_b_scale_0.bin")
+    gs.tofile(tmp_path / "global_tokens_per_local_expert_0.bin")
+    drive(tmp_path, kernel, t, k, n, tmp_path, "--experts", e, "--iters", 1, "--warmup", 0)
+    assert_close(bf16_file(tmp_path / "output_0.bin", (t, n)), orc.mx_gmm(pa, sa, pb, sb, n, k, fmt, 0, group_sizes=gs))

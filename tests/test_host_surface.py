@@ -1,0 +1,58 @@
+"""Host operator surface (registry, dispatch keys, error convention) without a GPU."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DRIVER = os.path.join(ROOT, "catccos_amd", "catccos_run")
+
+# registry names and CocCommType values of the reference (utils/info.h:46-83, :242-275)
+EXPECT = {
+    "mxqtag": ("MxQuantAllGather", 24, 36),
+    "agmmdq": ("AllGatherMatmulDequant", 13, 2),
+    "a5mxfp8mmrs": ("Ascend950MxFp8MatmulReduceScatter", 18, 36),
+    "dgds": ("DispatchGmmDequantSwiglu", 21, 2),
+    "a5fp4mxatavgmm": ("Ascend950Fp4MxAllToAllVGroupedMatmul", 28, 27),
+    "a5fp8mxatavgmm": ("Ascend950Fp8MxAllToAllVGroupedMatmul", 27, 27),
+}
+
+
+def run(*args):
+    return subprocess.run([DRIVER, *args], capture_output=True, text=True, timeout=120)
+
+
+def test_driver_is_built():
+    assert os.path.exists(DRIVER), "build with python -m catccos_amd.build"
+
+
+def test_registry_and_dispatch_keys_match_reference():
+    out = run("--list")
+    assert out.returncode == 0
+    ops = {l.split()[1] for l in out.stdout.splitlines() if l.startswith("operator ")}
+    assert ops == {v[0] for v in EXPECT.values()}
+    seen = {}
+    for l in out.stdout.splitlines():
+        if l.startswith("launcher "):
+            f = l.split()
+            kv = dict(x.split("=") for x in f[2:])
+            seen[f[1]] = (kv["name"], int(kv["type"]), int(kv["dtype"]), int(kv["key"]))
+    for short, (name, ctype, dtype) in EXPECT.items():
+        assert seen[short] == (name, ctype, dtype, (ctype << 8) | dtype)
+
+
+def test_unknown_kernel_and_bad_shape_fail_like_the_reference_main():
+    r = run("nosuchkernel", "128", "128", "128", "-")
+    assert r.returncode != 0 and "[ERROR]" in r.stdout
+    r = run("mxqtag", "128", "0", "100", "-")   # n not a multiple of 32
+    assert r.returncode != 0 and "[ERROR]" in r.stdout
+    r = run("mxqtag")
+    assert r.returncode != 0 and "usage" in r.stdout
+
+
+def test_no_device_is_an_error_not_a_fallback():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    r = run("agmmdq", "128", "128", "128", "-")
+    assert r.returncode != 0 and "cch_init failed" in r.stdout
