@@ -68,6 +68,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--only", choices=["copy", "quant"], help="profiling aid: run only a 512 MiB device copy (counter "
+                    "calibration) or only the config-1 MX quantiser, print a short JSON line and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the grouped GEMM; this build has no multi-GPU path "
@@ -81,6 +83,25 @@ def main():
     dev = "cuda"
     torch.manual_seed(5)
     rng = np.random.default_rng(5)
+
+    if args.only == "copy":
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).fill_(7)
+        dst = torch.empty_like(src)
+        _, ms = event_time_ms(lambda: dst.copy_(src), args.steps, args.warmup)
+        print(json.dumps({"only": "copy", "bytes_read": src.numel(), "bytes_written": src.numel(), "ms": float(np.mean(ms))}))
+        return
+    if args.only == "quant":
+        sets = [torch.randn(4096, 7168, device=dev).to(torch.bfloat16) for _ in range(6)]
+        idx = [0]
+
+        def qonly():
+            cc.mx_quant(sets[idx[0] % len(sets)], "e4m3")
+            idx[0] += 1
+
+        _, ms = event_time_ms(qonly, args.steps, args.warmup)
+        qb = 4096 * 7168 * 3 + 4096 * 224
+        print(json.dumps({"only": "quant", "bytes": qb, "us": float(np.mean(ms)) * 1e3, "gb_per_s": qb / (float(np.mean(ms)) * 1e-3) / 1e9}))
+        return
 
     # ------------------------------------------------------------ workload (config 5 shapes, E4M3 payload)
     E, T, K, N = 32, 16384, 7168, 4096
