@@ -6,14 +6,22 @@
 // from the prefix sums of the group sizes (a dense problem is one group).
 //   * K advances in steps of 128 bytes per row, the size of an L2 line: direct-to-LDS loads
 //     that cover whole lines reach about 1.5x the L2 throughput of half-line requests.  The A
-//     and B panels of a step (256 rows x 128 B each) and, for MX, the E8M0 scales of the step
-//     go global -> LDS without a VGPR round trip into a ring of two stages; the requests for
-//     step k+1 are issued one instruction at a time between the MFMAs of step k.
+//     and B panels of a step (256 rows x 128 B each) go global -> LDS without a VGPR round
+//     trip into a ring of two stages.  A stage is read for the last time about 5/8 through
+//     its step; the requests that refill it (two steps ahead of use) follow the step's one
+//     barrier and are threaded between the remaining MFMAs.
+//   * MX scales travel 16 bytes per row at a time (4 MXFP8 steps, 2 MXFP4 steps) into a pair of
+//     scale buffers: a per-step 4-byte fetch touches one L2 line per lane and costs as many
+//     line requests as the whole data panel.
 //   * Each wave owns 128 x 64 outputs as 4 x 2 MFMA tiles of 32 x 32 and reads its fragments
-//     with 16-byte LDS reads from an XOR-swizzled panel layout (no bank conflicts).
-//   * The next tile's first step is requested before the current tile's epilogue.
+//     with 16-byte LDS reads from an XOR-swizzled panel layout (no bank conflicts).  Fragment
+//     registers are refilled as soon as the MFMAs that read them have been issued, so LDS
+//     latency hides behind the other MFMAs of the step.
+//   * The K loop is a single basic block without compiler-visible memory loads; the last two
+//     steps of a tile are peeled and request the next tile's first two steps, with empty
+//     buffer descriptors when there is no next tile, so they are branch-free as well.
 //   * Epilogues (dequant, SwiGLU, bf16 rounding) run on the accumulators; results pass through
-//     a wave-private 2 KiB LDS buffer so that every lane stores 16 contiguous bytes.
+//     a wave-private 1 KiB LDS buffer so that every lane stores 16 contiguous bytes.
 //
 // Stands in for Catlass::Gemm::Block::BlockMmadTla<MmadMx<...>> as instantiated in
 // examples/ascend950_fp4_mx_alltoallv_grouped_matmul/ascend950_fp4_mx_alltoallv_grouped_matmul_device.h:59-71,
@@ -50,10 +58,10 @@ constexpr int NJ = PANEL_BYTES / 1024 / NWAVES;  // direct-to-LDS instructions p
 
 // dynamic LDS map
 constexpr int RING_OFF = 0;
-constexpr int SCALE_OFF = RING_OFF + NSTAGE * STAGE_BYTES;   // per stage: up to 2 x (256 A + 256 B) dwords
-constexpr int SCALE_STAGE = 4096;
-constexpr int EPI_OFF = SCALE_OFF + NSTAGE * SCALE_STAGE;    // per wave: 16 rows x 64 bf16
-constexpr int EPI_WAVE = 2048;
+constexpr int SCALE_OFF = RING_OFF + NSTAGE * STAGE_BYTES;   // two buffers of (256 A + 256 B rows) x 16 scale bytes
+constexpr int SCALE_BUF = 8192;
+constexpr int EPI_OFF = SCALE_OFF + 2 * SCALE_BUF;           // per wave: 1 KiB of output staging
+constexpr int EPI_WAVE = 1024;
 constexpr int PARAM_OFF = EPI_OFF + NWAVES * EPI_WAVE;       // per tile parity: 256 per_tok + 256 per_ch floats
 constexpr int PARAM_SET = 2048;
 constexpr int LDS_BYTES = PARAM_OFF + 2 * PARAM_SET;         // 156 KiB of the CU's 160 KiB
@@ -92,13 +100,13 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 // would otherwise drain every outstanding direct-to-LDS load before each LDS read;
 // completion is tracked by the explicit vmcnt waits instead.
 typedef int Rsrc __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ Rsrc make_rsrc(const void *base)
+__device__ __forceinline__ Rsrc make_rsrc(const void *base, uint32_t bytes = 0x7FFFFFFFu)
 {
     const uint64_t b = reinterpret_cast<uint64_t>(base);
     Rsrc rs;
     rs[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
     rs[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));  // stride 0, no swizzle
-    rs[2] = 0x7FFFFFFF;                                                // num_records (bytes)
+    rs[2] = __builtin_amdgcn_readfirstlane((int)bytes);                // num_records (bytes); reads past it return 0
     rs[3] = 0x00020000;                                                // raw 32-bit data format
     return rs;
 }
@@ -109,7 +117,7 @@ __device__ __forceinline__ Rsrc scalar_rsrc(Rsrc rs)
     Rsrc u;
     u[0] = __builtin_amdgcn_readfirstlane(rs[0]);
     u[1] = __builtin_amdgcn_readfirstlane(rs[1]);
-    u[2] = 0x7FFFFFFF;
+    u[2] = __builtin_amdgcn_readfirstlane(rs[2]);
     u[3] = 0x00020000;
     return u;
 }
@@ -122,6 +130,22 @@ __device__ __forceinline__ void load16_to_lds(Rsrc rs, uint32_t voff, uint32_t s
                  :
                  : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
                  : "memory", "m0");
+}
+// The same 16-byte load, performed only when `enable` (wave-uniform) is non-zero, without a
+// branch: the load is issued with an empty EXEC mask otherwise.  Keeps the K loop one basic
+// block, which the register allocator handles far better than a loop with a diamond in it.
+__device__ __forceinline__ void load16_to_lds_if(int enable, Rsrc rs, uint32_t voff, uint32_t soff, uint32_t lds_addr)
+{
+    rs = scalar_rsrc(rs);
+    soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
+    lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
+    enable = __builtin_amdgcn_readfirstlane(enable);
+    uint64_t saved;
+    asm volatile("s_mov_b64 %0, exec\n\ts_cmp_lg_u32 %1, 0\n\ts_cselect_b64 exec, %0, 0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\t"
+                 "buffer_load_dwordx4 %3, %4, %5 offen lds\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved)
+                 : "s"(enable), "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
+                 : "memory", "m0", "scc");
 }
 __device__ __forceinline__ void load4_to_lds(Rsrc rs, uint32_t voff, uint32_t soff, uint32_t lds_addr)
 {
@@ -144,6 +168,7 @@ __device__ __forceinline__ uint32_t swizzle_of_row(int row) { return (uint32_t)(
 // What one tile needs, all wave-uniform except the per-lane source offsets.
 struct TileCtx {
     int valid, e, m0, m_end, j0;
+    uint32_t lim;                       // descriptor size: 0 for a tile past the end, whose requests then fetch nothing
     Rsrc rs_a, rs_b, rs_sc;             // buffer descriptors: A rows from m0, B of the expert, scales
     uint32_t off_a[NJ], off_b[NJ];      // per lane: source row * pitch + chunk * 16
     uint32_t off_sc;                    // per lane: scale row * sld (A rows for waves 0-3, B columns for 4-7)
@@ -159,12 +184,14 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;   // output columns per tile
     constexpr int WN_OUT = SWIGLU ? WN / 2 : WN;   // output columns per wave
     constexpr int SCALE_DW = KT::SCALE_DW;         // scale dwords per row per step
-    constexpr int NV = 2 * NJ + SCALE_DW;          // direct-to-LDS instructions per wave per step
+    constexpr int NV = 2 * NJ;                     // direct-to-LDS instructions per wave per step
+    // MX scales travel 16 bytes per row at a time: one request per wave covers SPG steps
+    constexpr int SPG = SCALE_DW > 0 ? 4 / SCALE_DW : 1;
     constexpr int CBSZ = FMT == CCH_FMT_E2M1 ? 4 : (FMT == CCH_FMT_E5M2 ? 1 : 0);
     constexpr int ROWB = WN_OUT * 2;               // epilogue staging: bytes per row
     constexpr int CPR = ROWB / 16;                 // 16-byte chunks per staged row
-    constexpr int RPI = 64 / CPR;                  // rows covered by one read-back instruction
-    constexpr int NSTORES = MT * 2 * (16 / RPI);   // 16-byte stores per lane per tile
+    constexpr int PASS_ROWS = 64 / CPR;            // rows staged per pass: 1 KiB, one read-back instruction
+    constexpr int NPASS = 32 / PASS_ROWS;          // passes per 32-row MFMA tile
     constexpr int NP = EPI != EPI_PLAIN ? 2 : 0;   // extra requests in a tile's first batch (epilogue parameters)
 
     __shared__ GroupTable tab;
@@ -186,18 +213,25 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     // LDS read offsets of this lane inside a stage.
     const uint32_t swz = swizzle_of_row(r);
     const uint32_t rd_a = (uint32_t)(wm * WM + r) * BKB, rd_b = (uint32_t)PANEL_BYTES + (uint32_t)(wn * WN + r) * BKB;
-    const uint32_t rd_sa = (uint32_t)(wm * WM + r) * 4, rd_sb = 1024u + (uint32_t)(wn * WN + r) * 4;
+    const uint32_t rd_sa = (uint32_t)(wm * WM + r) * 16, rd_sb = 4096u + (uint32_t)(wn * WN + r) * 16;
+
+    int gi = 0;           // scale groups requested so far; group n lives in scale buffer n & 1
+    int gbase = 0;        // value of gi when the current tile's group 0 was requested
 
     auto decode = [&](int t, TileCtx &c) {
+        // A tile index past the end decodes to the last tile with empty descriptors: its requests
+        // can then be issued unconditionally (they read nothing and write zeros into LDS areas
+        // that are never used), which keeps the peeled steps free of branches.
         c.valid = t < total_tiles;
-        if (!c.valid) return;
+        c.lim = c.valid ? 0x7FFFFFFFu : 0u;
+        t = max(min(t, total_tiles - 1), 0);
         const int tr = t / n_tiles, nt = t - tr * n_tiles;
         c.e = uniform(find_group(tab, p.num_groups, tr));
         c.m0 = uniform(tab.row_start[c.e] + (tr - tab.tile_start[c.e]) * BM);
         c.m_end = uniform(tab.row_start[c.e + 1]);
         c.j0 = nt * BN_OUT;
-        c.rs_a = make_rsrc(p.a + (size_t)c.m0 * lda);
-        c.rs_b = make_rsrc(p.b + (size_t)c.e * p.b_stride);
+        c.rs_a = make_rsrc(p.a + (size_t)c.m0 * lda, c.lim);
+        c.rs_b = make_rsrc(p.b + (size_t)c.e * p.b_stride, c.lim);
         // Instruction j of this wave fills rows (wave*NJ + j)*8 .. +7 of a panel; lane l lands at
         // row l/8, chunk position l%8 and must therefore fetch chunk (l%8) ^ swizzle(row).  Rows
         // past the edge re-read the last valid row; their products land in accumulators that are
@@ -219,10 +253,10 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         if (MX) {
             const int idx = (wave & 3) * 64 + lane;
             if (wave < 4) {
-                c.rs_sc = make_rsrc(p.sa + (size_t)c.m0 * p.sld);
+                c.rs_sc = make_rsrc(p.sa + (size_t)c.m0 * p.sld, (uint32_t)min((int64_t)(p.T - c.m0) * p.sld, (int64_t)c.lim));
                 c.off_sc = (uint32_t)min(idx, c.m_end - 1 - c.m0) * (uint32_t)p.sld;
             } else {
-                c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride);
+                c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride, (uint32_t)min((int64_t)p.N * p.sld, (int64_t)c.lim));
                 c.off_sc = (uint32_t)min(c.j0 + idx, p.N - 1) * (uint32_t)p.sld;
             }
         }
@@ -238,13 +272,14 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             load16_to_lds(c.rs_a, c.off_a[piece], (uint32_t)kt * BKB, lds + piece * 1024u);
         } else if constexpr (piece < 2 * NJ) {
             load16_to_lds(c.rs_b, c.off_b[piece - NJ], (uint32_t)kt * BKB, lds + PANEL_BYTES + (piece - NJ) * 1024u);
-        } else if constexpr (piece < NV) {
-            // dword d of the step's scales: 4 E8M0 bytes per row
-            constexpr int d = piece - 2 * NJ;
-            load4_to_lds(c.rs_sc, c.off_sc, (uint32_t)(kt * SCALE_DW + d) * 4u,
-                         lds_base + (uint32_t)(SCALE_OFF + stage * SCALE_STAGE + d * 2048) + (uint32_t)(wave >= 4) * 1024u +
-                             (uint32_t)(wave & 3) * 256u);
         }
+    };
+    // Scale group `grp` of tile c (16 bytes per row: steps grp*SPG .. grp*SPG+SPG-1) into scale
+    // buffer `buf`; waves 0-3 fetch the A rows, waves 4-7 the B rows, one row per lane.
+    auto issue_scales = [&](int enable, const TileCtx &c, int grp, int buf) {
+        if constexpr (MX)
+            load16_to_lds_if(enable, c.rs_sc, c.off_sc, (uint32_t)grp * 16u,
+                             lds_base + (uint32_t)(SCALE_OFF + buf * SCALE_BUF) + (uint32_t)(wave >= 4) * 4096u + (uint32_t)(wave & 3) * 1024u);
     };
     auto issue_step = [&](const TileCtx &c, int kt, int stage) {
         static_for<NV>([&](auto piece_c) { issue_piece(c, kt, stage, piece_c); });
@@ -257,12 +292,14 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             const int idx = (wave & 3) * 64 + lane;
             // destination of lane 0 of this wave; lane l lands 4*l bytes further
             const uint32_t dst = lds_base + (uint32_t)(PARAM_OFF + parity * PARAM_SET) + (uint32_t)(wave & 3) * 256u;
-            load4_to_lds(make_rsrc(p.per_tok + c.m0), (uint32_t)min(idx, c.m_end - 1 - c.m0) * 4u, 0u, dst);
+            load4_to_lds(make_rsrc(p.per_tok + c.m0, c.lim), (uint32_t)min(idx, c.m_end - 1 - c.m0) * 4u, 0u, dst);
             int col;
             if (SWIGLU) col = ((idx >> 5) & 1) * p.n_out + min(c.j0 + (idx >> 6) * 32 + (idx & 31), p.n_out - 1);
             else col = min(c.j0 + idx, p.N - 1);
-            load4_to_lds(make_rsrc(p.per_ch + (size_t)c.e * p.N), (uint32_t)col * 4u, 0u, dst + 1024u);
+            load4_to_lds(make_rsrc(p.per_ch + (size_t)c.e * p.N, c.lim), (uint32_t)col * 4u, 0u, dst + 1024u);
         }
+        issue_scales(1, c, 0, gi & 1);
+        gi++;
         issue_step(c, 0, stage);
     };
 
@@ -272,15 +309,10 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     bool first = true;
     decode(t, cur);
     nxt.valid = 0;
-    if (cur.valid) setup(cur, 0, 0);
-
-#ifdef DBG_TIMING
-#define TSTAMP(slot) do { if (t == 2 * (int)gridDim.x && blockIdx.x == 0 && kt >= 16 && kt < 32) { \
-        unsigned long long ts_ = __builtin_readcyclecounter(); \
-        if (lane == 0) *reinterpret_cast<unsigned long long *>(smem + EPI_OFF + ((wave * 16 + (kt - 16)) * 4 + (slot)) * 8) = ts_; } } while (0)
-#else
-#define TSTAMP(slot) do { } while (0)
-#endif
+    if (cur.valid) {
+        setup(cur, 0, 0);
+        issue_step(cur, 1, 1);
+    }
     while (cur.valid) {
         Acc acc[MT][NT];
 #pragma unroll
@@ -290,8 +322,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 #pragma unroll
                 for (int x = 0; x < 16; x++) acc[i][j][x] = 0;
 
-        v8i fb[NT], fa[MT];              // B and A fragments of the current 64-byte substep
-        uint32_t sc[SCALE_DW > 0 ? SCALE_DW : 1][MT + NT];  // raw scale dwords of the current step
+        int nbase = 0;  // gi when the next tile's scale group 0 is requested
+        // Fragment registers.  fa[i] and fb0 hold the first 64-byte substep of the current
+        // step, fb1 the second; fa[i] is refilled with its next contents as soon as the MFMAs
+        // that read it have been issued, so that LDS latency hides behind the other MFMAs.
+        v8i fa[MT], fb0[NT], fb1[NT];
+        constexpr int NSC = SCALE_DW > 0 ? SCALE_DW : 1;
+        uint32_t sc[NSC][MT + NT];  // raw scale dwords of the current step
 
         auto read_frag = [&](uint32_t row_off, int ks) {
             // lane (r, g) feeds K bytes [16g, 16g+16) of each 32-byte half of the 64-byte substep
@@ -299,126 +336,142 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             const v4i lo = lds_read16(row_off + c0), hi = lds_read16(row_off + c1);
             return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         };
-        auto read_substep = [&](int stage, int ks) {
-            const uint32_t st = (uint32_t)(RING_OFF + stage * STAGE_BYTES);
-#pragma unroll
-            for (int s = 0; s < NT; s++) fb[s] = read_frag(st + rd_b + s * 32 * BKB, ks);
-#pragma unroll
-            for (int s = 0; s < MT; s++) fa[s] = read_frag(st + rd_a + s * 32 * BKB, ks);
-        };
-        auto read_scales = [&](int stage) {
+        auto frag_a = [&](int stage, int ks, int i) { return read_frag((uint32_t)(RING_OFF + stage * STAGE_BYTES) + rd_a + i * 32 * BKB, ks); };
+        auto frag_b = [&](int stage, int ks, int j) { return read_frag((uint32_t)(RING_OFF + stage * STAGE_BYTES) + rd_b + j * 32 * BKB, ks); };
+        // Scale dwords of K-step kt of the current tile
+        auto read_scales = [&](int kt, uint32_t (&dst)[NSC][MT + NT]) {
             if (!MX) return;
+            const uint32_t ss = (uint32_t)(SCALE_OFF + ((gbase + kt / SPG) & 1) * SCALE_BUF) + (uint32_t)(kt % SPG) * (SCALE_DW * 4u);
 #pragma unroll
             for (int d = 0; d < SCALE_DW; d++) {
-                const uint32_t ss = (uint32_t)(SCALE_OFF + stage * SCALE_STAGE + d * 2048);
 #pragma unroll
-                for (int s = 0; s < MT; s++) sc[d][s] = lds_read4(ss + rd_sa + s * 128);
+                for (int s = 0; s < MT; s++) dst[d][s] = lds_read4(ss + rd_sa + s * 512 + d * 4);
 #pragma unroll
-                for (int s = 0; s < NT; s++) sc[d][MT + s] = lds_read4(ss + rd_sb + s * 128);
+                for (int s = 0; s < NT; s++) dst[d][MT + s] = lds_read4(ss + rd_sb + s * 512 + d * 4);
             }
         };
-        // The MFMAs of one 64-byte substep.  DMA: between them, issue the requests of the next
-        // step (pieces PIECE0 .. PIECE0 + count - 1 of tile cur, step kt_next).
-        auto mfma_substep = [&](auto ks_c, auto dma_c, int kt_next, int stage_next) {
-            constexpr int ks = decltype(ks_c)::value;
-            constexpr bool DMA = decltype(dma_c)::value;
-            constexpr int PER = (NV + 1) / 2;            // pieces issued during one substep
-            constexpr int PIECE0 = ks * PER;
-            static_for<MT * NT>([&](auto idx_c) {
-                constexpr int idx = decltype(idx_c)::value;
-                constexpr int i = idx / NT, j = idx % NT;
-#ifndef DBG_NO_MFMA
-                if constexpr (KIND == KIND_F8) {
-                    // scale operands: lane group g presents byte 2*ks + g of the row's dword
-                    const int sh = 8 * (2 * ks) + 8 * g;
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], CBSZ, CBSZ, 0, (int)(sc[0][i] >> sh), 0,
-                                                                                (int)(sc[0][MT + j] >> sh));
-                } else if constexpr (KIND == KIND_F4) {
-                    // substep = 128 elements = scale dword ks; MFMA lo uses byte g, MFMA hi byte 2+g
-                    const int sA = (int)(sc[ks][i] >> (8 * g)), sB = (int)(sc[ks][MT + j] >> (8 * g));
-                    const v8i alo = (v8i){fa[i][0], fa[i][1], fa[i][2], fa[i][3], 0, 0, 0, 0};
-                    const v8i blo = (v8i){fb[j][0], fb[j][1], fb[j][2], fb[j][3], 0, 0, 0, 0};
-                    const v8i ahi = (v8i){fa[i][4], fa[i][5], fa[i][6], fa[i][7], 0, 0, 0, 0};
-                    const v8i bhi = (v8i){fb[j][4], fb[j][5], fb[j][6], fb[j][7], 0, 0, 0, 0};
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(alo, blo, acc[i][j], 4, 4, 0, sA, 0, sB);
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ahi, bhi, acc[i][j], 4, 4, 2, sA, 2, sB);
-                } else {
-                    const v4i alo = (v4i){fa[i][0], fa[i][1], fa[i][2], fa[i][3]}, ahi = (v4i){fa[i][4], fa[i][5], fa[i][6], fa[i][7]};
-                    const v4i blo = (v4i){fb[j][0], fb[j][1], fb[j][2], fb[j][3]}, bhi = (v4i){fb[j][4], fb[j][5], fb[j][6], fb[j][7]};
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo, blo, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi, bhi, acc[i][j], 0, 0, 0);
-                }
-#endif
-                if constexpr (DMA && idx < PER && PIECE0 + idx < NV) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    issue_piece(cur, kt_next, stage_next, IC<PIECE0 + idx>{});
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-#ifdef DBG_TIMING
-                if constexpr (ks == 0 && idx == 3) { const int kt = kt_next - 1; TSTAMP(2); }
-#endif
-            });
+        // One MFMA of row block i of a 64-byte substep; m = 0 .. MPR-1 walks the row: all
+        // column blocks on the low 32 bytes, then (int8 and FP4, which take two MFMAs per
+        // 64 bytes) all on the high 32 bytes, so that consecutive MFMAs never share an accumulator.
+        constexpr int MPR = KIND == KIND_F8 ? NT : 2 * NT;  // MFMAs per row block
+        auto mfma_one = [&](auto ks_c, auto i_c, auto m_c, const v8i &a, const v8i (&b)[NT]) {
+            constexpr int ks = decltype(ks_c)::value, i = decltype(i_c)::value, m = decltype(m_c)::value;
+            constexpr int j = m % NT, half = m / NT;
+            if constexpr (KIND == KIND_F8) {
+                // scale operands: lane group g presents byte 2*ks + g of the row's dword
+                const int sh = 8 * (2 * ks) + 8 * g;
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b[j], acc[i][j], CBSZ, CBSZ, 0, (int)(sc[0][i] >> sh), 0,
+                                                                            (int)(sc[0][MT + j] >> sh));
+            } else if constexpr (KIND == KIND_F4) {
+                // substep = 128 elements = scale dword ks; the low MFMA uses byte g, the high one byte 2+g
+                const int sA = (int)(sc[ks][i] >> (8 * g)), sB = (int)(sc[ks][MT + j] >> (8 * g));
+                const v8i ah = (v8i){a[4 * half], a[4 * half + 1], a[4 * half + 2], a[4 * half + 3], 0, 0, 0, 0};
+                const v8i bh = (v8i){b[j][4 * half], b[j][4 * half + 1], b[j][4 * half + 2], b[j][4 * half + 3], 0, 0, 0, 0};
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ah, bh, acc[i][j], 4, 4, 2 * half, sA, 2 * half, sB);
+            } else {
+                const v4i ah = (v4i){a[4 * half], a[4 * half + 1], a[4 * half + 2], a[4 * half + 3]};
+                const v4i bh = (v4i){b[j][4 * half], b[j][4 * half + 1], b[j][4 * half + 2], b[j][4 * half + 3]};
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah, bh, acc[i][j], 0, 0, 0);
+            }
+        };
+        auto mfma_row = [&](auto ks_c, auto i_c, const v8i &a, const v8i (&b)[NT]) {
+            static_for<MPR>([&](auto m_c) { mfma_one(ks_c, i_c, m_c, a, b); });
         };
 
-        // The requests of step 0 were the last direct-to-LDS loads this wave issued; only the
-        // previous tile's epilogue stores may have been issued after them.
-        if (first) CCH_WAIT_VM_LGKM0(0);
-        else CCH_WAIT_VM_LGKM0(NSTORES);
+        // One K-step.  On entry fa / fb0 / sc hold the step's first substep.  MODE 0: steady
+        // state, requests step kt+2 of this tile; 1: second to last step, requests the next
+        // tile's set-up and first step; 2: last step, requests the next tile's second step and
+        // prefetches no fragments.  The ring stage a step occupies is read for the last time
+        // just before the step's barrier, and the requests issued after that barrier refill
+        // it, two steps ahead of its use.  Everything that follows the barrier is threaded
+        // between the step's remaining MFMAs, one or two instructions at a time, so that the
+        // matrix pipe keeps running while the wave issues them.
+        auto step = [&](auto mode_c, int kt) {
+            constexpr int MODE = decltype(mode_c)::value;
+            const int stage = gstep & 1, nstage = stage ^ 1;
+            static_for<MT>([&](auto i_c) {
+                constexpr int i = decltype(i_c)::value;
+                mfma_row(IC<0>{}, i_c, fa[i], fb0);
+                __builtin_amdgcn_sched_barrier(0);
+                fa[i] = frag_a(stage, 1, i);
+                if constexpr (i < NT) fb1[i] = frag_b(stage, 1, i);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            mfma_row(IC<1>{}, IC<0>{}, fa[0], fb1);
+            __builtin_amdgcn_sched_barrier(0);
+            // Every LDS read of this step has been issued; once they have returned and the
+            // requests of step kt+1 have landed, for all waves, the stage can be refilled.
+            CCH_WAIT_VM_LGKM0(0);
+            __syncthreads();
+            constexpr int SLOTS = (MT - 1) * MPR;           // MFMAs left in this step
+            constexpr int NREQ = NV + (MX ? 1 : 0);         // requests of a steady step
+            constexpr int PER_SLOT = (NREQ + SLOTS - 2) / (SLOTS - 1);
+            const int newgrp = ((kt + 2) & (SPG - 1)) == 0;
+            static_for<SLOTS>([&](auto slot_c) {
+                constexpr int slot = decltype(slot_c)::value;
+                constexpr int i = 1 + slot / MPR, m = slot % MPR;
+                mfma_one(IC<1>{}, IC<i>{}, IC<m>{}, fa[i], fb1);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (slot == 0) {
+                    if constexpr (MODE != 2) {
+#pragma unroll
+                        for (int j = 0; j < NT; j++) fb0[j] = frag_b(nstage, 0, j);
+                        fa[0] = frag_a(nstage, 0, 0);
+                    }
+                    if constexpr (MODE == 1) {
+                        nbase = gi;
+                        setup(nxt, parity ^ 1, stage);
+                    } else if constexpr (MODE == 2) {
+                        issue_step(nxt, 1, stage);
+                    }
+                } else if constexpr (MODE == 0) {
+                    static_for<PER_SLOT>([&](auto q_c) {
+                        constexpr int piece = (slot - 1) * PER_SLOT + decltype(q_c)::value;
+                        if constexpr (piece < NV) issue_piece(cur, kt + 2, stage, IC<piece>{});
+                        else if constexpr (piece == NV && MX) issue_scales(newgrp, cur, (kt + 2) / SPG, gi & 1);
+                    });
+                }
+                if constexpr (MODE != 2 && m == MPR - 1) fa[i] = frag_a(nstage, 0, i);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            if constexpr (MODE == 0) gi += MX ? newgrp : 0;
+            if constexpr (MODE != 2) read_scales(kt + 1, sc);
+            if constexpr (MODE != 0) {
+                // Pin the accumulators here: otherwise the compiler sinks the MFMAs of the
+                // peeled steps into the epilogue and spills their fragments to get them there.
+#pragma unroll
+                for (int i = 0; i < MT; i++)
+#pragma unroll
+                    for (int j = 0; j < NT; j++) asm volatile("" : "+v"(acc[i][j]));
+            }
+            gstep++;
+        };
+        // Tile prologue.  In flight, oldest first: this tile's set-up and first step, its
+        // second step (NV requests), then the previous tile's epilogue stores.
+        constexpr int NSTORES = MT * NPASS;
+        if (first) CCH_WAIT_VM_LGKM0(NV);
+        else CCH_WAIT_VM_LGKM0(NV + NSTORES);
         __syncthreads();
-        // Steady state: right after the barrier that retires step kt-1, request step kt+1 into
-        // the stage it vacated, then compute step kt.  No branches.
-        for (int kt = 0; kt + 1 < ksteps; kt++, gstep++) {
-            const int stage = gstep & 1;
-            TSTAMP(0);
-#ifndef DBG_NO_LOADS
-            issue_step(cur, kt + 1, stage ^ 1);
-#endif
-            read_scales(stage);
-            read_substep(stage, 0);
-            TSTAMP(1);
-            mfma_substep(IC<0>{}, std::false_type{}, 0, 0);
-            TSTAMP(3);
-            read_substep(stage, 1);
-            mfma_substep(IC<1>{}, std::false_type{}, 0, 0);
-            CCH_WAIT_VM_LGKM0(0);  // this wave's requests for step kt+1 have landed
-#ifndef DBG_NO_BARRIER
-            __syncthreads();        // ... everybody's have, and everybody is done reading step kt
-#endif
-        }
-        // Last step: the other stage is free for the next tile's first step.
         {
             const int stage = gstep & 1;
-            decode(t + gridDim.x, nxt);
-#ifndef DBG_NO_LOADS
-            if (nxt.valid) setup(nxt, parity ^ 1, stage ^ 1);
-#endif
-            read_scales(stage);
-            read_substep(stage, 0);
-            mfma_substep(IC<0>{}, std::false_type{}, 0, 0);
-            read_substep(stage, 1);
-            mfma_substep(IC<1>{}, std::false_type{}, 0, 0);
-            gstep++;
+            read_scales(0, sc);
+#pragma unroll
+            for (int j = 0; j < NT; j++) fb0[j] = frag_b(stage, 0, j);
+#pragma unroll
+            for (int i = 0; i < MT; i++) fa[i] = frag_a(stage, 0, i);
         }
-#ifdef DBG_TIMING
-        if (t == 2 * (int)gridDim.x && blockIdx.x == 0) {
-            __syncthreads();
-            for (int i = threadIdx.x; i < 8 * 16 * 4; i += TILE_THREADS)
-                reinterpret_cast<unsigned long long *>(const_cast<uint8_t *>(p.sa))[i] =
-                    *reinterpret_cast<unsigned long long *>(smem + EPI_OFF + i * 8);
-            __syncthreads();
-        }
-#endif
+        for (int kt = 0; kt + 2 < ksteps; kt++) step(IC<0>{}, kt);
+        decode(t + gridDim.x, nxt);
+        step(IC<1>{}, ksteps - 2);
+        step(IC<2>{}, ksteps - 1);
         first = false;
 
-#ifdef DBG_NO_EPI
-        if (acc[0][0][0] != 12345) { cur = nxt; t += gridDim.x; parity ^= 1; continue; }
-#endif
         // Epilogue.  Lane (r, g) holds, for sub-tile (i, j), column r and rows
-        // (x/4)*8 + g*4 + x%4, x = 0..15.  Sixteen rows at a time go through the wave's private
-        // LDS buffer: neighbouring lanes exchange one value so that each writes two adjacent
-        // bf16, then every lane reads back 16 contiguous bytes and stores them.  Stores are raw
-        // buffer stores whose out-of-range lanes are dropped by the bounds check, so that every
-        // lane issues exactly NSTORES of them.
+        // q*8 + g*4 + xr at accumulator index 4q + xr.  PASS_ROWS rows at a time go through the
+        // wave's private 1 KiB LDS buffer: neighbouring lanes exchange one value so that each
+        // writes two adjacent bf16, then every lane reads back 16 contiguous bytes and stores
+        // them.  Stores are raw buffer stores whose out-of-range lanes are dropped by the
+        // bounds check.
         {
             const uint32_t epi = (uint32_t)(EPI_OFF + wave * EPI_WAVE);
             const uint32_t prm = (uint32_t)(PARAM_OFF + parity * PARAM_SET);
@@ -433,32 +486,30 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 #pragma unroll
             for (int i = 0; i < MT; i++) {
 #pragma unroll
-                for (int hh = 0; hh < 2; hh++) {
-                    float tok[2][4];
-                    if (EPI != EPI_PLAIN) {
+                for (int ps = 0; ps < NPASS; ps++) {
 #pragma unroll
-                        for (int xq = 0; xq < 2; xq++) {
-                            const v4i tv = lds_read16(prm + (uint32_t)(wm * WM + i * 32 + hh * 16 + xq * 8 + g * 4) * 4u);
+                    for (int qq = 0; qq < PASS_ROWS / 8; qq++) {
+                        const int q = ps * (PASS_ROWS / 8) + qq;
+                        float tok[4];
+                        if (EPI != EPI_PLAIN) {
+                            const v4i tv = lds_read16(prm + (uint32_t)(wm * WM + i * 32 + q * 8 + g * 4) * 4u);
 #pragma unroll
-                            for (int xr = 0; xr < 4; xr++) tok[xq][xr] = __int_as_float(tv[xr]);
+                            for (int xr = 0; xr < 4; xr++) tok[xr] = __int_as_float(tv[xr]);
                         }
-                    }
-#pragma unroll
-                    for (int xq = 0; xq < 2; xq++)
 #pragma unroll
                         for (int xr = 0; xr < 4; xr += 2)
 #pragma unroll
                             for (int j = 0; j < (SWIGLU ? 1 : NT); j++) {
-                                const int x = (2 * hh + xq) * 4 + xr;
+                                const int x = q * 4 + xr;
                                 float v[2];
 #pragma unroll
                                 for (int d = 0; d < 2; d++) {
                                     if (SWIGLU) {
-                                        const float gate = (float)acc[i][0][x + d] * chs[0] * tok[xq][xr + d];
-                                        const float up = (float)acc[i][1][x + d] * chs[1] * tok[xq][xr + d];
+                                        const float gate = (float)acc[i][0][x + d] * chs[0] * tok[xr + d];
+                                        const float up = (float)acc[i][1][x + d] * chs[1] * tok[xr + d];
                                         v[d] = gate * (1.0f / (1.0f + expf(-gate))) * up;
                                     } else if (EPI == EPI_DEQUANT) {
-                                        v[d] = (float)acc[i][j][x + d] * tok[xq][xr + d] * chs[j];
+                                        v[d] = (float)acc[i][j][x + d] * tok[xr + d] * chs[j];
                                     } else {
                                         v[d] = (float)acc[i][j][x + d];
                                     }
@@ -467,26 +518,24 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                                 const uint32_t send = f32_to_bf16_bits(odd ? v[0] : v[1]);
                                 const uint32_t recv = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, 0xB1, 0xF, 0xF, true);
                                 const uint32_t packed = odd ? (recv | (keep << 16)) : (keep | (recv << 16));
-                                const int lrow = xq * 8 + g * 4 + xr + (odd ? 1 : 0);
+                                const int lrow = qq * 8 + g * 4 + xr + (odd ? 1 : 0);
                                 const int lcol = j * 32 + (r & ~1);
                                 *reinterpret_cast<uint32_t *>(smem + epi + (uint32_t)(lrow * ROWB + lcol * 2)) = packed;
                             }
-                    const int row0 = wm * WM + i * 32 + hh * 16;  // relative to m0
-                    const int col0 = cur.j0 + wn * WN_OUT;
-#pragma unroll
-                    for (int q = 0; q < 16 / RPI; q++) {
-                        const int lrow = q * RPI + lane / CPR, chunk = lane % CPR;
-                        const v4i val = lds_read16(epi + (uint32_t)(lrow * ROWB + chunk * 16));
-                        const int row = row0 + lrow, col = col0 + chunk * 8;
-                        const bool ok = (cur.m0 + row < cur.m_end) && (col + 8 <= p.n_out);
-                        const uint32_t off = ok ? ((uint32_t)row * (uint32_t)p.n_out + (uint32_t)col) * 2u : 0xFFFFFFF0u;
-                        __builtin_amdgcn_raw_buffer_store_b128((v4u){(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]},
-                                                               rs_out, (int)off, 0, 0);
                     }
+                    const int lrow = lane / CPR, chunk = lane % CPR;
+                    const v4i val = lds_read16(epi + (uint32_t)(lrow * ROWB + chunk * 16));
+                    const int row = wm * WM + i * 32 + ps * PASS_ROWS + lrow;  // relative to m0
+                    const int col = cur.j0 + wn * WN_OUT + chunk * 8;
+                    const bool ok = (cur.m0 + row < cur.m_end) && (col + 8 <= p.n_out);
+                    const uint32_t off = ok ? ((uint32_t)row * (uint32_t)p.n_out + (uint32_t)col) * 2u : 0xFFFFFFF0u;
+                    __builtin_amdgcn_raw_buffer_store_b128((v4u){(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]},
+                                                           rs_out, (int)off, 0, 0);
                 }
             }
         }
         cur = nxt;
+        gbase = nbase;
         t += gridDim.x;
         parity ^= 1;
     }
@@ -532,7 +581,7 @@ bool gemm_tile_supports(const GemmProblem &p, int kind)
     const int epb = kind == KIND_F4 ? 2 : 1;
     if (!p.trans_b) return false;
     // whole 128-byte K-steps; output rows must take 16-byte stores
-    if (p.K <= 0 || p.K % (BKB * epb) != 0) return false;
+    if (p.K < 2 * BKB * epb || p.K % (BKB * epb) != 0) return false;
     if (p.n_out % 8 != 0 || !aligned(p.out, 16)) return false;
     if ((int64_t)BM * p.n_out * 2 >= ((int64_t)1 << 31)) return false;
     if (p.num_groups > MAX_GROUPS) return false;
