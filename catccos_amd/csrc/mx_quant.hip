@@ -15,10 +15,22 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int QUANT_THREADS = 256;
-constexpr int QUANT_UNROLL = 4;  // wave-steps (64 lanes x 8 elements) per wave
+#ifndef QUANT_UNROLL_V
+#define QUANT_UNROLL_V 2
+#endif
+#ifndef QUANT_BPC_V
+#define QUANT_BPC_V 8
+#endif
+constexpr int QUANT_UNROLL = QUANT_UNROLL_V;          // wave-steps (64 lanes x 8 elements) per batch
+constexpr int QUANT_BLOCKS_PER_CU = QUANT_BPC_V;      // resident workgroups per CU the grid is sized for
 
-template <int FMT, int RND, bool HWCVT>
-__device__ __forceinline__ void quant8(const uint32_t (&w)[4], int e, bool is_nan, uint32_t (&out)[2])
+typedef short s16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// Software path: scale in fp32, round with the integer encoder (any rounding rule).
+template <int FMT, int RND>
+__device__ __forceinline__ void quant8_soft(const uint32_t (&w)[4], int e, bool is_nan, uint32_t (&out)[2])
 {
     using T = FmtTraits<FMT>;
     const float inv = pow2i(-e);
@@ -34,17 +46,6 @@ __device__ __forceinline__ void quant8(const uint32_t (&w)[4], int e, bool is_na
         for (int i = 0; i < 8; i++) r |= (is_nan ? T::NANCODE : encode_small<FMT, RND>(y[i])) << (4 * i);
         out[0] = r;
         out[1] = 0;
-    } else if constexpr (HWCVT) {
-        // Hardware cast: round to nearest even; the clamp keeps it away from its overflow rule.
-        int r0 = 0, r1 = 0;
-#pragma unroll
-        for (int i = 0; i < 8; i++) y[i] = __builtin_amdgcn_fmed3f(y[i], -T::MAXV, T::MAXV);
-        r0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], r0, false);
-        r0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], r0, true);
-        r1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], r1, false);
-        r1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], r1, true);
-        out[0] = is_nan ? 0x7F7F7F7Fu : (uint32_t)r0;
-        out[1] = is_nan ? 0x7F7F7F7Fu : (uint32_t)r1;
     } else {
         uint32_t r0 = 0, r1 = 0;
 #pragma unroll
@@ -57,23 +58,81 @@ __device__ __forceinline__ void quant8(const uint32_t (&w)[4], int e, bool is_na
     }
 }
 
+// Hardware path (round to nearest even, sign kept on zero): the packed bf16 -> FP8 / FP4
+// conversions of gfx950 divide by a power-of-two scale and round in one instruction, two values
+// at a time, straight from the packed bf16 input.  The FP4 form saturates; the FP8 forms return
+// NaN above the format maximum, so magnitudes are first clamped, as 16-bit integers, to the bf16
+// pattern of MAXV * 2^e.  Checked against the software path for every finite bf16 input and
+// every applied exponent from -127 to 119.
+template <int FMT>
+__device__ __forceinline__ void quant8_hw(const uint32_t (&w)[4], int e, bool is_nan, uint32_t (&out)[2])
+{
+    using T = FmtTraits<FMT>;
+    const float scale = __uint_as_float((uint32_t)(e + 127) << 23);  // exponent field 0 stands for 2^-127
+    if constexpr (FMT == CCH_FMT_E2M1) {
+        uint32_t r = 0;
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(bf16x2, w[0]), scale, 0);
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(bf16x2, w[1]), scale, 1);
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(bf16x2, w[2]), scale, 2);
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(bf16x2, w[3]), scale, 3);
+        out[0] = is_nan ? 0x77777777u : r;
+        out[1] = 0;
+    } else {
+        // MAXV = 1.75 * 2^EMAX in both FP8 formats: mantissa bits 1100000 under exponent e + EMAX
+        const int te = e + T::EMAX + 127;
+        const uint32_t t16 = te > 254 ? 0x7F7Fu : (((uint32_t)te << 7) | 0x60u);
+        const u16x2 lim = {(unsigned short)t16, (unsigned short)t16};
+        bf16x2 c[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const u16x2 mag = __builtin_elementwise_min(__builtin_bit_cast(u16x2, w[i] & 0x7FFF7FFFu), lim);
+            c[i] = __builtin_bit_cast(bf16x2, __builtin_bit_cast(uint32_t, mag) | (w[i] & 0x80008000u));
+        }
+        s16x2 r0 = {0, 0}, r1 = {0, 0};
+        if constexpr (FMT == CCH_FMT_E4M3) {
+            r0 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(r0, c[0], scale, false);
+            r0 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(r0, c[1], scale, true);
+            r1 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(r1, c[2], scale, false);
+            r1 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(r1, c[3], scale, true);
+        } else {
+            r0 = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(r0, c[0], scale, false);
+            r0 = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(r0, c[1], scale, true);
+            r1 = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(r1, c[2], scale, false);
+            r1 = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(r1, c[3], scale, true);
+        }
+        out[0] = is_nan ? 0x7F7F7F7Fu : __builtin_bit_cast(uint32_t, r0);
+        out[1] = is_nan ? 0x7F7F7F7Fu : __builtin_bit_cast(uint32_t, r1);
+    }
+}
+
+template <int FMT, int RND, bool HWCVT>
+__device__ __forceinline__ void quant8(const uint32_t (&w)[4], int e, bool is_nan, uint32_t (&out)[2])
+{
+    if constexpr (HWCVT) quant8_hw<FMT>(w, e, is_nan, out);
+    else quant8_soft<FMT, RND>(w, e, is_nan, out);
+}
+
 // Largest |bf16| bit pattern among the 8 values packed in w, then across the 4 lanes of the quad.
 __device__ __forceinline__ uint32_t block_amax_bits(const uint32_t (&w)[4])
 {
-    uint32_t m = 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t a = w[i] & 0x7FFF7FFFu;
-        m = max(m, max(a & 0xFFFFu, a >> 16));
-    }
+    const u16x2 a0 = __builtin_bit_cast(u16x2, w[0] & 0x7FFF7FFFu), a1 = __builtin_bit_cast(u16x2, w[1] & 0x7FFF7FFFu);
+    const u16x2 a2 = __builtin_bit_cast(u16x2, w[2] & 0x7FFF7FFFu), a3 = __builtin_bit_cast(u16x2, w[3] & 0x7FFF7FFFu);
+    const u16x2 mm = __builtin_elementwise_max(__builtin_elementwise_max(a0, a1), __builtin_elementwise_max(a2, a3));
+    uint32_t m = max((uint32_t)mm[0], (uint32_t)mm[1]);
     m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
     m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
     return m;
 }
 
 // x [rows,K] bf16.  One wave-step = 64 lanes x 8 elements of one row; a row has `wpr` wave-steps.
+// The grid is sized to the machine, not to the problem: every wave walks the list of wave-steps
+// with a grid stride, QUANT_UNROLL at a time, and requests the next batch before it converts the
+// current one, so that each wave always has loads in flight.
 // VEC: K % 8 == 0 and all pointers suitably aligned, so whole-vector accesses are legal.
-template <int FMT, int RND, bool HWCVT, bool VEC>
+// PAIR (needs VEC, K % 16 == 0 and 16-byte aligned payload rows): neighbouring lanes swap halves
+// of two wave-steps so that each lane stores one 16-byte (FP8) or 8-byte (FP4) piece instead of
+// two of half that size; the store path's cost is per instruction, not per byte.
+template <int FMT, int RND, bool HWCVT, bool VEC, bool PAIR>
 __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
     const uint16_t *__restrict__ x, uint8_t *__restrict__ payload, uint8_t *__restrict__ scales, int rows, int K,
     int nblk, int sld, int pld, int wpr, int total_ws)
@@ -81,61 +140,196 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
     constexpr bool FP4 = FMT == CCH_FMT_E2M1;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (QUANT_THREADS / 64) + (threadIdx.x >> 6)));
-    uint32_t w[QUANT_UNROLL][4];
-    int row[QUANT_UNROLL], k0[QUANT_UNROLL];
+    const int stride = (int)gridDim.x * (QUANT_THREADS / 64) * QUANT_UNROLL;
 
+    struct Batch {
+        uint32_t w[QUANT_UNROLL][4];
+        int row[QUANT_UNROLL], k0[QUANT_UNROLL];
+    };
+    auto fetch = [&](int ws0, Batch &bt) {
 #pragma unroll
-    for (int u = 0; u < QUANT_UNROLL; u++) {
-        const int ws = wave * QUANT_UNROLL + u;
-        const int r = ws / wpr;
-        row[u] = ws < total_ws ? r : -1;
-        k0[u] = ((ws - r * wpr) * 64 + lane) * 8;
-        w[u][0] = w[u][1] = w[u][2] = w[u][3] = 0;
-        if (row[u] >= 0 && k0[u] < K) {
-            const uint16_t *src = x + (size_t)row[u] * K + k0[u];
-            if (VEC) {
-                const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src));
-                w[u][0] = v[0]; w[u][1] = v[1]; w[u][2] = v[2]; w[u][3] = v[3];
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; i++)
-                    if (k0[u] + i < K) w[u][i >> 1] |= (uint32_t)src[i] << ((i & 1) * 16);
-            }
-        }
-    }
-
-#pragma unroll
-    for (int u = 0; u < QUANT_UNROLL; u++) {
-        if (row[u] < 0) continue;  // wave-uniform
-        const uint32_t amax_bits = block_amax_bits(w[u]);
-        int e;
-        bool is_nan;
-        const uint32_t sbyte = shared_exp_byte<FMT>(amax_bits, e, is_nan);
-        uint32_t q[2];
-        quant8<FMT, RND, HWCVT>(w[u], e, is_nan, q);
-        const int blk = k0[u] >> 5;
-        if (k0[u] < K) {
-            uint8_t *dst = payload + (size_t)row[u] * pld + (FP4 ? (k0[u] >> 1) : k0[u]);
-            if (VEC) {
-                if (FP4) {
-                    __builtin_nontemporal_store(q[0], reinterpret_cast<uint32_t *>(dst));
+        for (int u = 0; u < QUANT_UNROLL; u++) {
+            const int ws = ws0 + u;
+            const int r = ws / wpr;
+            bt.row[u] = ws < total_ws ? r : -1;
+            bt.k0[u] = ((ws - r * wpr) * 64 + lane) * 8;
+            bt.w[u][0] = bt.w[u][1] = bt.w[u][2] = bt.w[u][3] = 0;
+            if (bt.row[u] >= 0 && bt.k0[u] < K) {
+                const uint16_t *src = x + (size_t)bt.row[u] * K + bt.k0[u];
+                if (VEC) {
+                    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src));
+                    bt.w[u][0] = v[0]; bt.w[u][1] = v[1]; bt.w[u][2] = v[2]; bt.w[u][3] = v[3];
                 } else {
-                    u32x2 o = {q[0], q[1]};
-                    __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(dst));
+#pragma unroll
+                    for (int i = 0; i < 8; i++)
+                        if (bt.k0[u] + i < K) bt.w[u][i >> 1] |= (uint32_t)src[i] << ((i & 1) * 16);
                 }
-            } else if (FP4) {
-                for (int i = 0; i < 4; i++)
-                    if (k0[u] + 2 * i < K) dst[i] = (uint8_t)(q[0] >> (8 * i)) & (k0[u] + 2 * i + 1 < K ? 0xFF : 0x0F);
-            } else {
-                for (int i = 0; i < 8; i++)
-                    if (k0[u] + i < K) dst[i] = (uint8_t)(q[i >> 2] >> (8 * (i & 3)));
             }
         }
-        if (blk < nblk) {
-            uint8_t *srow = scales + (size_t)row[u] * sld;
-            if ((lane & 3) == 0) srow[blk] = (uint8_t)sbyte;
-            if ((lane & 3) == 1 && blk == nblk - 1 && sld != nblk) srow[nblk] = 127;  // even padding, 1.0
+    };
+    auto convert = [&](const Batch &bt) {
+        uint32_t held[2] = {0, 0};  // PAIR: payload of the even wave-step, waiting for its partner
+#pragma unroll
+        for (int u = 0; u < QUANT_UNROLL; u++) {
+            if (bt.row[u] < 0) continue;  // wave-uniform
+            const uint32_t amax_bits = block_amax_bits(bt.w[u]);
+            int e;
+            bool is_nan;
+            const uint32_t sbyte = shared_exp_byte<FMT>(amax_bits, e, is_nan);
+            uint32_t q[2];
+            quant8<FMT, RND, HWCVT>(bt.w[u], e, is_nan, q);
+            const int k0 = bt.k0[u], blk = k0 >> 5;
+            if (PAIR) {
+                // Wave-steps come in pairs (u even, u odd); a pair is complete unless the list
+                // ends on the even one.  Even lanes end up with the even step's 16 (8) bytes of
+                // lanes l and l+1, odd lanes with the odd step's bytes of lanes l-1 and l.
+                const bool odd_lane = lane & 1;
+                const bool partner = (u & 1) || (u + 1 < QUANT_UNROLL && bt.row[u + 1] >= 0);  // wave-uniform
+                if (!(u & 1) && partner) {
+                    held[0] = q[0];
+                    held[1] = q[1];
+                } else if (u & 1) {
+                    const int ke = bt.k0[u - 1], ko = k0;  // same lane offset in both steps unless the row changed
+                    uint32_t send0 = odd_lane ? held[0] : q[0], send1 = odd_lane ? held[1] : q[1];
+                    const uint32_t recv0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send0, 0xB1, 0xF, 0xF, true);
+                    const uint32_t recv1 = FP4 ? 0u : (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send1, 0xB1, 0xF, 0xF, true);
+                    const int rw = odd_lane ? bt.row[u] : bt.row[u - 1];
+                    const int kk = odd_lane ? ko - 8 : ke;
+                    if (kk < K) {
+                        uint8_t *dst = payload + (size_t)rw * pld + (FP4 ? (kk >> 1) : kk);
+                        if (FP4) {
+                            u32x2 o = odd_lane ? (u32x2){recv0, q[0]} : (u32x2){held[0], recv0};
+                            __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(dst));
+                        } else {
+                            u32x4 o = odd_lane ? (u32x4){recv0, recv1, q[0], q[1]} : (u32x4){held[0], held[1], recv0, recv1};
+                            __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(dst));
+                        }
+                    }
+                } else if (k0 < K) {  // unpaired last step
+                    uint8_t *dst = payload + (size_t)bt.row[u] * pld + (FP4 ? (k0 >> 1) : k0);
+                    if (FP4) {
+                        __builtin_nontemporal_store(q[0], reinterpret_cast<uint32_t *>(dst));
+                    } else {
+                        u32x2 o = {q[0], q[1]};
+                        __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(dst));
+                    }
+                }
+            } else if (k0 < K) {
+                uint8_t *dst = payload + (size_t)bt.row[u] * pld + (FP4 ? (k0 >> 1) : k0);
+                if (VEC) {
+                    if (FP4) {
+                        __builtin_nontemporal_store(q[0], reinterpret_cast<uint32_t *>(dst));
+                    } else {
+                        u32x2 o = {q[0], q[1]};
+                        __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(dst));
+                    }
+                } else if (FP4) {
+                    for (int i = 0; i < 4; i++)
+                        if (k0 + 2 * i < K) dst[i] = (uint8_t)(q[0] >> (8 * i)) & (k0 + 2 * i + 1 < K ? 0xFF : 0x0F);
+                } else {
+                    for (int i = 0; i < 8; i++)
+                        if (k0 + i < K) dst[i] = (uint8_t)(q[i >> 2] >> (8 * (i & 3)));
+                }
+            }
+            if (blk < nblk) {
+                uint8_t *srow = scales + (size_t)bt.row[u] * sld;
+                if ((lane & 3) == 0) srow[blk] = (uint8_t)sbyte;
+                if ((lane & 3) == 1 && blk == nblk - 1 && sld != nblk) srow[nblk] = 127;  // even padding, 1.0
+            }
         }
+    };
+
+    // Two batches in ping-pong: while one is converted and stored, the other's loads are in flight.
+    Batch b0, b1;
+    int ws0 = wave * QUANT_UNROLL;
+    if (ws0 >= total_ws) return;
+    fetch(ws0, b0);
+    for (;;) {
+        const int ws1 = ws0 + stride, ws2 = ws1 + stride;  // all wave-uniform
+        if (ws1 < total_ws) fetch(ws1, b1);
+        convert(b0);
+        if (ws1 >= total_ws) break;
+        if (ws2 < total_ws) fetch(ws2, b0);
+        convert(b1);
+        if (ws2 >= total_ws) break;
+        ws0 = ws2;
+    }
+}
+
+// Fast path of the row quantiser: round to nearest even with the hardware conversions, K a
+// multiple of 1024 (so that wave-steps pair up inside a row and none is partial) and 16-byte
+// aligned buffers.  No per-lane bounds checks; a wave owns pairs of adjacent wave-steps
+// (1024 elements of one row), keeps the next pair's loads in flight while it converts the
+// current one, stores 16 (FP8) or 8 (FP4) payload bytes per lane and writes the 32 scale bytes
+// of the pair as dwords gathered with row shifts.
+template <int FMT>
+__global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_fast_kernel(
+    const uint16_t *__restrict__ x, uint8_t *__restrict__ payload, uint8_t *__restrict__ scales, int K, int sld, int pld,
+    int ppr, int npairs)
+{
+    constexpr bool FP4 = FMT == CCH_FMT_E2M1;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (QUANT_THREADS / 64) + (threadIdx.x >> 6)));
+    const int stride = (int)gridDim.x * (QUANT_THREADS / 64);
+    const bool odd_lane = lane & 1;
+
+    auto fetch = [&](int p, u32x4 (&v)[2]) {
+        const int r = p / ppr, c = p - r * ppr;  // row, pair within the row (wave-uniform)
+        const uint16_t *src = x + (size_t)r * K + (size_t)c * 1024 + lane * 8;
+        v[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src));
+        v[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 512));
+    };
+    auto convert = [&](int p, const u32x4 (&v)[2]) {
+        const int r = p / ppr, c = p - r * ppr;
+        uint32_t q[2][2], sdw[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t w[4] = {v[h][0], v[h][1], v[h][2], v[h][3]};
+            const uint32_t amax_bits = block_amax_bits(w);
+            int e;
+            bool is_nan;
+            const uint32_t sbyte = shared_exp_byte<FMT>(amax_bits, e, is_nan);
+            quant8_hw<FMT>(w, e, is_nan, q[h]);
+            // lanes 4j hold block j's scale byte: gather 4 of them into lanes 0, 16, 32, 48
+            const uint32_t b1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)sbyte, 0x104, 0xF, 0xF, true);  // row_shl:4
+            const uint32_t b2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)sbyte, 0x108, 0xF, 0xF, true);  // row_shl:8
+            const uint32_t b3 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)sbyte, 0x10C, 0xF, 0xF, true);  // row_shl:12
+            sdw[h] = sbyte | (b1 << 8) | (b2 << 16) | (b3 << 24);
+        }
+        // Neighbouring lanes swap: even lanes take both halves of step 0, odd lanes of step 1.
+        const uint32_t send0 = odd_lane ? q[0][0] : q[1][0], send1 = odd_lane ? q[0][1] : q[1][1];
+        const uint32_t recv0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send0, 0xB1, 0xF, 0xF, true);
+        const uint32_t recv1 = FP4 ? 0u : (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send1, 0xB1, 0xF, 0xF, true);
+        // element offset inside the row of the first value this lane stores
+        const int k = c * 1024 + (odd_lane ? 512 + (lane - 1) * 8 : lane * 8);
+        uint8_t *dst = payload + (size_t)r * pld + (FP4 ? (k >> 1) : k);
+        if (FP4) {
+            const u32x2 o = odd_lane ? (u32x2){recv0, q[1][0]} : (u32x2){q[0][0], recv0};
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(dst));
+        } else {
+            const u32x4 o = odd_lane ? (u32x4){recv0, recv1, q[1][0], q[1][1]} : (u32x4){q[0][0], q[0][1], recv0, recv1};
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(dst));
+        }
+        if ((lane & 15) == 0) {
+            uint32_t *sp = reinterpret_cast<uint32_t *>(scales + (size_t)r * sld + c * 32 + (lane >> 4) * 4);
+            sp[0] = sdw[0];
+            sp[4] = sdw[1];
+        }
+    };
+
+    u32x4 v0[2], v1[2];
+    int p0 = wave;
+    if (p0 >= npairs) return;
+    fetch(p0, v0);
+    for (;;) {
+        const int p1 = p0 + stride, p2 = p1 + stride;  // wave-uniform
+        if (p1 < npairs) fetch(p1, v1);
+        convert(p0, v0);
+        if (p1 >= npairs) break;
+        if (p2 < npairs) fetch(p2, v0);
+        convert(p1, v1);
+        if (p2 >= npairs) break;
+        p0 = p2;
     }
 }
 
@@ -146,20 +340,36 @@ static int launch_rows(const void *x, void *payload, void *scales, int64_t m, in
     const int64_t nblk = (k + 31) / 32, sld = 2 * ((nblk + 1) / 2), pld = fp4 ? (k + 1) / 2 : k;
     const int64_t wpr = (nblk * 4 + 63) / 64;
     const bool vec = (k % 8 == 0) && aligned(x, 16) && aligned(payload, 8);
+    const bool pair = vec && (k % 16 == 0) && aligned(payload, 16) && QUANT_UNROLL % 2 == 0;
+    int dev = 0, cus = 0;
+    CCH_HIP(hipGetDevice(&dev));
+    CCH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int64_t max_blocks = (int64_t)cus * QUANT_BLOCKS_PER_CU;
+    if (HWCVT && k % 1024 == 0 && aligned(x, 16) && aligned(payload, 16) && aligned(scales, 4) && m * (k / 1024) < ((int64_t)1 << 30)) {
+        const int64_t npairs = m * (k / 1024);
+        const unsigned grid = (unsigned)std::min<int64_t>((npairs + QUANT_THREADS / 64 - 1) / (QUANT_THREADS / 64), max_blocks);
+        hipLaunchKernelGGL((mx_quant_rows_fast_kernel<FMT>), dim3(grid), dim3(QUANT_THREADS), 0, stream,
+                           static_cast<const uint16_t *>(x), static_cast<uint8_t *>(payload), static_cast<uint8_t *>(scales),
+                           (int)k, (int)sld, (int)pld, (int)(k / 1024), (int)npairs);
+        return launch_status("mx_quant_rows_fast_kernel");
+    }
     const int64_t rows_per_launch = std::max<int64_t>(1, (int64_t)(1 << 30) / wpr);
     for (int64_t r0 = 0; r0 < m; r0 += rows_per_launch) {
         const int64_t rows = std::min(rows_per_launch, m - r0);
         const int64_t total_ws = rows * wpr;
         const int64_t waves = (total_ws + QUANT_UNROLL - 1) / QUANT_UNROLL;
-        const unsigned grid = (unsigned)((waves + QUANT_THREADS / 64 - 1) / (QUANT_THREADS / 64));
+        const unsigned grid = (unsigned)std::min<int64_t>((waves + QUANT_THREADS / 64 - 1) / (QUANT_THREADS / 64), max_blocks);
         const uint16_t *xs = static_cast<const uint16_t *>(x) + r0 * k;
         uint8_t *ps = static_cast<uint8_t *>(payload) + r0 * pld;
         uint8_t *ss = static_cast<uint8_t *>(scales) + r0 * sld;
-        if (vec)
-            hipLaunchKernelGGL((mx_quant_rows_kernel<FMT, RND, HWCVT, true>), dim3(grid), dim3(QUANT_THREADS), 0, stream,
+        if (vec && pair)
+            hipLaunchKernelGGL((mx_quant_rows_kernel<FMT, RND, HWCVT, true, true>), dim3(grid), dim3(QUANT_THREADS), 0, stream,
+                               xs, ps, ss, (int)rows, (int)k, (int)nblk, (int)sld, (int)pld, (int)wpr, (int)total_ws);
+        else if (vec)
+            hipLaunchKernelGGL((mx_quant_rows_kernel<FMT, RND, HWCVT, true, false>), dim3(grid), dim3(QUANT_THREADS), 0, stream,
                                xs, ps, ss, (int)rows, (int)k, (int)nblk, (int)sld, (int)pld, (int)wpr, (int)total_ws);
         else
-            hipLaunchKernelGGL((mx_quant_rows_kernel<FMT, RND, HWCVT, false>), dim3(grid), dim3(QUANT_THREADS), 0,
+            hipLaunchKernelGGL((mx_quant_rows_kernel<FMT, RND, HWCVT, false, false>), dim3(grid), dim3(QUANT_THREADS), 0,
                                stream, xs, ps, ss, (int)rows, (int)k, (int)nblk, (int)sld, (int)pld, (int)wpr,
                                (int)total_ws);
         int rc = launch_status("mx_quant_rows_kernel");
@@ -260,10 +470,10 @@ extern "C" int cch_mx_quant_rows(const void *x, void *payload, void *scales, int
                        : launch_rows<CCH_FMT_E4M3, CCH_ROUND_RNE, true>(x, payload, scales, m, k, s);
         case CCH_FMT_E5M2:
             return lut ? launch_rows<CCH_FMT_E5M2, CCH_ROUND_LUT, false>(x, payload, scales, m, k, s)
-                       : launch_rows<CCH_FMT_E5M2, CCH_ROUND_RNE, false>(x, payload, scales, m, k, s);
+                       : launch_rows<CCH_FMT_E5M2, CCH_ROUND_RNE, true>(x, payload, scales, m, k, s);
         case CCH_FMT_E2M1:
             return lut ? launch_rows<CCH_FMT_E2M1, CCH_ROUND_LUT, false>(x, payload, scales, m, k, s)
-                       : launch_rows<CCH_FMT_E2M1, CCH_ROUND_RNE, false>(x, payload, scales, m, k, s);
+                       : launch_rows<CCH_FMT_E2M1, CCH_ROUND_RNE, true>(x, payload, scales, m, k, s);
         default:
             return fail(CCH_EINVAL, "cch_mx_quant_rows: unknown format %d", fmt);
     }
