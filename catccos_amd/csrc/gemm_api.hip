@@ -8,14 +8,14 @@
 namespace cch {
 int launch_gemm_naive(const GemmProblem &p, int kind, int epi, hipStream_t stream);
 int launch_gemm_tile(const GemmProblem &p, int kind, int epi, hipStream_t stream);
-bool gemm_tile_supports(const GemmProblem &p, int kind);
+bool gemm_tile_supports(const GemmProblem &p, int kind, int epi);
 
 static std::atomic<int> g_force_generic{0};
 
 static int run(const GemmProblem &p, int kind, int epi, hipStream_t stream)
 {
     if (p.T == 0 || p.n_out == 0) return CCH_OK;
-    if (!g_force_generic.load() && gemm_tile_supports(p, kind)) return launch_gemm_tile(p, kind, epi, stream);
+    if (!g_force_generic.load() && gemm_tile_supports(p, kind, epi)) return launch_gemm_tile(p, kind, epi, stream);
     return launch_gemm_naive(p, kind, epi, stream);
 }
 

@@ -38,6 +38,7 @@
 
 namespace cch {
 
+typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -174,7 +175,14 @@ struct TileCtx {
     uint32_t off_sc;                    // per lane: scale row * sld (A rows for waves 0-3, B columns for 4-7)
 };
 
-template <int KIND, int EPI, int FMT>
+// TB = 1: B is stored [N, K] (K contiguous) and its panel is staged like A's.  TB = 0 (int8 and
+// MXFP8): B is stored [K, N]; a step's panel is staged as 128 K-rows of 256 bytes and the MFMA
+// operand, which wants K-contiguous bytes per column, is read with the transposing LDS load
+// ds_read_b64_tr_b8.  Inside a group of 16 lanes that load treats the lanes' addresses as 16
+// row segments of 8 bytes and returns to lane j byte (j & 7) of segments (j >> 3), (j >> 3) + 2,
+// ..., (j >> 3) + 14.  Lane i of a group therefore addresses K-row i/2 at columns 8*(i & 1) ..
+// +7, and lane j receives 8 consecutive K bytes of column j.
+template <int KIND, int EPI, int FMT, int TB>
 __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 {
     using KT = KindTraits<KIND>;
@@ -213,8 +221,17 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     // LDS read offsets of this lane inside a stage.
     const uint32_t swz = swizzle_of_row(r);
     const uint32_t rd_a = (uint32_t)(wm * WM + r) * BKB, rd_b = (uint32_t)PANEL_BYTES + (uint32_t)(wn * WN + r) * BKB;
-    const uint32_t rd_sa = (uint32_t)(wm * WM + r) * 16, rd_sb = 4096u + (uint32_t)(wn * WN + r) * 16;
-
+    const uint32_t rd_sa = (uint32_t)(wm * WM + r) * 16;
+    // B scales: TB = 1 like A's, 16 bytes per column; TB = 0 two 512-byte rows per step,
+    // [K64 block][column][2], in the buffer of the step's parity
+    const uint32_t rd_sb = TB ? 4096u + (uint32_t)(wn * WN + r) * 16 : 4096u + (uint32_t)(wn * WN + r) * 2;
+    // TB = 0 fragment reads: lane (q = lane / 16, i = lane % 16) addresses K-row 16*(q/2) + i/2 of
+    // the substep part and the 8-byte half (i & 1) of 16-byte chunk wn*4 + j*2 + (q & 1), whose
+    // position in the row is swizzled by the row's low bits (i / 2)
+    const int tq = lane >> 4, ti = lane & 15;
+    const uint32_t rd_bt = (uint32_t)PANEL_BYTES + (uint32_t)(16 * (tq >> 1) + (ti >> 1)) * 256u +
+                           ((uint32_t)((wn * 4 + (tq & 1)) ^ (ti >> 1)) << 4) + (uint32_t)(ti & 1) * 8u;
+    const int ldb = TB ? lda : p.N;   // bytes between consecutive rows of B as stored
     int gi = 0;           // scale groups requested so far; group n lives in scale buffer n & 1
     int gbase = 0;        // value of gi when the current tile's group 0 was requested
 
@@ -241,23 +258,40 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             const int row = (wave * NJ + j) * 8 + (lane >> 3);
             const uint32_t chunk = ((uint32_t)(lane & 7) ^ swizzle_of_row(row)) * 16u;
             c.off_a[j] = (uint32_t)min(row, c.m_end - 1 - c.m0) * (uint32_t)lda + chunk;
-            int col;  // B row (= logical column) feeding tile row `row`
-            if (SWIGLU) {
-                // tile row = wn*64 + h*32 + c: h = 0 gate, 1 up; output column j0 + wn*32 + c
-                col = ((row >> 5) & 1) * p.n_out + min(c.j0 + (row >> 6) * 32 + (row & 31), p.n_out - 1);
+            if (TB) {
+                int col;  // B row (= logical column) feeding tile row `row`
+                if (SWIGLU) {
+                    // tile row = wn*64 + h*32 + c: h = 0 gate, 1 up; output column j0 + wn*32 + c
+                    col = ((row >> 5) & 1) * p.n_out + min(c.j0 + (row >> 6) * 32 + (row & 31), p.n_out - 1);
+                } else {
+                    col = min(c.j0 + row, p.N - 1);
+                }
+                c.off_b[j] = (uint32_t)col * (uint32_t)lda + chunk;
             } else {
-                col = min(c.j0 + row, p.N - 1);
+                // Instruction j fills K-rows (wave*NJ + j)*4 .. +3 of the panel, 256 bytes each;
+                // lane l lands at row l/16, chunk position l%16 and fetches tile chunk
+                // (l%16) ^ (row & 7): 16 tile columns, clamped to stay inside the row of B.
+                const int kr = (wave * NJ + j) * 4 + (lane >> 4);
+                const int tc = (lane & 15) ^ (kr & 7);
+                int col;
+                if (SWIGLU) col = ((tc >> 1) & 1) * p.n_out + min(c.j0 + (tc >> 2) * 32 + (tc & 1) * 16, p.n_out - 16);
+                else col = min(c.j0 + tc * 16, p.N - 16);
+                c.off_b[j] = (uint32_t)kr * (uint32_t)ldb + (uint32_t)col;
             }
-            c.off_b[j] = (uint32_t)col * (uint32_t)lda + chunk;
         }
         if (MX) {
             const int idx = (wave & 3) * 64 + lane;
             if (wave < 4) {
                 c.rs_sc = make_rsrc(p.sa + (size_t)c.m0 * p.sld, (uint32_t)min((int64_t)(p.T - c.m0) * p.sld, (int64_t)c.lim));
                 c.off_sc = (uint32_t)min(idx, c.m_end - 1 - c.m0) * (uint32_t)p.sld;
-            } else {
+            } else if (TB) {
                 c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride, (uint32_t)min((int64_t)p.N * p.sld, (int64_t)c.lim));
                 c.off_sc = (uint32_t)min(c.j0 + idx, p.N - 1) * (uint32_t)p.sld;
+            } else {
+                // [K/64][N][2]: wave 4 fetches, per step, two 512-byte rows (the step's two
+                // K64 blocks, 256 columns); lane l takes 16 bytes of row l/32
+                c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride, (uint32_t)min((int64_t)p.N * p.sld, (int64_t)c.lim));
+                c.off_sc = (uint32_t)(lane >> 5) * (uint32_t)p.N * 2u + (uint32_t)c.j0 * 2u + (uint32_t)(lane & 31) * 16u;
             }
         }
     };
@@ -271,15 +305,26 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         if constexpr (piece < NJ) {
             load16_to_lds(c.rs_a, c.off_a[piece], (uint32_t)kt * BKB, lds + piece * 1024u);
         } else if constexpr (piece < 2 * NJ) {
-            load16_to_lds(c.rs_b, c.off_b[piece - NJ], (uint32_t)kt * BKB, lds + PANEL_BYTES + (piece - NJ) * 1024u);
+            load16_to_lds(c.rs_b, c.off_b[piece - NJ], TB ? (uint32_t)kt * BKB : (uint32_t)kt * BKB * (uint32_t)ldb,
+                          lds + PANEL_BYTES + (piece - NJ) * 1024u);
         }
     };
     // Scale group `grp` of tile c (16 bytes per row: steps grp*SPG .. grp*SPG+SPG-1) into scale
     // buffer `buf`; waves 0-3 fetch the A rows, waves 4-7 the B rows, one row per lane.
-    auto issue_scales = [&](int enable, const TileCtx &c, int grp, int buf) {
+    // With TB = 0 only waves 0-3 take part (the others issue the instruction with an empty EXEC
+    // mask, which keeps the code free of branches); the B scales then come per step, see below.
+    auto issue_scales = [&](int newgrp, const TileCtx &c, int grp, int buf) {
         if constexpr (MX)
-            load16_to_lds_if(enable, c.rs_sc, c.off_sc, (uint32_t)grp * 16u,
+            load16_to_lds_if(newgrp & (int)(TB || wave < 4), c.rs_sc, c.off_sc, (uint32_t)grp * 16u,
                              lds_base + (uint32_t)(SCALE_OFF + buf * SCALE_BUF) + (uint32_t)(wave >= 4) * 4096u + (uint32_t)(wave & 3) * 1024u);
+    };
+    // TB = 0: B scales of K-step kt, stored [K/64][N][2]: two 512-byte rows (the step's two K64
+    // blocks x 256 columns), fetched by wave 4 into the B half of the scale buffer of the
+    // step's ring stage.
+    auto issue_bscale = [&](const TileCtx &c, int kt, int stage) {
+        if constexpr (MX && !TB)
+            load16_to_lds_if(wave == 4, c.rs_sc, c.off_sc, (uint32_t)kt * 4u * (uint32_t)p.N,
+                             lds_base + (uint32_t)(SCALE_OFF + stage * SCALE_BUF) + 4096u);
     };
     auto issue_step = [&](const TileCtx &c, int kt, int stage) {
         static_for<NV>([&](auto piece_c) { issue_piece(c, kt, stage, piece_c); });
@@ -300,6 +345,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         }
         issue_scales(1, c, 0, gi & 1);
         gi++;
+        issue_bscale(c, 0, stage);
         issue_step(c, 0, stage);
     };
 
@@ -311,6 +357,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     nxt.valid = 0;
     if (cur.valid) {
         setup(cur, 0, 0);
+        issue_bscale(cur, 1, 1);
         issue_step(cur, 1, 1);
     }
     while (cur.valid) {
@@ -337,9 +384,22 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         };
         auto frag_a = [&](int stage, int ks, int i) { return read_frag((uint32_t)(RING_OFF + stage * STAGE_BYTES) + rd_a + i * 32 * BKB, ks); };
-        auto frag_b = [&](int stage, int ks, int j) { return read_frag((uint32_t)(RING_OFF + stage * STAGE_BYTES) + rd_b + j * 32 * BKB, ks); };
+        auto frag_b = [&](int stage, int ks, int j) {
+            if constexpr (TB) {
+                return read_frag((uint32_t)(RING_OFF + stage * STAGE_BYTES) + rd_b + j * 32 * BKB, ks);
+            } else {
+                // four transposing loads: K bytes 16g+0..7, 16g+8..15, 32+16g+0..7, 32+16g+8..15 of the substep
+                const uint32_t base = (uint32_t)(RING_OFF + stage * STAGE_BYTES) + (rd_bt ^ ((uint32_t)j << 5)) + (uint32_t)ks * (64u * 256u);
+                typedef __attribute__((address_space(3))) v2i *LdsV2;
+                const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base));
+                const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 8u * 256u));
+                const v2i t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 32u * 256u));
+                const v2i t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 40u * 256u));
+                return (v8i){t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
+            }
+        };
         // Scale dwords of K-step kt of the current tile
-        auto read_scales = [&](int kt, uint32_t (&dst)[NSC][MT + NT]) {
+        auto read_scales = [&](int kt, int kt_stage, uint32_t (&dst)[NSC][MT + NT]) {
             if (!MX) return;
             const uint32_t ss = (uint32_t)(SCALE_OFF + ((gbase + kt / SPG) & 1) * SCALE_BUF) + (uint32_t)(kt % SPG) * (SCALE_DW * 4u);
 #pragma unroll
@@ -347,7 +407,16 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 #pragma unroll
                 for (int s = 0; s < MT; s++) dst[d][s] = lds_read4(ss + rd_sa + s * 512 + d * 4);
 #pragma unroll
-                for (int s = 0; s < NT; s++) dst[d][MT + s] = lds_read4(ss + rd_sb + s * 512 + d * 4);
+                for (int s = 0; s < NT; s++) {
+                    if constexpr (TB) {
+                        dst[d][MT + s] = lds_read4(ss + rd_sb + s * 512 + d * 4);
+                    } else {
+                        // bytes 2*ks + g of the step's dword: the two blocks of K64 block ks sit side by side
+                        const uint32_t sb0 = (uint32_t)(SCALE_OFF + kt_stage * SCALE_BUF) + rd_sb + s * 64;
+                        dst[d][MT + s] = (uint32_t)*reinterpret_cast<const uint16_t *>(smem + sb0) |
+                                         ((uint32_t)*reinterpret_cast<const uint16_t *>(smem + sb0 + 512) << 16);
+                    }
+                }
             }
         };
         // One MFMA of row block i of a 64-byte substep; m = 0 .. MPR-1 walks the row: all
@@ -422,20 +491,24 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                         nbase = gi;
                         setup(nxt, parity ^ 1, stage);
                     } else if constexpr (MODE == 2) {
+                        issue_bscale(nxt, 1, stage);
                         issue_step(nxt, 1, stage);
                     }
                 } else if constexpr (MODE == 0) {
                     static_for<PER_SLOT>([&](auto q_c) {
                         constexpr int piece = (slot - 1) * PER_SLOT + decltype(q_c)::value;
                         if constexpr (piece < NV) issue_piece(cur, kt + 2, stage, IC<piece>{});
-                        else if constexpr (piece == NV && MX) issue_scales(newgrp, cur, (kt + 2) / SPG, gi & 1);
+                        else if constexpr (piece == NV && MX) {
+                            issue_scales(newgrp, cur, (kt + 2) / SPG, gi & 1);
+                            issue_bscale(cur, kt + 2, stage);
+                        }
                     });
                 }
                 if constexpr (MODE != 2 && m == MPR - 1) fa[i] = frag_a(nstage, 0, i);
                 __builtin_amdgcn_sched_barrier(0);
             });
             if constexpr (MODE == 0) gi += MX ? newgrp : 0;
-            if constexpr (MODE != 2) read_scales(kt + 1, sc);
+            if constexpr (MODE != 2) read_scales(kt + 1, nstage, sc);
             if constexpr (MODE != 0) {
                 // Pin the accumulators here: otherwise the compiler sinks the MFMAs of the
                 // peeled steps into the epilogue and spills their fragments to get them there.
@@ -449,12 +522,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // Tile prologue.  In flight, oldest first: this tile's set-up and first step, its
         // second step (NV requests), then the previous tile's epilogue stores.
         constexpr int NSTORES = MT * NPASS;
-        if (first) CCH_WAIT_VM_LGKM0(NV);
-        else CCH_WAIT_VM_LGKM0(NV + NSTORES);
+        constexpr int NSTEP1 = NV + (MX && !TB ? 1 : 0);  // requests of the tile's second step
+        if (first) CCH_WAIT_VM_LGKM0(NSTEP1);
+        else CCH_WAIT_VM_LGKM0(NSTEP1 + NSTORES);
         __syncthreads();
         {
             const int stage = gstep & 1;
-            read_scales(0, sc);
+            read_scales(0, stage, sc);
 #pragma unroll
             for (int j = 0; j < NT; j++) fb0[j] = frag_b(stage, 0, j);
 #pragma unroll
@@ -552,11 +626,11 @@ __global__ __launch_bounds__(256) void zero_tail_rows_kernel(uint16_t *out, cons
     for (size_t i = begin + (size_t)blockIdx.x * 256 + threadIdx.x; i < end; i += (size_t)gridDim.x * 256) out[i] = 0;
 }
 
-template <int KIND, int EPI, int FMT>
+template <int KIND, int EPI, int FMT, int TB>
 static int launch_tile_t(const GemmProblem &p, hipStream_t stream)
 {
     static bool attr_set = false;
-    auto kern = gemm_tile_kernel<KIND, EPI, FMT>;
+    auto kern = gemm_tile_kernel<KIND, EPI, FMT, TB>;
     if (!attr_set) {
         CCH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
         attr_set = true;
@@ -576,11 +650,10 @@ static int launch_tile_t(const GemmProblem &p, hipStream_t stream)
 }
 
 // True when the tiled kernels take this problem; otherwise the caller uses the generic path.
-bool gemm_tile_supports(const GemmProblem &p, int kind)
+bool gemm_tile_supports(const GemmProblem &p, int kind, int epi)
 {
     const int epb = kind == KIND_F4 ? 2 : 1;
-    if (!p.trans_b) return false;
-    // whole 128-byte K-steps; output rows must take 16-byte stores
+    // whole 128-byte K-steps, at least two of them; output rows must take 16-byte stores
     if (p.K < 2 * BKB * epb || p.K % (BKB * epb) != 0) return false;
     if (p.n_out % 8 != 0 || !aligned(p.out, 16)) return false;
     if ((int64_t)BM * p.n_out * 2 >= ((int64_t)1 << 31)) return false;
@@ -588,17 +661,29 @@ bool gemm_tile_supports(const GemmProblem &p, int kind)
     if ((int64_t)p.N * (p.K / epb) >= ((int64_t)1 << 31)) return false;  // 32-bit source offsets
     if (!aligned(p.a, 16) || !aligned(p.b, 16) || p.b_stride % 16 != 0) return false;
     if (kind != KIND_I8 && (!aligned(p.sa, 4) || !aligned(p.sb, 4) || p.sb_stride % 4 != 0 || p.sld % 4 != 0)) return false;
+    if (!p.trans_b) {
+        // [K, N] operands: byte-wide kinds only (the FP4 nibble transpose is not implemented);
+        // 16-byte pieces of a row of B must not straddle its end
+        if (kind == KIND_F4) return false;
+        if ((epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) % 16 != 0 || (epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) < 16) return false;
+        if (kind != KIND_I8 && p.K % 64 != 0) return false;
+    }
     return true;
 }
 
 int launch_gemm_tile(const GemmProblem &p, int kind, int epi, hipStream_t stream)
 {
-    if (kind == KIND_I8 && epi == EPI_DEQUANT) return launch_tile_t<KIND_I8, EPI_DEQUANT, 0>(p, stream);
-    if (kind == KIND_I8 && epi == EPI_DEQUANT_SWIGLU) return launch_tile_t<KIND_I8, EPI_DEQUANT_SWIGLU, 0>(p, stream);
-    if (kind == KIND_F8 && epi == EPI_PLAIN && p.fmt == CCH_FMT_E4M3) return launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E4M3>(p, stream);
-    if (kind == KIND_F8 && epi == EPI_PLAIN && p.fmt == CCH_FMT_E5M2) return launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E5M2>(p, stream);
-    if (kind == KIND_F4 && epi == EPI_PLAIN) return launch_tile_t<KIND_F4, EPI_PLAIN, CCH_FMT_E2M1>(p, stream);
-    return fail(CCH_ENOSUP, "no tiled GEMM kernel for kind %d with epilogue %d", kind, epi);
+    const bool tb = p.trans_b != 0;
+    if (kind == KIND_I8 && epi == EPI_DEQUANT)
+        return tb ? launch_tile_t<KIND_I8, EPI_DEQUANT, 0, 1>(p, stream) : launch_tile_t<KIND_I8, EPI_DEQUANT, 0, 0>(p, stream);
+    if (kind == KIND_I8 && epi == EPI_DEQUANT_SWIGLU)
+        return tb ? launch_tile_t<KIND_I8, EPI_DEQUANT_SWIGLU, 0, 1>(p, stream) : launch_tile_t<KIND_I8, EPI_DEQUANT_SWIGLU, 0, 0>(p, stream);
+    if (kind == KIND_F8 && epi == EPI_PLAIN && p.fmt == CCH_FMT_E4M3)
+        return tb ? launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E4M3, 1>(p, stream) : launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E4M3, 0>(p, stream);
+    if (kind == KIND_F8 && epi == EPI_PLAIN && p.fmt == CCH_FMT_E5M2)
+        return tb ? launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E5M2, 1>(p, stream) : launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E5M2, 0>(p, stream);
+    if (kind == KIND_F4 && epi == EPI_PLAIN && tb) return launch_tile_t<KIND_F4, EPI_PLAIN, CCH_FMT_E2M1, 1>(p, stream);
+    return fail(CCH_ENOSUP, "no tiled GEMM kernel for kind %d with epilogue %d, trans_b %d", kind, epi, p.trans_b);
 }
 
 }  // namespace cch
