@@ -11,11 +11,15 @@ int launch_gemm_tile(const GemmProblem &p, int kind, int epi, hipStream_t stream
 bool gemm_tile_supports(const GemmProblem &p, int kind, int epi);
 
 static std::atomic<int> g_force_generic{0};
+static std::atomic<int> g_require_tiled{0};
 
 static int run(const GemmProblem &p, int kind, int epi, hipStream_t stream)
 {
     if (p.T == 0 || p.n_out == 0) return CCH_OK;
     if (!g_force_generic.load() && gemm_tile_supports(p, kind, epi)) return launch_gemm_tile(p, kind, epi, stream);
+    if (g_require_tiled.load())
+        return fail(CCH_ENOSUP, "the tiled MFMA kernels do not take this problem (T=%d N=%d K=%d trans_b=%d) and "
+                                "require_tiled_gemm is set", p.T, p.N, p.K, p.trans_b);
     return launch_gemm_naive(p, kind, epi, stream);
 }
 
@@ -36,6 +40,10 @@ int cch_set_option(const char *name, int value)
     CCH_REQUIRE(name != nullptr, "cch_set_option: null name");
     if (strcmp(name, "force_generic_gemm") == 0) {
         g_force_generic.store(value);
+        return CCH_OK;
+    }
+    if (strcmp(name, "require_tiled_gemm") == 0) {
+        g_require_tiled.store(value);
         return CCH_OK;
     }
     return fail(CCH_EINVAL, "cch_set_option: unknown option %s", name);

@@ -228,10 +228,20 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     // TB = 0 fragment reads: lane (q = lane / 16, i = lane % 16) addresses K-row 16*(q/2) + i/2 of
     // the substep part and the 8-byte half (i & 1) of 16-byte chunk wn*4 + j*2 + (q & 1), whose
     // position in the row is swizzled by the row's low bits (i / 2)
+    // For FP4 the panel has 256 K-rows of 128 bytes (two columns per byte) and the 4-bit form of
+    // the load is a 16 x 16 nibble transpose: lane i addresses K-row i at 16 columns (8 bytes) and
+    // lane j receives 16 consecutive K nibbles of column j; the chunk swizzle uses row bits 1..3.
+    constexpr bool FP4K = KIND == KIND_F4;
+    constexpr int EPB = KT::ELEMS_PER_BYTE;
+    constexpr int BROW = BN / EPB;               // bytes per K-row of the TB = 0 panel
+    constexpr int BCPR = BROW / 16;              // 16-byte chunks per K-row
+    constexpr int BRPI = 64 / BCPR;              // K-rows filled by one direct-to-LDS instruction
     const int tq = lane >> 4, ti = lane & 15;
-    const uint32_t rd_bt = (uint32_t)PANEL_BYTES + (uint32_t)(16 * (tq >> 1) + (ti >> 1)) * 256u +
-                           ((uint32_t)((wn * 4 + (tq & 1)) ^ (ti >> 1)) << 4) + (uint32_t)(ti & 1) * 8u;
-    const int ldb = TB ? lda : p.N;   // bytes between consecutive rows of B as stored
+    const uint32_t rd_bt = FP4K ? (uint32_t)PANEL_BYTES + (uint32_t)(32 * (tq >> 1) + ti) * 128u +
+                                      ((uint32_t)((wn * 2) ^ (ti >> 1)) << 4) + (uint32_t)(tq & 1) * 8u
+                                : (uint32_t)PANEL_BYTES + (uint32_t)(16 * (tq >> 1) + (ti >> 1)) * 256u +
+                                      ((uint32_t)((wn * 4 + (tq & 1)) ^ (ti >> 1)) << 4) + (uint32_t)(ti & 1) * 8u;
+    const int ldb = TB ? lda : p.N / EPB;   // bytes between consecutive rows of B as stored
     int gi = 0;           // scale groups requested so far; group n lives in scale buffer n & 1
     int gbase = 0;        // value of gi when the current tile's group 0 was requested
 
@@ -271,12 +281,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 // Instruction j fills K-rows (wave*NJ + j)*4 .. +3 of the panel, 256 bytes each;
                 // lane l lands at row l/16, chunk position l%16 and fetches tile chunk
                 // (l%16) ^ (row & 7): 16 tile columns, clamped to stay inside the row of B.
-                const int kr = (wave * NJ + j) * 4 + (lane >> 4);
-                const int tc = (lane & 15) ^ (kr & 7);
+                const int kr = (wave * NJ + j) * BRPI + lane / BCPR;
+                const int tc = (lane % BCPR) ^ (FP4K ? (kr >> 1) & 7 : kr & 7);
+                constexpr int CPC = 16 * EPB;  // columns per chunk
                 int col;
                 if (SWIGLU) col = ((tc >> 1) & 1) * p.n_out + min(c.j0 + (tc >> 2) * 32 + (tc & 1) * 16, p.n_out - 16);
-                else col = min(c.j0 + tc * 16, p.N - 16);
-                c.off_b[j] = (uint32_t)kr * (uint32_t)ldb + (uint32_t)col;
+                else col = min(c.j0 + tc * CPC, p.N - CPC);
+                c.off_b[j] = (uint32_t)kr * (uint32_t)ldb + (uint32_t)(col / EPB);
             }
         }
         if (MX) {
@@ -291,7 +302,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 // [K/64][N][2]: wave 4 fetches, per step, two 512-byte rows (the step's two
                 // K64 blocks, 256 columns); lane l takes 16 bytes of row l/32
                 c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride, (uint32_t)min((int64_t)p.N * p.sld, (int64_t)c.lim));
-                c.off_sc = (uint32_t)(lane >> 5) * (uint32_t)p.N * 2u + (uint32_t)c.j0 * 2u + (uint32_t)(lane & 31) * 16u;
+                c.off_sc = (uint32_t)((lane >> 5) + 2 * (wave - 4)) * (uint32_t)p.N * 2u + (uint32_t)c.j0 * 2u + (uint32_t)(lane & 31) * 16u;
             }
         }
     };
@@ -305,7 +316,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         if constexpr (piece < NJ) {
             load16_to_lds(c.rs_a, c.off_a[piece], (uint32_t)kt * BKB, lds + piece * 1024u);
         } else if constexpr (piece < 2 * NJ) {
-            load16_to_lds(c.rs_b, c.off_b[piece - NJ], TB ? (uint32_t)kt * BKB : (uint32_t)kt * BKB * (uint32_t)ldb,
+            load16_to_lds(c.rs_b, c.off_b[piece - NJ], TB ? (uint32_t)kt * BKB : (uint32_t)kt * (BKB * EPB) * (uint32_t)ldb,
                           lds + PANEL_BYTES + (piece - NJ) * 1024u);
         }
     };
@@ -318,13 +329,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             load16_to_lds_if(newgrp & (int)(TB || wave < 4), c.rs_sc, c.off_sc, (uint32_t)grp * 16u,
                              lds_base + (uint32_t)(SCALE_OFF + buf * SCALE_BUF) + (uint32_t)(wave >= 4) * 4096u + (uint32_t)(wave & 3) * 1024u);
     };
-    // TB = 0: B scales of K-step kt, stored [K/64][N][2]: two 512-byte rows (the step's two K64
-    // blocks x 256 columns), fetched by wave 4 into the B half of the scale buffer of the
-    // step's ring stage.
+    // TB = 0: B scales of K-step kt, stored [K/64][N][2]: one 512-byte row per K64 block of the
+    // step (2 for MXFP8, 4 for MXFP4) x 256 columns, two rows per wave starting at wave 4, into
+    // the B half of the scale buffer of the step's ring stage.
     auto issue_bscale = [&](const TileCtx &c, int kt, int stage) {
         if constexpr (MX && !TB)
-            load16_to_lds_if(wave == 4, c.rs_sc, c.off_sc, (uint32_t)kt * 4u * (uint32_t)p.N,
-                             lds_base + (uint32_t)(SCALE_OFF + stage * SCALE_BUF) + 4096u);
+            load16_to_lds_if(wave >= 4 && wave < 4 + SCALE_DW, c.rs_sc, c.off_sc, (uint32_t)kt * (4u * SCALE_DW) * (uint32_t)p.N,
+                             lds_base + (uint32_t)(SCALE_OFF + stage * SCALE_BUF) + 4096u + (uint32_t)(wave & 3) * 1024u);
     };
     auto issue_step = [&](const TileCtx &c, int kt, int stage) {
         static_for<NV>([&](auto piece_c) { issue_piece(c, kt, stage, piece_c); });
@@ -388,13 +399,23 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             if constexpr (TB) {
                 return read_frag((uint32_t)(RING_OFF + stage * STAGE_BYTES) + rd_b + j * 32 * BKB, ks);
             } else {
-                // four transposing loads: K bytes 16g+0..7, 16g+8..15, 32+16g+0..7, 32+16g+8..15 of the substep
-                const uint32_t base = (uint32_t)(RING_OFF + stage * STAGE_BYTES) + (rd_bt ^ ((uint32_t)j << 5)) + (uint32_t)ks * (64u * 256u);
                 typedef __attribute__((address_space(3))) v2i *LdsV2;
-                const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base));
-                const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 8u * 256u));
-                const v2i t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 32u * 256u));
-                const v2i t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 40u * 256u));
+                v2i t0, t1, t2, t3;
+                if constexpr (FP4K) {
+                    // four nibble transposes: K elements 32g+0..15, 32g+16..31, 64+32g+0..15, 64+32g+16..31 of the substep
+                    const uint32_t base = (uint32_t)(RING_OFF + stage * STAGE_BYTES) + (rd_bt ^ ((uint32_t)j << 4)) + (uint32_t)ks * (128u * 128u);
+                    t0 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base));
+                    t1 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 16u * 128u));
+                    t2 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 64u * 128u));
+                    t3 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 80u * 128u));
+                } else {
+                    // four byte transposes: K bytes 16g+0..7, 16g+8..15, 32+16g+0..7, 32+16g+8..15 of the substep
+                    const uint32_t base = (uint32_t)(RING_OFF + stage * STAGE_BYTES) + (rd_bt ^ ((uint32_t)j << 5)) + (uint32_t)ks * (64u * 256u);
+                    t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base));
+                    t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 8u * 256u));
+                    t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 32u * 256u));
+                    t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 40u * 256u));
+                }
                 return (v8i){t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
             }
         };
@@ -412,7 +433,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                         dst[d][MT + s] = lds_read4(ss + rd_sb + s * 512 + d * 4);
                     } else {
                         // bytes 2*ks + g of the step's dword: the two blocks of K64 block ks sit side by side
-                        const uint32_t sb0 = (uint32_t)(SCALE_OFF + kt_stage * SCALE_BUF) + rd_sb + s * 64;
+                        const uint32_t sb0 = (uint32_t)(SCALE_OFF + kt_stage * SCALE_BUF) + rd_sb + s * 64 + d * 1024;
                         dst[d][MT + s] = (uint32_t)*reinterpret_cast<const uint16_t *>(smem + sb0) |
                                          ((uint32_t)*reinterpret_cast<const uint16_t *>(smem + sb0 + 512) << 16);
                     }
@@ -662,10 +683,9 @@ bool gemm_tile_supports(const GemmProblem &p, int kind, int epi)
     if (!aligned(p.a, 16) || !aligned(p.b, 16) || p.b_stride % 16 != 0) return false;
     if (kind != KIND_I8 && (!aligned(p.sa, 4) || !aligned(p.sb, 4) || p.sb_stride % 4 != 0 || p.sld % 4 != 0)) return false;
     if (!p.trans_b) {
-        // [K, N] operands: byte-wide kinds only (the FP4 nibble transpose is not implemented);
-        // 16-byte pieces of a row of B must not straddle its end
-        if (kind == KIND_F4) return false;
-        if ((epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) % 16 != 0 || (epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) < 16) return false;
+        // [K, N] operands: 16-byte pieces of a row of B must not straddle its end
+        const int cpc = 16 * epb;  // columns per 16-byte piece
+        if ((epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) % cpc != 0 || (epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) < cpc) return false;
         if (kind != KIND_I8 && p.K % 64 != 0) return false;
     }
     return true;
@@ -682,7 +702,8 @@ int launch_gemm_tile(const GemmProblem &p, int kind, int epi, hipStream_t stream
         return tb ? launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E4M3, 1>(p, stream) : launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E4M3, 0>(p, stream);
     if (kind == KIND_F8 && epi == EPI_PLAIN && p.fmt == CCH_FMT_E5M2)
         return tb ? launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E5M2, 1>(p, stream) : launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E5M2, 0>(p, stream);
-    if (kind == KIND_F4 && epi == EPI_PLAIN && tb) return launch_tile_t<KIND_F4, EPI_PLAIN, CCH_FMT_E2M1, 1>(p, stream);
+    if (kind == KIND_F4 && epi == EPI_PLAIN)
+        return tb ? launch_tile_t<KIND_F4, EPI_PLAIN, CCH_FMT_E2M1, 1>(p, stream) : launch_tile_t<KIND_F4, EPI_PLAIN, CCH_FMT_E2M1, 0>(p, stream);
     return fail(CCH_ENOSUP, "no tiled GEMM kernel for kind %d with epilogue %d, trans_b %d", kind, epi, p.trans_b);
 }
 

@@ -127,8 +127,10 @@ int cch_mx_gemm(const void *a, const void *sa, const void *b, const void *sb, vo
 int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes, void *out,
                int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, void *stream);
 
-/* Library switches for tests: "force_generic_gemm" = 1 routes every GEMM entry point through
- * the shape-agnostic one-thread-per-element kernels instead of the tiled MFMA kernels. */
+/* Library switches for tests and benchmarks: "force_generic_gemm" = 1 routes every GEMM entry
+ * point through the shape-agnostic one-thread-per-element kernels instead of the tiled MFMA
+ * kernels; "require_tiled_gemm" = 1 makes a GEMM entry point return CCH_ENOSUP instead of
+ * falling back to them when the tiled kernels do not take the problem. */
 int cch_set_option(const char *name, int value);
 
 #ifdef __cplusplus

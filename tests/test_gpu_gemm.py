@@ -168,3 +168,79 @@ def test_mx_gmm(fmt, cfg, trans_b, path):
     got = out_f32(cc.mx_grouped_matmul(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), fmt, trans_b))
     assert_close(got, want)
     assert np.all(got[int(gs.sum()):] == 0)
+
+
+# ---------------------------------------------------------------- shapes chosen for the tiled MFMA kernels
+# Every case below must run on the tiled kernels (require_tiled_gemm makes a silent fall-back to
+# the generic kernels an error): several K-steps, ragged last row and column tiles, both operand
+# layouts of B, empty and one-row groups.
+
+@pytest.fixture
+def tiled_only():
+    cc.set_option("force_generic_gemm", 0)
+    cc.set_option("require_tiled_gemm", 1)
+    yield
+    cc.set_option("require_tiled_gemm", 0)
+
+
+@pytest.mark.parametrize("shape", [(300, 528, 512), (513, 272, 768), (1, 16, 256), (1024, 1040, 1280)])
+@pytest.mark.parametrize("trans_b", [0, 1])
+def test_i8_dequant_tiled(shape, trans_b, tiled_only):
+    m, n, k = shape
+    rng = np.random.default_rng(100 + m + trans_b)
+    a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    pt = rng.uniform(0.001, 0.02, m).astype(np.float32)
+    pc = rng.uniform(0.001, 0.02, n).astype(np.float32)
+    want = orc.gemm_i8_dequant(a, b, pt, pc)
+    bb = np.ascontiguousarray(b.T) if trans_b else b
+    got = out_f32(cc.w8a8_matmul_dequant(dev(a), dev(bb), dev(pt), dev(pc), trans_b))
+    assert_close(got, want, ("i8 tiled", shape, trans_b))
+
+
+@pytest.mark.parametrize("cfg", [(4, 700, 512, 1056, [300, 0, 143, 257]), (3, 300, 256, 512, [1, 0, 299]), (6, 2000, 768, 2080, None)])
+@pytest.mark.parametrize("trans_b", [0, 1])
+def test_gmm_swiglu_tiled(cfg, trans_b, tiled_only):
+    e, t, k, n, gs = cfg
+    rng = np.random.default_rng(200 + t + trans_b)
+    gs = np.array(gs, np.int32) if gs is not None else zipf_groups(rng, t, e)
+    x = rng.integers(-127, 128, (t, k)).astype(np.int8)
+    w = rng.integers(-127, 128, (e, k, n)).astype(np.int8)
+    pt = rng.uniform(0.001, 0.02, t).astype(np.float32)
+    pc = rng.uniform(0.001, 0.02, (e, n)).astype(np.float32)
+    want = orc.gmm_i8_dequant_swiglu(x, w, gs, pt, pc)
+    ww = np.ascontiguousarray(w.transpose(0, 2, 1)) if trans_b else w
+    got = out_f32(cc.gmm_dequant_swiglu(dev(x), dev(ww), dev(gs), dev(pt), dev(pc), trans_b))
+    assert_close(got, want, ("swiglu tiled", cfg[:4], trans_b))
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
+@pytest.mark.parametrize("shape", [(300, 544, 1024), (513, 288, 768), (2, 32, 512), (700, 1312, 1536)])
+@pytest.mark.parametrize("trans_b", [0, 1])
+def test_mx_gemm_tiled(fmt, shape, trans_b, tiled_only):
+    m, n, k = shape
+    rng = np.random.default_rng(300 + m + trans_b)
+    pa, sa, pb, sb = mx_operands(rng, m, n, k, fmt, trans_b)
+    want = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], trans_b)
+    got = out_f32(cc.mx_matmul(dev(pa), dev(sa), dev(pb), dev(sb), fmt, trans_b))
+    assert_close(got, want, ("mx tiled", fmt, shape, trans_b))
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e2m1"])
+@pytest.mark.parametrize("cfg", [(5, 900, 1024, 416, [0, 300, 1, 0, 500]), (8, 3000, 768, 1056, None)])
+@pytest.mark.parametrize("trans_b", [0, 1])
+def test_mx_gmm_tiled(fmt, cfg, trans_b, tiled_only):
+    e, t, k, n, gs = cfg
+    rng = np.random.default_rng(400 + t + trans_b)
+    gs = np.array(gs, np.int32) if gs is not None else zipf_groups(rng, t - 37, e)   # leaves 37 rows that belong to no group
+    sigma = 0.02 if fmt == "e2m1" else 1.0
+    pa, sa = orc.mx_quant_rows(rand_bf16(rng, (t, k), sigma), FMT[fmt])
+    pbs, sbs = [], []
+    for _ in range(e):
+        pb, sb = orc.mx_quant_b(rand_bf16(rng, (k, n), sigma), FMT[fmt], orc.RNE, trans_b)
+        pbs.append(pb)
+        sbs.append(sb)
+    pb, sb = np.stack(pbs), np.stack(sbs)
+    want = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], trans_b, group_sizes=gs)
+    got = out_f32(cc.mx_grouped_matmul(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), fmt, trans_b))
+    assert_close(got, want, ("mx gmm tiled", fmt, cfg[:4], trans_b))
