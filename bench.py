@@ -133,13 +133,14 @@ def main():
 
     # ------------------------------------------------------------ workload (config 5 shapes, E4M3 payload)
     E, T, K, N = 32, 16384, 7168, 4096
-    TRANS_B = 1   # W stored [E, N, K] (K-contiguous), the layout the reference's MXFP8 run uses (transB=1)
+    TRANS_B = 0   # W stored [E, K, N] as the configurations name it (B scales [E, K/64, N, 2])
+    cc.set_option("require_tiled_gemm", 1)   # a fall-back to the generic kernels is an error here, not a slow number
     gs_host = zipf_groups(rng, T, E)
     gs = torch.from_numpy(gs_host).to(dev)
     x0 = (torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16)
     a, sa = cc.mx_quant(x0, "e4m3")
-    b = torch.empty((E, N, K), dtype=torch.uint8, device=dev)
-    sb = torch.empty((E, N, K // 32), dtype=torch.uint8, device=dev)
+    b = torch.empty((E, K, N), dtype=torch.uint8, device=dev)
+    sb = torch.empty((E, K // 64, N, 2), dtype=torch.uint8, device=dev)
     for e in range(E):
         w0 = (torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16)
         b[e], sb[e] = cc.mx_quant_b(w0, "e4m3", trans_b=TRANS_B)
@@ -175,7 +176,7 @@ def main():
                    "n": N, "trans_b": TRANS_B, "group_sizes": gs_host.tolist()},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / FP8_PEAK_TFLOPS, 4), "traffic": GMM_TRAFFIC_BYTES,
-                     "kernel": "gemm_tile_kernel<KIND_F8, EPI_PLAIN, E4M3>", "algorithmic_flop_per_launch": flop,
+                     "kernel": "gemm_tile_kernel<KIND_F8, EPI_PLAIN, E4M3, TB=0>", "algorithmic_flop_per_launch": flop,
                      "kernel_ms_min": round(float(np.min(per_ms)), 4), "kernel_ms_mean": round(kernel_ms, 4)},
     }
 
@@ -217,38 +218,38 @@ def main():
         # config 2: int8 W8A8 + dequant
         m2, k2, n2 = 8192, 4096, 8192
         a2 = torch.randint(-127, 128, (m2, k2), dtype=torch.int8, device=dev)
-        b2 = torch.randint(-127, 128, (n2, k2), dtype=torch.int8, device=dev)
+        b2 = torch.randint(-127, 128, (k2, n2), dtype=torch.int8, device=dev)
         pt2 = torch.rand(m2, device=dev) * 0.019 + 0.001
         pc2 = torch.rand(n2, device=dev) * 0.019 + 0.001
-        _, t2 = event_time_ms(lambda: cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, 1), 10, 3)
+        _, t2 = event_time_ms(lambda: cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, TRANS_B), 10, 3)
         extra["w8a8_dequant_cfg2"] = {"tops": round(2.0 * m2 * n2 * k2 / (np.mean(t2) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t2)) * 1e3, 1)}
         extra["w8a8_dequant_cfg2"]["frac_of_int8_peak"] = round(extra["w8a8_dequant_cfg2"]["tops"] / FP8_PEAK_TFLOPS, 4)
         del a2, b2
         # config 3: MXFP8 dense
         m3, k3, n3 = 4096, 2048, 7168
         a3, sa3 = cc.mx_quant(torch.randn(m3, k3, device=dev).to(torch.bfloat16), "e4m3")
-        b3, sb3 = cc.mx_quant_b(torch.randn(k3, n3, device=dev).to(torch.bfloat16), "e4m3", trans_b=1)
-        _, t3 = event_time_ms(lambda: cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", 1), 20, 5)
+        b3, sb3 = cc.mx_quant_b(torch.randn(k3, n3, device=dev).to(torch.bfloat16), "e4m3", trans_b=TRANS_B)
+        _, t3 = event_time_ms(lambda: cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", TRANS_B), 20, 5)
         extra["mxfp8_dense_cfg3"] = {"tflops": round(2.0 * m3 * n3 * k3 / (np.mean(t3) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t3)) * 1e3, 1)}
         extra["mxfp8_dense_cfg3"]["frac_of_fp8_peak"] = round(extra["mxfp8_dense_cfg3"]["tflops"] / FP8_PEAK_TFLOPS, 4)
         # config 4: MoE W8A8 grouped + dequant + SwiGLU
         e4, t4, k4, n4 = 16, 8192, 7168, 4096
         gs4 = torch.from_numpy(zipf_groups(rng, t4, e4)).to(dev)
         x4 = torch.randint(-127, 128, (t4, k4), dtype=torch.int8, device=dev)
-        w4 = torch.randint(-127, 128, (e4, n4, k4), dtype=torch.int8, device=dev)
+        w4 = torch.randint(-127, 128, (e4, k4, n4), dtype=torch.int8, device=dev)
         pt4 = torch.rand(t4, device=dev) * 0.019 + 0.001
         pc4 = torch.rand(e4, n4, device=dev) * 0.019 + 0.001
-        _, tt4 = event_time_ms(lambda: cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, 1), 10, 3)
+        _, tt4 = event_time_ms(lambda: cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), 10, 3)
         extra["moe_w8a8_swiglu_cfg4"] = {"tops": round(2.0 * t4 * n4 * k4 / (np.mean(tt4) * 1e-3) / 1e12, 1), "us": round(float(np.mean(tt4)) * 1e3, 1)}
         extra["moe_w8a8_swiglu_cfg4"]["frac_of_int8_peak"] = round(extra["moe_w8a8_swiglu_cfg4"]["tops"] / FP8_PEAK_TFLOPS, 4)
         del x4, w4
         # config 5: MXFP4 grouped (same groups as the headline)
         a5, sa5 = cc.mx_quant((torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16), "e2m1")
-        b5 = torch.empty((E, N, K // 2), dtype=torch.uint8, device=dev)
-        sb5 = torch.empty((E, N, K // 32), dtype=torch.uint8, device=dev)
+        b5 = torch.empty((E, K, N // 2), dtype=torch.uint8, device=dev)
+        sb5 = torch.empty((E, K // 64, N, 2), dtype=torch.uint8, device=dev)
         for e in range(E):
-            b5[e], sb5[e] = cc.mx_quant_b((torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16), "e2m1", trans_b=1)
-        _, t5 = event_time_ms(lambda: cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", 1), 10, 3)
+            b5[e], sb5[e] = cc.mx_quant_b((torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16), "e2m1", trans_b=TRANS_B)
+        _, t5 = event_time_ms(lambda: cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", TRANS_B), 10, 3)
         extra["mxfp4_grouped_cfg5"] = {"tflops": round(flop / (np.mean(t5) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t5)) * 1e3, 1)}
         extra["mxfp4_grouped_cfg5"]["frac_of_fp4_peak"] = round(extra["mxfp4_grouped_cfg5"]["tflops"] / FP4_PEAK_TFLOPS, 4)
         result["extra"] = extra
