@@ -243,6 +243,30 @@ def main():
         extra["moe_w8a8_swiglu_cfg4"] = {"tops": round(2.0 * t4 * n4 * k4 / (np.mean(tt4) * 1e-3) / 1e12, 1), "us": round(float(np.mean(tt4)) * 1e3, 1)}
         extra["moe_w8a8_swiglu_cfg4"]["frac_of_int8_peak"] = round(extra["moe_w8a8_swiglu_cfg4"]["tops"] / FP8_PEAK_TFLOPS, 4)
         del x4, w4
+        # input side of config 4: per-token dynamic int8 quantisation of the bf16 tokens (queued launches through the C ABI)
+        from catccos_amd import _abi
+        xs4 = [torch.randn(t4, k4, device=dev).to(torch.bfloat16) for _ in range(4)]
+        q4 = torch.empty((t4, k4), dtype=torch.int8, device=dev)
+        s4 = torch.empty((t4,), dtype=torch.float32, device=dev)
+        st4 = torch.cuda.current_stream().cuda_stream
+
+        def dq_launch(i):
+            _abi.check(_abi.lib().cch_dyn_quant_i8_rows(xs4[i % 4].data_ptr(), None, q4.data_ptr(), s4.data_ptr(), t4, t4, k4, 1, 0, st4))
+
+        for i in range(8):
+            dq_launch(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(60):
+            dq_launch(i)
+        e1.record()
+        torch.cuda.synchronize()
+        dq_us = e0.elapsed_time(e1) * 1e3 / 60
+        dq_bytes = t4 * k4 * 3 + t4 * 4
+        extra["dyn_quant_i8_cfg4_tokens"] = {"gb_per_s": round(dq_bytes / dq_us / 1e3, 1), "frac_of_hbm_peak": round(dq_bytes / dq_us / 1e3 / HBM_PEAK_GBS, 4),
+                                             "us": round(dq_us, 2), "bytes": dq_bytes}
+        del xs4, q4
         # config 5: MXFP4 grouped (same groups as the headline)
         a5, sa5 = cc.mx_quant((torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16), "e2m1")
         b5 = torch.empty((E, K, N // 2), dtype=torch.uint8, device=dev)

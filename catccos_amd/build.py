@@ -29,6 +29,8 @@ HIP_FLAGS = [
     # packed fp32 VALU forms are kept out of all device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
+    # the direct-to-LDS loads are inline assembly that writes M0 and names it as clobbered
+    "-Wno-inline-asm",
 ]
 
 

@@ -1,0 +1,183 @@
+// Per-token dynamic int8 quantiser with row gather: the step that turns bf16 tokens into the
+// int8 rows and per-token scales the MoE grouped GEMM consumes.  Streaming, HBM-bound: one wave
+// owns one output row, keeps it in registers (16-byte non-temporal loads, up to 8192 columns),
+// reduces |x| across the wave, and writes 8 int8 per lane per chunk.  Longer rows are read twice.
+//
+// Follows MoeV2GatherDynamicQuant::Compute
+// (examples/aux_ops/moe_init_routing_quant_v2/moe_v2_gather_dynamic_quant.h:117-150) and its
+// gather loop (:229-236); CCH_DQ_GOLDEN follows the generator's golden
+// (examples/utils/gen_data_dispatch_gmm_dequant_swiglu.py:275-280).  The smoothing vector of the
+// reference kernel is not part of this entry point.
+#include "common.h"
+#include "mx_formats.h"
+
+namespace cch {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int DQ_THREADS = 256;   // 4 rows per workgroup
+constexpr int DQ_MAX_CHUNKS = 16; // 16 x 512 columns held in registers
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, off, 64));
+    return v;
+}
+
+// Correctly rounded a / b for a divisor shared by a whole row.  With y = RN(1/b), q0 = RN(a*y)
+// and the exact remainder r = a - b*q0 (one FMA), RN(q0 + r*y) is the correctly rounded quotient
+// (Markstein) provided b's significand is not all ones and nothing leaves the normal range; the
+// caller falls back to the division instruction sequence otherwise (`fast` false).
+struct RowDivisor {
+    float b, y;
+    bool fast;
+};
+__device__ __forceinline__ RowDivisor make_divisor(float b)
+{
+    RowDivisor d;
+    d.b = b;
+    d.y = 1.0f / b;
+    const uint32_t bits = __float_as_uint(b);
+    const int e = (int)((bits >> 23) & 0xFF);
+    d.fast = e > 40 && e < 215 && (bits & 0x7FFFFFu) != 0x7FFFFFu;
+    return d;
+}
+__device__ __forceinline__ float row_div(float a, const RowDivisor &d)
+{
+    if (!d.fast) return a / d.b;   // wave-uniform
+    const float q0 = a * d.y;
+    const float r = __builtin_fmaf(-d.b, q0, a);
+    return __builtin_fmaf(r, d.y, q0);
+}
+
+// One value: MODE 0 = fp32 divide by the scale, truncate to half, round halves away from zero;
+// MODE 1 = rint(x * 127 / amax).  `d` divides by the scale (MODE 0) or by amax (MODE 1).
+template <int MODE>
+__device__ __forceinline__ int quant_one(float v, const RowDivisor &d)
+{
+    float y;
+    if (MODE == 0) {
+        float t = row_div(v, d);
+        // |t| <= 127.000008: a half in that range keeps 10 fraction bits of the fp32 pattern; values
+        // below the half normal range end up as 0 either way
+        t = __uint_as_float(__float_as_uint(t) & 0xFFFFE000u);
+        y = truncf(t + copysignf(0.5f, t));
+    } else {
+        y = rintf(row_div(v * 127.0f, d));
+    }
+    return (int)y;   // |y| <= 127: |x| <= amax, and the quotient of amax itself rounds to 127
+}
+
+template <int MODE, int CHUNKS>
+__global__ __launch_bounds__(DQ_THREADS) void dyn_quant_rows_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ src,
+                                                                   int8_t *__restrict__ q, float *__restrict__ scale, int rows_in,
+                                                                   int T, int K, int topk)
+{
+    const int lane = threadIdx.x & 63;
+    const int row = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (DQ_THREADS / 64) + (threadIdx.x >> 6)));
+    if (row >= T) return;
+    int r = row;
+    if (src) {
+        const int s = src[row];
+        r = s < 0 ? -1 : s / topk;
+    }
+    int8_t *qo = q + (size_t)row * K;
+    const bool live = r >= 0 && r < rows_in;   // wave-uniform
+    const uint16_t *xr = x + (size_t)(live ? r : 0) * K;
+    const bool vec = (K % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(q)) % 16 == 0);
+
+    if (CHUNKS > 0 && vec) {
+        // register path
+        uint32_t w[CHUNKS > 0 ? CHUNKS : 1][4];
+        uint32_t m = 0;
+#pragma unroll
+        for (int c = 0; c < CHUNKS; c++) {
+            const int k0 = (c * 64 + lane) * 8;
+            w[c][0] = w[c][1] = w[c][2] = w[c][3] = 0;
+            if (live && k0 < K) {
+                const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xr + k0));
+                w[c][0] = v[0]; w[c][1] = v[1]; w[c][2] = v[2]; w[c][3] = v[3];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const u16x2 a = __builtin_bit_cast(u16x2, w[c][i] & 0x7FFF7FFFu);
+                m = max(m, max((uint32_t)a[0], (uint32_t)a[1]));
+            }
+        }
+        m = wave_max_u32(m);   // the largest |bf16| pattern is the largest magnitude
+        const float amax = __uint_as_float(m << 16);
+        const bool zero = !(amax > 0.0f);
+        const float sc = zero ? 0.0f : amax / 127.0f;
+        if (lane == 0) scale[row] = sc;
+        const RowDivisor dv = make_divisor(zero ? 1.0f : (MODE == 0 ? sc : amax));
+#pragma unroll
+        for (int c = 0; c < CHUNKS; c++) {
+            const int k0 = (c * 64 + lane) * 8;
+            if (k0 >= K) continue;
+            uint32_t o[2] = {0, 0};
+            if (!zero) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int q0 = quant_one<MODE>(__uint_as_float(w[c][i] << 16), dv);
+                    const int q1 = quant_one<MODE>(__uint_as_float(w[c][i] & 0xFFFF0000u), dv);
+                    o[i >> 1] |= ((uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8)) << (16 * (i & 1));
+                }
+            }
+            __builtin_nontemporal_store((u32x2){o[0], o[1]}, reinterpret_cast<u32x2 *>(qo + k0));
+        }
+    } else {
+        // two passes over the row, any K and alignment
+        uint32_t m = 0;
+        if (live)
+            for (int k = lane; k < K; k += 64) m = max(m, (uint32_t)(xr[k] & 0x7FFFu));
+        m = wave_max_u32(m);
+        const float amax = __uint_as_float(m << 16);
+        const bool zero = !(amax > 0.0f);
+        const float sc = zero ? 0.0f : amax / 127.0f;
+        if (lane == 0) scale[row] = sc;
+        const RowDivisor dv = make_divisor(zero ? 1.0f : (MODE == 0 ? sc : amax));
+        for (int k = lane; k < K; k += 64)
+            qo[k] = zero ? (int8_t)0 : (int8_t)quant_one<MODE>(__uint_as_float((uint32_t)xr[k] << 16), dv);
+    }
+}
+
+template <int MODE>
+static int launch_dq(const void *x, const int32_t *src, void *q, float *scale, int64_t rows_in, int64_t t, int64_t k, int topk,
+                     hipStream_t stream)
+{
+    const unsigned grid = (unsigned)((t + DQ_THREADS / 64 - 1) / (DQ_THREADS / 64));
+    const int chunks = (int)((k + 511) / 512);
+#define CCH_DQ_LAUNCH(C)                                                                                                   \
+    hipLaunchKernelGGL((dyn_quant_rows_kernel<MODE, C>), dim3(grid), dim3(DQ_THREADS), 0, stream,                          \
+                       static_cast<const uint16_t *>(x), src, static_cast<int8_t *>(q), scale, (int)rows_in, (int)t, (int)k, topk)
+    if (chunks <= 4) CCH_DQ_LAUNCH(4);
+    else if (chunks <= 8) CCH_DQ_LAUNCH(8);
+    else if (chunks <= DQ_MAX_CHUNKS) CCH_DQ_LAUNCH(DQ_MAX_CHUNKS);
+    else CCH_DQ_LAUNCH(0);
+#undef CCH_DQ_LAUNCH
+    return launch_status("dyn_quant_rows_kernel");
+}
+
+}  // namespace cch
+
+extern "C" int cch_dyn_quant_i8_rows(const void *x, const int32_t *src_rows, void *q, float *scale, int64_t rows_in, int64_t t,
+                                     int64_t k, int topk, int mode, void *stream)
+{
+    using namespace cch;
+    CCH_REQUIRE(rows_in >= 0 && t >= 0 && k >= 0, "cch_dyn_quant_i8_rows: negative shape");
+    CCH_REQUIRE(rows_in < ((int64_t)1 << 31) && t < ((int64_t)1 << 31) && k < ((int64_t)1 << 31), "cch_dyn_quant_i8_rows: shape too large");
+    CCH_REQUIRE(topk >= 1, "cch_dyn_quant_i8_rows: topk %d", topk);
+    CCH_REQUIRE(mode == CCH_DQ_DEVICE || mode == CCH_DQ_GOLDEN, "cch_dyn_quant_i8_rows: mode %d", mode);
+    if (t == 0) return CCH_OK;
+    CCH_REQUIRE(q != nullptr || k == 0, "cch_dyn_quant_i8_rows: null output");
+    CCH_REQUIRE(scale != nullptr, "cch_dyn_quant_i8_rows: null scale");
+    CCH_REQUIRE(x != nullptr || rows_in == 0 || k == 0, "cch_dyn_quant_i8_rows: null input");
+    CCH_REQUIRE(src_rows != nullptr || t <= rows_in, "cch_dyn_quant_i8_rows: %lld output rows from %lld input rows without a row map",
+                (long long)t, (long long)rows_in);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return mode == CCH_DQ_DEVICE ? launch_dq<0>(x, src_rows, q, scale, rows_in, t, k, topk, s)
+                                 : launch_dq<1>(x, src_rows, q, scale, rows_in, t, k, topk, s);
+}

@@ -200,7 +200,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     constexpr int CPR = ROWB / 16;                 // 16-byte chunks per staged row
     constexpr int PASS_ROWS = 64 / CPR;            // rows staged per pass: 1 KiB, one read-back instruction
     constexpr int NPASS = 32 / PASS_ROWS;          // passes per 32-row MFMA tile
-    constexpr int NP = EPI != EPI_PLAIN ? 2 : 0;   // extra requests in a tile's first batch (epilogue parameters)
 
     __shared__ GroupTable tab;
     if (threadIdx.x == 0) build_group_table(tab, p.group_sizes, p.num_groups, p.T, BM);

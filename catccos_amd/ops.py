@@ -84,6 +84,35 @@ def mx_quant_b(b, fmt="e4m3", rounding=ROUND_RNE, trans_b=0):
     return payload, scales
 
 
+DQ_DEVICE, DQ_GOLDEN = 0, 1
+
+
+def dynamic_quant_i8(x, src_rows=None, topk=1, mode=DQ_DEVICE):
+    """Per-token dynamic int8 quantisation of a 2-D bf16 tensor, optionally gathering rows.
+
+    Output row i quantises x[src_rows[i] // topk] (x[i] without a row map).  Returns
+    (q int8 [T, K], scale float32 [T]) with scale = amax(row) / 127.
+    """
+    _require_gpu(x)
+    if x.dim() != 2 or x.dtype != torch.bfloat16:
+        raise ValueError("dynamic_quant_i8 expects a 2-D bfloat16 tensor")
+    x = x.contiguous()
+    rows_in, k = x.shape
+    if src_rows is not None:
+        if src_rows.dim() != 1 or src_rows.dtype != torch.int32:
+            raise ValueError("src_rows must be a 1-D int32 tensor")
+        _require_gpu(src_rows)
+        src_rows = src_rows.contiguous()
+        t = src_rows.shape[0]
+    else:
+        t = rows_in
+    q = torch.empty((t, k), dtype=torch.int8, device=x.device)
+    scale = torch.empty((t,), dtype=torch.float32, device=x.device)
+    check(_abi.lib().cch_dyn_quant_i8_rows(_ptr(x), _ptr(src_rows) if src_rows is not None else None, _ptr(q), _ptr(scale),
+                                           rows_in, t, k, int(topk), int(mode), _stream()))
+    return q, scale
+
+
 def set_option(name, value):
     """Library switch (see cch_set_option in include/catccos_hip.h)."""
     check(_abi.lib().cch_set_option(name.encode(), int(value)))

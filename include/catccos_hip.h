@@ -127,6 +127,24 @@ int cch_mx_gemm(const void *a, const void *sa, const void *b, const void *sb, vo
 int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes, void *out,
                int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, void *stream);
 
+/* ---- Per-token dynamic int8 quantisation with row gather (feeds config 4) ----
+ * Replaces MoeV2GatherDynamicQuant (examples/aux_ops/moe_init_routing_quant_v2/
+ * moe_v2_gather_dynamic_quant.h:117-150 Compute, :213-250 the gather loop), without its
+ * smoothing vector.
+ *   x         bf16 [rows_in, k] row-major
+ *   src_rows  int32 [t] or NULL: output row i quantises input row src_rows[i] / topk
+ *             (the reference's sorted expanded-row index divided by top-K); a negative
+ *             entry or one past the input gives a zero row with scale 0.  NULL: row i.
+ *   q         int8 [t, k];  scale  fp32 [t] = amax(row) / 127 (0 for an all-zero row)
+ *   mode      CCH_DQ_DEVICE: y = x / scale in fp32, truncated to half, rounded to the nearest
+ *             integer with halves away from zero (the reference kernel's casts);
+ *             CCH_DQ_GOLDEN: rint(x * 127 / amax), ties to even (the reference's Python
+ *             golden, examples/utils/gen_data_dispatch_gmm_dequant_swiglu.py:275-280). */
+#define CCH_DQ_DEVICE 0
+#define CCH_DQ_GOLDEN 1
+int cch_dyn_quant_i8_rows(const void *x, const int32_t *src_rows, void *q, float *scale, int64_t rows_in, int64_t t,
+                          int64_t k, int topk, int mode, void *stream);
+
 /* Library switches for tests and benchmarks: "force_generic_gemm" = 1 routes every GEMM entry
  * point through the shape-agnostic one-thread-per-element kernels instead of the tiled MFMA
  * kernels; "require_tiled_gemm" = 1 makes a GEMM entry point return CCH_ENOSUP instead of

@@ -49,6 +49,8 @@ def lib():
         L.orc_decode.argtypes = [c.c_uint8, c.c_int]
         L.orc_round_through_f16.restype = c.c_float
         L.orc_round_through_f16.argtypes = [c.c_float]
+        L.orc_trunc_through_f16.restype = c.c_float
+        L.orc_trunc_through_f16.argtypes = [c.c_float]
         L.orc_shared_exp.restype = c.c_int
         L.orc_shared_exp.argtypes = [c.c_float, c.c_int, c.POINTER(c.c_int)]
         L.orc_sched_src_prev_sum.restype = c.c_int32
@@ -162,6 +164,25 @@ def mx_dequant_rows(payload, scales, k, fmt=E4M3):
 
 
 # -------------------------------------------------------------------- GEMMs
+
+DQ_DEVICE, DQ_GOLDEN = 0, 1
+
+
+def dyn_quant_i8_rows(x_bf16, src=None, topk=1, mode=DQ_DEVICE):
+    """Per-token dynamic int8 quantisation: x uint16 [rows_in,K] -> (q int8 [T,K], scale float32 [T])."""
+    x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
+    rows_in, k = x.shape
+    if src is not None:
+        src = np.ascontiguousarray(src, dtype=np.int32)
+        t = src.shape[0]
+    else:
+        t = rows_in
+    q = np.empty((t, k), dtype=np.int8)
+    scale = np.empty(t, dtype=np.float32)
+    lib().orc_dyn_quant_i8_rows(_p(x), _p(src) if src is not None else None, _i64(rows_in), _i64(t), _i64(k), int(topk),
+                                int(mode), _p(q), _p(scale))
+    return q, scale
+
 
 def gemm_i8_dequant(a, b, per_tok, per_ch, trans_b=0, rows=None, want_bf16=False):
     a = np.ascontiguousarray(a, dtype=np.int8)

@@ -404,6 +404,85 @@ float orc_round_through_f16(float v)
 }
 static float f32_to_f16_to_f32(float v) { return orc_round_through_f16(v); }
 
+/* Truncate an fp32 value toward zero to IEEE half precision and widen it back
+ * (the reference's Cast(..., RoundMode::CAST_TRUNC) to half).  Finite inputs
+ * below the half range only.  pinned by: brute force over all 65536 half bit
+ * patterns (largest |half| not above |v|). */
+float orc_trunc_through_f16(float v)
+{
+    if (v != v) return v;
+    float a = fabsf(v);
+    if (a >= 65504.0f) a = 65504.0f;
+    int e;
+    (void)frexpf(a, &e);                      /* a = f * 2^e, f in [0.5,1) */
+    int q = (e - 1 < -14 ? -14 : e - 1) - 10; /* spacing of halves near a is 2^q */
+    float r = ldexpf(floorf(ldexpf(a, -q)), q);
+    return v < 0 ? -r : r;
+}
+
+/*
+ * Per-token dynamic int8 quantisation with an optional row gather, the step
+ * that feeds the MoE int8 grouped GEMM
+ * (examples/aux_ops/moe_init_routing_quant_v2/moe_v2_gather_dynamic_quant.h).
+ *   x        bf16 [rows_in, K]
+ *   src      int32 [T] or NULL: output row i quantises input row src[i] / topk
+ *            (:229-236, srcIdx / k); a negative entry or one past the input
+ *            gives a zero row with scale 0 (the reference skips such rows,
+ *            :198-201).  NULL: row i.
+ *   mode 0   the device kernel's arithmetic (:132-150): scale = amax / 127
+ *            (fp32), y = x / scale (fp32), y truncated to half, then rounded
+ *            to the nearest integer with halves away from zero
+ *   mode 1   the generator's golden (gen_data_dispatch_gmm_dequant_swiglu.py
+ *            :275-280): q = rint(x * 127 / amax) in fp32 (ties to even),
+ *            scale = amax / 127
+ *   An all-zero row gives q = 0 and scale 0 in both modes (the reference
+ *   divides 0 by 0 there).
+ * pinned by: mode 1 against torch (abs/max/round on the same data); mode 0
+ *            against a numpy restatement built on the brute-force half
+ *            truncation; |q| <= 127 with 127 reached in every non-zero row;
+ *            |x - q*scale| <= scale (mode 0) and <= scale/2 (mode 1).
+ */
+void orc_dyn_quant_i8_rows(const uint16_t *x, const int32_t *src, int64_t rows_in, int64_t T, int64_t K, int topk,
+                           int mode, int8_t *q, float *scale)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < T; i++) {
+        int64_t r = src ? (src[i] < 0 ? -1 : (int64_t)src[i] / topk) : i;
+        int8_t *qo = q + i * K;
+        if (r < 0 || r >= rows_in) {
+            memset(qo, 0, (size_t)K);
+            scale[i] = 0.0f;
+            continue;
+        }
+        const uint16_t *xr = x + r * K;
+        float amax = 0.0f;
+        for (int64_t k = 0; k < K; k++) {
+            float a = fabsf(orc_bf16_to_f32(xr[k]));
+            if (a > amax) amax = a;
+        }
+        if (!(amax > 0.0f)) {
+            memset(qo, 0, (size_t)K);
+            scale[i] = 0.0f;
+            continue;
+        }
+        const float sc = amax / 127.0f;
+        scale[i] = sc;
+        for (int64_t k = 0; k < K; k++) {
+            const float v = orc_bf16_to_f32(xr[k]);
+            float y;
+            if (mode == 0) {
+                const float t = orc_trunc_through_f16(v / sc);
+                y = truncf(t + (t < 0 ? -0.5f : 0.5f));   /* exact: t has at most 11 significant bits */
+            } else {
+                y = rintf(v * 127.0f / amax);
+            }
+            if (y > 127.0f) y = 127.0f;
+            if (y < -128.0f) y = -128.0f;
+            qo[k] = (int8_t)y;
+        }
+    }
+}
+
 /*
  * Grouped int8 GEMM + per-channel dequant + per-token dequant + SwiGLU
  * (gen_data_dispatch_gmm_dequant_swiglu.py:298-320, swiglu :269-273).
