@@ -44,6 +44,8 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int BM = 256, BN = 256;        // output tile
 constexpr int BKB = 128;                 // bytes of K per step (per row) = one L2 line
@@ -601,17 +603,20 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                                     if (SWIGLU) {
                                         const float gate = (float)acc[i][0][x + d] * chs[0] * tok[xr + d];
                                         const float up = (float)acc[i][1][x + d] * chs[1] * tok[xr + d];
-                                        v[d] = gate * (1.0f / (1.0f + expf(-gate))) * up;
+                                        // hardware exp2 and reciprocal: relative error ~1e-6, far inside the bf16 result
+                                        v[d] = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;
                                     } else if (EPI == EPI_DEQUANT) {
                                         v[d] = (float)acc[i][j][x + d] * tok[xr + d] * chs[j];
                                     } else {
                                         v[d] = (float)acc[i][j][x + d];
                                     }
                                 }
-                                const uint32_t keep = f32_to_bf16_bits(odd ? v[1] : v[0]);
-                                const uint32_t send = f32_to_bf16_bits(odd ? v[0] : v[1]);
-                                const uint32_t recv = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, 0xB1, 0xF, 0xF, true);
-                                const uint32_t packed = odd ? (recv | (keep << 16)) : (keep | (recv << 16));
+                                // hardware RNE to bf16, both rows in one dword; then the neighbour's dword
+                                // and one byte permute: even lanes keep the low halves (row x), odd lanes
+                                // the high halves (row x+1), own column in its place
+                                const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){v[0], v[1]}, bf16x2));
+                                const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, true);
+                                const uint32_t packed = __builtin_amdgcn_perm(nb, pk, odd ? 0x03020706u : 0x05040100u);
                                 const int lrow = qq * 8 + g * 4 + xr + (odd ? 1 : 0);
                                 const int lcol = j * 32 + (r & ~1);
                                 *reinterpret_cast<uint32_t *>(smem + epi + (uint32_t)(lrow * ROWB + lcol * 2)) = packed;
