@@ -223,9 +223,10 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     const uint32_t swz = swizzle_of_row(r);
     const uint32_t rd_a = (uint32_t)(wm * WM + r) * BKB, rd_b = (uint32_t)PANEL_BYTES + (uint32_t)(wn * WN + r) * BKB;
     const uint32_t rd_sa = (uint32_t)(wm * WM + r) * 16;
-    // B scales: TB = 1 like A's, 16 bytes per column; TB = 0 two 512-byte rows per step,
-    // [K64 block][column][2], in the buffer of the step's parity
-    const uint32_t rd_sb = TB ? 4096u + (uint32_t)(wn * WN + r) * 16 : 4096u + (uint32_t)(wn * WN + r) * 2;
+    // B scales: TB = 1 like A's, 16 bytes per column; TB = 0 eight 512-byte rows per group,
+    // [K64 block][column][2]
+    const uint32_t rd_sb = TB ? 4096u + (uint32_t)(wn * WN + r) * 16 : 4096u + (((uint32_t)(wn * WN + r) * 2) & ~3u);
+    const uint32_t sb_sel = (r & 1) ? 0x07060302u : 0x05040100u;   // TB = 0: which half of the dwords holds this column
     // TB = 0 fragment reads: lane (q = lane / 16, i = lane % 16) addresses K-row 16*(q/2) + i/2 of
     // the substep part and the 8-byte half (i & 1) of 16-byte chunk wn*4 + j*2 + (q & 1), whose
     // position in the row is swizzled by the row's low bits (i / 2)
@@ -300,8 +301,8 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride, (uint32_t)min((int64_t)p.N * p.sld, (int64_t)c.lim));
                 c.off_sc = (uint32_t)min(c.j0 + idx, p.N - 1) * (uint32_t)p.sld;
             } else {
-                // [K/64][N][2]: wave 4 fetches, per step, two 512-byte rows (the step's two
-                // K64 blocks, 256 columns); lane l takes 16 bytes of row l/32
+                // [K/64][N][2]: a scale group is 8 rows of K64 blocks (4 MXFP8 steps, 2 MXFP4 steps)
+                // x 256 columns x 2 bytes; wave 4+i fetches rows 2i, 2i+1, lane l 16 bytes of row l/32
                 c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride, (uint32_t)min((int64_t)p.N * p.sld, (int64_t)c.lim));
                 c.off_sc = (uint32_t)((lane >> 5) + 2 * (wave - 4)) * (uint32_t)p.N * 2u + (uint32_t)c.j0 * 2u + (uint32_t)(lane & 31) * 16u;
             }
@@ -321,22 +322,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                           lds + PANEL_BYTES + (piece - NJ) * 1024u);
         }
     };
-    // Scale group `grp` of tile c (16 bytes per row: steps grp*SPG .. grp*SPG+SPG-1) into scale
-    // buffer `buf`; waves 0-3 fetch the A rows, waves 4-7 the B rows, one row per lane.
-    // With TB = 0 only waves 0-3 take part (the others issue the instruction with an empty EXEC
-    // mask, which keeps the code free of branches); the B scales then come per step, see below.
+    // Scale group `grp` of tile c (steps grp*SPG .. grp*SPG+SPG-1) into scale buffer `buf`: waves
+    // 0-3 fetch 16 bytes of each A row, one row per lane; waves 4-7 the same for the B rows
+    // (TB = 1) or 1 KiB each of the group's eight [column][2] rows (TB = 0).
     auto issue_scales = [&](int newgrp, const TileCtx &c, int grp, int buf) {
         if constexpr (MX)
-            load16_to_lds_if(newgrp & (int)(TB || wave < 4), c.rs_sc, c.off_sc, (uint32_t)grp * 16u,
+            load16_to_lds_if(newgrp, c.rs_sc, c.off_sc, (TB || wave < 4) ? (uint32_t)grp * 16u : (uint32_t)grp * 16u * (uint32_t)p.N,
                              lds_base + (uint32_t)(SCALE_OFF + buf * SCALE_BUF) + (uint32_t)(wave >= 4) * 4096u + (uint32_t)(wave & 3) * 1024u);
-    };
-    // TB = 0: B scales of K-step kt, stored [K/64][N][2]: one 512-byte row per K64 block of the
-    // step (2 for MXFP8, 4 for MXFP4) x 256 columns, two rows per wave starting at wave 4, into
-    // the B half of the scale buffer of the step's ring stage.
-    auto issue_bscale = [&](const TileCtx &c, int kt, int stage) {
-        if constexpr (MX && !TB)
-            load16_to_lds_if(wave >= 4 && wave < 4 + SCALE_DW, c.rs_sc, c.off_sc, (uint32_t)kt * (4u * SCALE_DW) * (uint32_t)p.N,
-                             lds_base + (uint32_t)(SCALE_OFF + stage * SCALE_BUF) + 4096u + (uint32_t)(wave & 3) * 1024u);
     };
     auto issue_step = [&](const TileCtx &c, int kt, int stage) {
         static_for<NV>([&](auto piece_c) { issue_piece(c, kt, stage, piece_c); });
@@ -357,7 +349,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         }
         issue_scales(1, c, 0, gi & 1);
         gi++;
-        issue_bscale(c, 0, stage);
         issue_step(c, 0, stage);
     };
 
@@ -369,7 +360,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     nxt.valid = 0;
     if (cur.valid) {
         setup(cur, 0, 0);
-        issue_bscale(cur, 1, 1);
         issue_step(cur, 1, 1);
     }
     while (cur.valid) {
@@ -421,7 +411,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             }
         };
         // Scale dwords of K-step kt of the current tile
-        auto read_scales = [&](int kt, int kt_stage, uint32_t (&dst)[NSC][MT + NT]) {
+        auto read_scales = [&](int kt, uint32_t (&dst)[NSC][MT + NT]) {
             if (!MX) return;
             const uint32_t ss = (uint32_t)(SCALE_OFF + ((gbase + kt / SPG) & 1) * SCALE_BUF) + (uint32_t)(kt % SPG) * (SCALE_DW * 4u);
 #pragma unroll
@@ -433,10 +423,12 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                     if constexpr (TB) {
                         dst[d][MT + s] = lds_read4(ss + rd_sb + s * 512 + d * 4);
                     } else {
-                        // bytes 2*ks + g of the step's dword: the two blocks of K64 block ks sit side by side
-                        const uint32_t sb0 = (uint32_t)(SCALE_OFF + kt_stage * SCALE_BUF) + rd_sb + s * 64 + d * 1024;
-                        dst[d][MT + s] = (uint32_t)*reinterpret_cast<const uint16_t *>(smem + sb0) |
-                                         ((uint32_t)*reinterpret_cast<const uint16_t *>(smem + sb0 + 512) << 16);
+                        // The two K32 scales of K64 row 2x and of row 2x+1, for this column: bytes
+                        // 2*ks + g of the step's dword as in the TB = 1 layout.  Each row holds two
+                        // columns per dword; the permute keeps this column's half of both.
+                        const uint32_t sb0 = (uint32_t)(SCALE_OFF + ((gbase + kt / SPG) & 1) * SCALE_BUF) + rd_sb + s * 64 +
+                                             (uint32_t)((kt % SPG) * (2 * SCALE_DW) + d * 2) * 512u;
+                        dst[d][MT + s] = __builtin_amdgcn_perm(lds_read4(sb0 + 512), lds_read4(sb0), sb_sel);
                     }
                 }
             }
@@ -513,7 +505,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                         nbase = gi;
                         setup(nxt, parity ^ 1, stage);
                     } else if constexpr (MODE == 2) {
-                        issue_bscale(nxt, 1, stage);
                         issue_step(nxt, 1, stage);
                     }
                 } else if constexpr (MODE == 0) {
@@ -522,7 +513,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                         if constexpr (piece < NV) issue_piece(cur, kt + 2, stage, IC<piece>{});
                         else if constexpr (piece == NV && MX) {
                             issue_scales(newgrp, cur, (kt + 2) / SPG, gi & 1);
-                            issue_bscale(cur, kt + 2, stage);
                         }
                     });
                 }
@@ -530,7 +520,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 __builtin_amdgcn_sched_barrier(0);
             });
             if constexpr (MODE == 0) gi += MX ? newgrp : 0;
-            if constexpr (MODE != 2) read_scales(kt + 1, nstage, sc);
+            if constexpr (MODE != 2) read_scales(kt + 1, sc);
             if constexpr (MODE != 0) {
                 // Pin the accumulators here: otherwise the compiler sinks the MFMAs of the
                 // peeled steps into the epilogue and spills their fragments to get them there.
@@ -544,13 +534,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // Tile prologue.  In flight, oldest first: this tile's set-up and first step, its
         // second step (NV requests), then the previous tile's epilogue stores.
         constexpr int NSTORES = MT * NPASS;
-        constexpr int NSTEP1 = NV + (MX && !TB ? 1 : 0);  // requests of the tile's second step
+        constexpr int NSTEP1 = NV;  // requests of the tile's second step
         if (first) CCH_WAIT_VM_LGKM0(NSTEP1);
         else CCH_WAIT_VM_LGKM0(NSTEP1 + NSTORES);
         __syncthreads();
         {
             const int stage = gstep & 1;
-            read_scales(0, stage, sc);
+            read_scales(0, sc);
 #pragma unroll
             for (int j = 0; j < NT; j++) fb0[j] = frag_b(stage, 0, j);
 #pragma unroll
