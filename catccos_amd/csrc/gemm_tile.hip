@@ -244,6 +244,16 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                                 : (uint32_t)PANEL_BYTES + (uint32_t)(16 * (tq >> 1) + (ti >> 1)) * 256u +
                                       ((uint32_t)((wn * 4 + (tq & 1)) ^ (ti >> 1)) << 4) + (uint32_t)(ti & 1) * 8u;
     const int ldb = TB ? lda : p.N / EPB;   // bytes between consecutive rows of B as stored
+    // Rows that belong to no group are written as zeros (the reference's golden pads them,
+    // examples/utils/gen_data_fp4_mx_alltoallv_gmm.py:788-790): all workgroups share the range,
+    // 16 bytes per thread and pass; usually it is empty.
+    if (p.group_sizes) {
+        const size_t begin = (size_t)uniform(tab.row_start[p.num_groups]) * p.n_out / 8, end = (size_t)p.T * p.n_out / 8;
+        v4u *o16 = reinterpret_cast<v4u *>(p.out);
+        for (size_t i = begin + (size_t)blockIdx.x * TILE_THREADS + threadIdx.x; i < end; i += (size_t)gridDim.x * TILE_THREADS)
+            o16[i] = (v4u){0, 0, 0, 0};
+    }
+
     int gi = 0;           // scale groups requested so far; group n lives in scale buffer n & 1
     int gbase = 0;        // value of gi when the current tile's group 0 was requested
 
@@ -630,17 +640,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     }
 }
 
-// Rows that belong to no group are written as zeros (the reference's golden pads them,
-// examples/utils/gen_data_fp4_mx_alltoallv_gmm.py:788-790).
-__global__ __launch_bounds__(256) void zero_tail_rows_kernel(uint16_t *out, const int32_t *group_sizes, int num_groups, int T,
-                                                             int n_out)
-{
-    int used = 0;
-    for (int gidx = 0; gidx < num_groups; gidx++) used += max(0, min(group_sizes[gidx], T - used));
-    const size_t begin = (size_t)used * n_out, end = (size_t)T * n_out;
-    for (size_t i = begin + (size_t)blockIdx.x * 256 + threadIdx.x; i < end; i += (size_t)gridDim.x * 256) out[i] = 0;
-}
-
 template <int KIND, int EPI, int FMT, int TB>
 static int launch_tile_t(const GemmProblem &p, hipStream_t stream)
 {
@@ -658,10 +657,7 @@ static int launch_tile_t(const GemmProblem &p, hipStream_t stream)
     const int64_t tiles = row_tiles * ((p.n_out + bn_out - 1) / bn_out);
     const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>(tiles, cus));
     hipLaunchKernelGGL(kern, dim3(grid), dim3(TILE_THREADS), LDS_BYTES, stream, p);
-    int rc = launch_status("gemm_tile_kernel");
-    if (rc || !p.group_sizes) return rc;
-    hipLaunchKernelGGL(zero_tail_rows_kernel, dim3(64), dim3(256), 0, stream, p.out, p.group_sizes, p.num_groups, p.T, p.n_out);
-    return launch_status("zero_tail_rows_kernel");
+    return launch_status("gemm_tile_kernel");
 }
 
 // True when the tiled kernels take this problem; otherwise the caller uses the generic path.
