@@ -59,15 +59,17 @@ constexpr int WM = 128, WN = 64;         // wave tile
 constexpr int MT = WM / 32, NT = WN / 32;  // 32x32 MFMA tiles per wave
 constexpr int NJ = PANEL_BYTES / 1024 / NWAVES;  // direct-to-LDS instructions per wave per panel (4)
 
-// dynamic LDS map
-constexpr int RING_OFF = 0;
-constexpr int SCALE_OFF = RING_OFF + NSTAGE * STAGE_BYTES;   // two buffers of (256 A + 256 B rows) x 16 scale bytes
+// dynamic LDS map.  The small areas come first so that every read of them is one base register
+// plus a 16-bit instruction offset; behind the 128 KiB ring each distinct offset would need an
+// address register of its own.
+constexpr int SCALE_OFF = 0;                                 // two buffers of (256 A + 256 B rows) x 16 scale bytes
 constexpr int SCALE_BUF = 8192;
 constexpr int EPI_OFF = SCALE_OFF + 2 * SCALE_BUF;           // per wave: 1 KiB of output staging
 constexpr int EPI_WAVE = 1024;
 constexpr int PARAM_OFF = EPI_OFF + NWAVES * EPI_WAVE;       // per tile parity: 256 per_tok + 256 per_ch floats
 constexpr int PARAM_SET = 2048;
-constexpr int LDS_BYTES = PARAM_OFF + 2 * PARAM_SET;         // 156 KiB of the CU's 160 KiB
+constexpr int RING_OFF = PARAM_OFF + 2 * PARAM_SET;          // NSTAGE stages of an A panel and a B panel
+constexpr int LDS_BYTES = RING_OFF + NSTAGE * STAGE_BYTES;   // 156 KiB of the CU's 160 KiB
 
 template <int KIND> struct KindTraits;
 template <> struct KindTraits<KIND_I8> { static constexpr int ELEMS_PER_BYTE = 1, SCALE_DW = 0; using Acc = v16i; };
@@ -479,53 +481,67 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // it, two steps ahead of its use.  Everything that follows the barrier is threaded
         // between the step's remaining MFMAs, one or two instructions at a time, so that the
         // matrix pipe keeps running while the wave issues them.
-        auto step = [&](auto mode_c, int kt) {
+        auto step = [&](auto mode_c, auto mta_c, int kt) {
             constexpr int MODE = decltype(mode_c)::value;
+            constexpr int MTA = decltype(mta_c)::value;   // row blocks of this wave that hold rows of the group
             const int stage = gstep & 1, nstage = stage ^ 1;
             static_for<MT>([&](auto i_c) {
                 constexpr int i = decltype(i_c)::value;
-                mfma_row(IC<0>{}, i_c, fa[i], fb0);
+                if constexpr (i < MTA) mfma_row(IC<0>{}, i_c, fa[i], fb0);
                 __builtin_amdgcn_sched_barrier(0);
-                fa[i] = frag_a(stage, 1, i);
-                if constexpr (i < NT) fb1[i] = frag_b(stage, 1, i);
+                if constexpr (i < MTA) fa[i] = frag_a(stage, 1, i);
+                if constexpr (i < NT && MTA > 0) fb1[i] = frag_b(stage, 1, i);
                 __builtin_amdgcn_sched_barrier(0);
             });
-            mfma_row(IC<1>{}, IC<0>{}, fa[0], fb1);
+            if constexpr (MTA > 0) mfma_row(IC<1>{}, IC<0>{}, fa[0], fb1);
             __builtin_amdgcn_sched_barrier(0);
             // Every LDS read of this step has been issued; once they have returned and the
             // requests of step kt+1 have landed, for all waves, the stage can be refilled.
             CCH_WAIT_VM_LGKM0(0);
             __syncthreads();
-            constexpr int SLOTS = (MT - 1) * MPR;           // MFMAs left in this step
-            constexpr int NREQ = NV + (MX ? 1 : 0);         // requests of a steady step
-            constexpr int PER_SLOT = (NREQ + SLOTS - 2) / (SLOTS - 1);
+            constexpr int SLOTS = MTA > 0 ? (MTA - 1) * MPR : 0;   // MFMAs left in this step
+            constexpr int NREQ = NV + (MX ? 1 : 0);                // requests of a steady step
+            constexpr int PER_SLOT = SLOTS >= 2 ? (NREQ + SLOTS - 2) / (SLOTS - 1) : NREQ;
             const int newgrp = ((kt + 2) & (SPG - 1)) == 0;
-            static_for<SLOTS>([&](auto slot_c) {
-                constexpr int slot = decltype(slot_c)::value;
-                constexpr int i = 1 + slot / MPR, m = slot % MPR;
-                mfma_one(IC<1>{}, IC<i>{}, IC<m>{}, fa[i], fb1);
-                __builtin_amdgcn_sched_barrier(0);
-                if constexpr (slot == 0) {
-                    if constexpr (MODE != 2) {
+            // what follows the first MFMA after the barrier: the next step's first fragments, and
+            // in the peeled steps the next tile's requests
+            auto after_barrier = [&]() {
+                if constexpr (MODE != 2 && MTA > 0) {
 #pragma unroll
-                        for (int j = 0; j < NT; j++) fb0[j] = frag_b(nstage, 0, j);
-                        fa[0] = frag_a(nstage, 0, 0);
-                    }
-                    if constexpr (MODE == 1) {
-                        nbase = gi;
-                        setup(nxt, parity ^ 1, stage);
-                    } else if constexpr (MODE == 2) {
-                        issue_step(nxt, 1, stage);
-                    }
-                } else if constexpr (MODE == 0) {
+                    for (int j = 0; j < NT; j++) fb0[j] = frag_b(nstage, 0, j);
+                    fa[0] = frag_a(nstage, 0, 0);
+                }
+                if constexpr (MODE == 1) {
+                    nbase = gi;
+                    setup(nxt, parity ^ 1, stage);
+                } else if constexpr (MODE == 2) {
+                    issue_step(nxt, 1, stage);
+                }
+            };
+            auto requests = [&](auto first_c) {
+                constexpr int first_piece = decltype(first_c)::value;
+                if constexpr (MODE == 0) {
                     static_for<PER_SLOT>([&](auto q_c) {
-                        constexpr int piece = (slot - 1) * PER_SLOT + decltype(q_c)::value;
+                        constexpr int piece = first_piece + decltype(q_c)::value;
                         if constexpr (piece < NV) issue_piece(cur, kt + 2, stage, IC<piece>{});
                         else if constexpr (piece == NV && MX) {
                             issue_scales(newgrp, cur, (kt + 2) / SPG, gi & 1);
                         }
                     });
                 }
+            };
+            if constexpr (SLOTS == 0) {
+                // a wave with at most one row block to compute: nothing to hide the requests behind
+                after_barrier();
+                requests(IC<0>{});
+            }
+            static_for<SLOTS>([&](auto slot_c) {
+                constexpr int slot = decltype(slot_c)::value;
+                constexpr int i = 1 + slot / MPR, m = slot % MPR;
+                mfma_one(IC<1>{}, IC<i>{}, IC<m>{}, fa[i], fb1);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (slot == 0) after_barrier();
+                else requests(IC<(slot - 1) * PER_SLOT>{});
                 if constexpr (MODE != 2 && m == MPR - 1) fa[i] = frag_a(nstage, 0, i);
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -548,18 +564,36 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         if (first) CCH_WAIT_VM_LGKM0(NSTEP1);
         else CCH_WAIT_VM_LGKM0(NSTEP1 + NSTORES);
         __syncthreads();
-        {
+        // Row blocks of this wave that hold rows of the group: the K loop is instantiated for
+        // each count, and a wave whose rows lie wholly past the end of a short group issues its
+        // requests and barriers but no matrix instruction (its SIMD then belongs to the other
+        // wave it hosts, which covers the other half of the tile's rows).
+        auto k_loop = [&](auto mta_c) {
+            constexpr int MTA = decltype(mta_c)::value;
             const int stage = gstep & 1;
-            read_scales(0, sc);
+            if constexpr (MTA > 0) {
+                read_scales(0, sc);
 #pragma unroll
-            for (int j = 0; j < NT; j++) fb0[j] = frag_b(stage, 0, j);
+                for (int j = 0; j < NT; j++) fb0[j] = frag_b(stage, 0, j);
 #pragma unroll
-            for (int i = 0; i < MT; i++) fa[i] = frag_a(stage, 0, i);
-        }
-        for (int kt = 0; kt + 2 < ksteps; kt++) step(IC<0>{}, kt);
-        decode(t + gridDim.x, nxt);
-        step(IC<1>{}, ksteps - 2);
-        step(IC<2>{}, ksteps - 1);
+                for (int i = 0; i < MTA; i++) fa[i] = frag_a(stage, 0, i);
+            }
+            // The step count is made opaque per tile: addresses that depend on it (the scale
+            // reads of the peeled steps) would otherwise be hoisted out of the tile loop and
+            // held in registers through the K loop.
+            int nk = ksteps;
+            asm volatile("" : "+s"(nk));
+            for (int kt = 0; kt + 2 < nk; kt++) step(IC<0>{}, mta_c, kt);
+            decode(t + gridDim.x, nxt);
+            step(IC<1>{}, mta_c, nk - 2);
+            step(IC<2>{}, mta_c, nk - 1);
+        };
+        const int mta = uniform(min(max((cur.m_end - cur.m0 - wm * WM + 31) >> 5, 0), MT));
+        if (mta == MT) k_loop(IC<MT>{});
+        else if (mta == 0) k_loop(IC<0>{});
+        else if (mta == 1) k_loop(IC<1>{});
+        else if (mta == 2) k_loop(IC<2>{});
+        else k_loop(IC<3>{});
         first = false;
 
         // Epilogue.  Lane (r, g) holds, for sub-tile (i, j), column r and rows
@@ -572,6 +606,11 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             const uint32_t epi = (uint32_t)(EPI_OFF + wave * EPI_WAVE);
             const uint32_t prm = (uint32_t)(PARAM_OFF + parity * PARAM_SET);
             const bool odd = lane & 1;
+            // The lane number as the store addresses see it is made opaque per tile: otherwise
+            // the sixteen per-pass row offsets are hoisted out of the tile loop and occupy
+            // registers that the K loop needs.
+            int lane_e = lane;
+            asm volatile("" : "+v"(lane_e));
             const __amdgpu_buffer_rsrc_t rs_out =
                 __builtin_amdgcn_make_buffer_rsrc(p.out + (size_t)cur.m0 * p.n_out, 0, 0x7FFFFFFF, 0x00020000);
             float chs[NT];
@@ -622,7 +661,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                                 *reinterpret_cast<uint32_t *>(smem + epi + (uint32_t)(lrow * ROWB + lcol * 2)) = packed;
                             }
                     }
-                    const int lrow = lane / CPR, chunk = lane % CPR;
+                    const int lrow = lane_e / CPR, chunk = lane_e % CPR;
                     const v4i val = lds_read16(epi + (uint32_t)(lrow * ROWB + chunk * 16));
                     const int row = wm * WM + i * 32 + ps * PASS_ROWS + lrow;  // relative to m0
                     const int col = cur.j0 + wn * WN_OUT + chunk * 8;
