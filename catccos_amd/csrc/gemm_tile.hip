@@ -271,17 +271,18 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         c.m0 = uniform(tab.row_start[c.e] + (tr - tab.tile_start[c.e]) * BM);
         c.m_end = uniform(tab.row_start[c.e + 1]);
         c.j0 = nt * BN_OUT;
-        c.rs_a = make_rsrc(p.a + (size_t)c.m0 * lda, c.lim);
+        // A's descriptor ends with the group: requests for tile rows past it are dropped by the
+        // bounds check (LDS receives zeros), and their products land in accumulators that are
+        // never stored.
+        c.rs_a = make_rsrc(p.a + (size_t)c.m0 * lda, min((uint32_t)min(c.m_end - c.m0, BM) * (uint32_t)lda, c.lim));
         c.rs_b = make_rsrc(p.b + (size_t)c.e * p.b_stride, c.lim);
         // Instruction j of this wave fills rows (wave*NJ + j)*8 .. +7 of a panel; lane l lands at
-        // row l/8, chunk position l%8 and must therefore fetch chunk (l%8) ^ swizzle(row).  Rows
-        // past the edge re-read the last valid row; their products land in accumulators that are
-        // never stored.
+        // row l/8, chunk position l%8 and must therefore fetch chunk (l%8) ^ swizzle(row).
 #pragma unroll
         for (int j = 0; j < NJ; j++) {
             const int row = (wave * NJ + j) * 8 + (lane >> 3);
             const uint32_t chunk = ((uint32_t)(lane & 7) ^ swizzle_of_row(row)) * 16u;
-            c.off_a[j] = (uint32_t)min(row, c.m_end - 1 - c.m0) * (uint32_t)lda + chunk;
+            c.off_a[j] = (uint32_t)row * (uint32_t)lda + chunk;
             if (TB) {
                 int col;  // B row (= logical column) feeding tile row `row`
                 if (SWIGLU) {
