@@ -46,12 +46,22 @@ def zipf_groups(rng, t, e):
     return gs
 
 
-def event_time_ms(fn, steps, warmup):
-    """Mean and per-launch durations of fn() on the current stream, by HIP events."""
+def event_time_ms(fn, steps, warmup, warm_ms=0.0):
+    """Mean and per-launch durations of fn() on the current stream, by HIP events.
+
+    The shader clock needs some tens of milliseconds of load to reach its steady state (launch
+    durations fall by 15-20 % over the first 50 ms after an idle period), so the untimed part must
+    be long enough: `warmup` launches, then more until `warm_ms` of wall time have passed.
+    """
     import torch
+    t0 = time.perf_counter()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    while (time.perf_counter() - t0) * 1e3 < warm_ms:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     t0 = time.perf_counter()
@@ -109,8 +119,8 @@ def quant_batch_time_us(sets, launches, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=100, help="untimed launches (about 55 ms: the clock's ramp from idle)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--only", choices=["copy", "quant"], help="profiling aid: run only a 512 MiB device copy (counter "
@@ -220,7 +230,7 @@ def main():
         # config 1: MX quantiser, rotating buffer sets larger than the 256 MB Infinity Cache
         M1, K1 = 4096, 7168
         sets = quant_inputs(dev, M1, K1, 6)
-        q_us = quant_batch_time_us(sets, 120, 12)
+        q_us = quant_batch_time_us(sets, 120, 1500)
         qbytes = M1 * K1 * 2 + M1 * K1 + M1 * K1 // 32
         q_gbs = qbytes / (q_us * 1e-6) / 1e9
         extra["mx_quant_cfg1"] = {"gb_per_s": round(q_gbs, 1), "frac_of_hbm_peak": round(q_gbs / HBM_PEAK_GBS, 4),
@@ -232,7 +242,7 @@ def main():
         b2 = torch.randint(-127, 128, (k2, n2), dtype=torch.int8, device=dev)
         pt2 = torch.rand(m2, device=dev) * 0.019 + 0.001
         pc2 = torch.rand(n2, device=dev) * 0.019 + 0.001
-        _, t2 = event_time_ms(lambda: cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, TRANS_B), 10, 3)
+        _, t2 = event_time_ms(lambda: cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, TRANS_B), 30, 3, 60.0)
         extra["w8a8_dequant_cfg2"] = {"tops": round(2.0 * m2 * n2 * k2 / (np.mean(t2) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t2)) * 1e3, 1)}
         extra["w8a8_dequant_cfg2"]["frac_of_int8_peak"] = round(extra["w8a8_dequant_cfg2"]["tops"] / FP8_PEAK_TFLOPS, 4)
         del a2, b2
@@ -240,7 +250,7 @@ def main():
         m3, k3, n3 = 4096, 2048, 7168
         a3, sa3 = cc.mx_quant(torch.randn(m3, k3, device=dev).to(torch.bfloat16), "e4m3")
         b3, sb3 = cc.mx_quant_b(torch.randn(k3, n3, device=dev).to(torch.bfloat16), "e4m3", trans_b=TRANS_B)
-        _, t3 = event_time_ms(lambda: cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", TRANS_B), 20, 5)
+        _, t3 = event_time_ms(lambda: cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", TRANS_B), 30, 5, 60.0)
         extra["mxfp8_dense_cfg3"] = {"tflops": round(2.0 * m3 * n3 * k3 / (np.mean(t3) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t3)) * 1e3, 1)}
         extra["mxfp8_dense_cfg3"]["frac_of_fp8_peak"] = round(extra["mxfp8_dense_cfg3"]["tflops"] / FP8_PEAK_TFLOPS, 4)
         # config 4: MoE W8A8 grouped + dequant + SwiGLU
@@ -250,7 +260,7 @@ def main():
         w4 = torch.randint(-127, 128, (e4, k4, n4), dtype=torch.int8, device=dev)
         pt4 = torch.rand(t4, device=dev) * 0.019 + 0.001
         pc4 = torch.rand(e4, n4, device=dev) * 0.019 + 0.001
-        _, tt4 = event_time_ms(lambda: cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), 10, 3)
+        _, tt4 = event_time_ms(lambda: cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), 30, 3, 60.0)
         extra["moe_w8a8_swiglu_cfg4"] = {"tops": round(2.0 * t4 * n4 * k4 / (np.mean(tt4) * 1e-3) / 1e12, 1), "us": round(float(np.mean(tt4)) * 1e3, 1)}
         extra["moe_w8a8_swiglu_cfg4"]["frac_of_int8_peak"] = round(extra["moe_w8a8_swiglu_cfg4"]["tops"] / FP8_PEAK_TFLOPS, 4)
         del x4, w4
@@ -264,7 +274,7 @@ def main():
         def dq_launch(i):
             _abi.check(_abi.lib().cch_dyn_quant_i8_rows(xs4[i % 4].data_ptr(), None, q4.data_ptr(), s4.data_ptr(), t4, t4, k4, 1, 0, st4))
 
-        for i in range(8):
+        for i in range(800):
             dq_launch(i)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -284,7 +294,7 @@ def main():
         sb5 = torch.empty((E, K // 64, N, 2), dtype=torch.uint8, device=dev)
         for e in range(E):
             b5[e], sb5[e] = cc.mx_quant_b((torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16), "e2m1", trans_b=TRANS_B)
-        _, t5 = event_time_ms(lambda: cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", TRANS_B), 10, 3)
+        _, t5 = event_time_ms(lambda: cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", TRANS_B), 30, 3, 60.0)
         extra["mxfp4_grouped_cfg5"] = {"tflops": round(flop / (np.mean(t5) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t5)) * 1e3, 1)}
         extra["mxfp4_grouped_cfg5"]["frac_of_fp4_peak"] = round(extra["mxfp4_grouped_cfg5"]["tflops"] / FP4_PEAK_TFLOPS, 4)
         result["extra"] = extra
