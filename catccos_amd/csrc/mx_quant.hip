@@ -132,11 +132,19 @@ __device__ __forceinline__ uint32_t block_amax_bits(const uint32_t (&w)[4])
 // PAIR (needs VEC, K % 16 == 0 and 16-byte aligned payload rows): neighbouring lanes swap halves
 // of two wave-steps so that each lane stores one 16-byte (FP8) or 8-byte (FP4) piece instead of
 // two of half that size; the store path's cost is per instruction, not per byte.
-template <int FMT, int RND, bool HWCVT, bool VEC, bool PAIR>
+// SCATTER (without PAIR): row r of x is written to rows dst_idx[r*topk + 0 .. topk-1] of the output
+// instead of row r; negative entries are skipped.  The row's destinations are read with the row
+// itself, one batch ahead of their use.  `sstride` is the distance between scale rows (equal to
+// `sld` unless payload and scales share one packed row).
+constexpr int QUANT_MAX_TOPK = 8;
+template <int FMT, int RND, bool HWCVT, bool VEC, bool PAIR, bool SCATTER = false>
 __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
     const uint16_t *__restrict__ x, uint8_t *__restrict__ payload, uint8_t *__restrict__ scales, int rows, int K,
-    int nblk, int sld, int pld, int wpr, int total_ws)
+    int nblk, int sld, int pld, int wpr, int total_ws, const int32_t *__restrict__ dst_idx = nullptr, int topk = 1,
+    int sstride = 0)
 {
+    static_assert(!(SCATTER && PAIR), "the scatter variant stores one wave-step at a time");
+    if (!SCATTER) sstride = sld;
     constexpr bool FP4 = FMT == CCH_FMT_E2M1;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (QUANT_THREADS / 64) + (threadIdx.x >> 6)));
@@ -145,6 +153,7 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
     struct Batch {
         uint32_t w[QUANT_UNROLL][4];
         int row[QUANT_UNROLL], k0[QUANT_UNROLL];
+        int dst[QUANT_UNROLL][SCATTER ? QUANT_MAX_TOPK : 1];
     };
     auto fetch = [&](int ws0, Batch &bt) {
 #pragma unroll
@@ -154,6 +163,11 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
             bt.row[u] = ws < total_ws ? r : -1;
             bt.k0[u] = ((ws - r * wpr) * 64 + lane) * 8;
             bt.w[u][0] = bt.w[u][1] = bt.w[u][2] = bt.w[u][3] = 0;
+            if constexpr (SCATTER) {
+#pragma unroll
+                for (int t = 0; t < QUANT_MAX_TOPK; t++)
+                    bt.dst[u][t] = (bt.row[u] >= 0 && t < topk) ? dst_idx[(size_t)bt.row[u] * topk + t] : -1;
+            }
             if (bt.row[u] >= 0 && bt.k0[u] < K) {
                 const uint16_t *src = x + (size_t)bt.row[u] * K + bt.k0[u];
                 if (VEC) {
@@ -214,6 +228,35 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
                         __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(dst));
                     }
                 }
+            } else if (SCATTER) {
+#pragma unroll
+                for (int t = 0; t < QUANT_MAX_TOPK; t++) {
+                    const int drow = bt.dst[u][t];
+                    if (drow < 0) continue;  // wave-uniform
+                    if (k0 < K) {
+                        uint8_t *dst = payload + (size_t)drow * pld + (FP4 ? (k0 >> 1) : k0);
+                        if (VEC) {
+                            if (FP4) {
+                                __builtin_nontemporal_store(q[0], reinterpret_cast<uint32_t *>(dst));
+                            } else {
+                                u32x2 o = {q[0], q[1]};
+                                __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(dst));
+                            }
+                        } else if (FP4) {
+                            for (int i = 0; i < 4; i++)
+                                if (k0 + 2 * i < K) dst[i] = (uint8_t)(q[0] >> (8 * i)) & (k0 + 2 * i + 1 < K ? 0xFF : 0x0F);
+                        } else {
+                            for (int i = 0; i < 8; i++)
+                                if (k0 + i < K) dst[i] = (uint8_t)(q[i >> 2] >> (8 * (i & 3)));
+                        }
+                    }
+                    if (blk < nblk) {
+                        uint8_t *srow = scales + (size_t)drow * sstride;
+                        if ((lane & 3) == 0) srow[blk] = (uint8_t)sbyte;
+                        if ((lane & 3) == 1 && blk == nblk - 1 && sld != nblk) srow[nblk] = 127;  // even padding, 1.0
+                    }
+                }
+                continue;
             } else if (k0 < K) {
                 uint8_t *dst = payload + (size_t)bt.row[u] * pld + (FP4 ? (k0 >> 1) : k0);
                 if (VEC) {
@@ -451,7 +494,74 @@ static int launch_b(const void *b, void *payload, void *scales, int64_t k, int64
     return launch_status("mx_quant_b_kernel");
 }
 
+// Quantise-once, scatter-to-top-K launch: packed output rows of `row_bytes` = payload bytes +
+// padded scale bytes.
+template <int FMT, int RND, bool HWCVT>
+static int launch_scatter(const void *x, const int32_t *dst_idx, void *packed, int64_t tokens, int64_t k, int topk,
+                          hipStream_t stream)
+{
+    const bool fp4 = FMT == CCH_FMT_E2M1;
+    const int64_t nblk = (k + 31) / 32, sld = 2 * ((nblk + 1) / 2), pbytes = fp4 ? (k + 1) / 2 : k;
+    const int64_t row_bytes = pbytes + sld;
+    const int64_t wpr = (nblk * 4 + 63) / 64;
+    const bool vec = (k % 8 == 0) && aligned(x, 16) && aligned(packed, 8) && row_bytes % 8 == 0;
+    int dev = 0, cus = 0;
+    CCH_HIP(hipGetDevice(&dev));
+    CCH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int64_t max_blocks = (int64_t)cus * QUANT_BLOCKS_PER_CU;
+    const int64_t rows_per_launch = std::max<int64_t>(1, (int64_t)(1 << 30) / wpr);
+    uint8_t *out = static_cast<uint8_t *>(packed);
+    for (int64_t r0 = 0; r0 < tokens; r0 += rows_per_launch) {
+        const int64_t rows = std::min(rows_per_launch, tokens - r0);
+        const int64_t total_ws = rows * wpr;
+        const int64_t waves = (total_ws + QUANT_UNROLL - 1) / QUANT_UNROLL;
+        const unsigned grid = (unsigned)std::min<int64_t>((waves + QUANT_THREADS / 64 - 1) / (QUANT_THREADS / 64), max_blocks);
+        const uint16_t *xs = static_cast<const uint16_t *>(x) + r0 * k;
+        const int32_t *ds = dst_idx + r0 * topk;
+        if (vec)
+            hipLaunchKernelGGL((mx_quant_rows_kernel<FMT, RND, HWCVT, true, false, true>), dim3(grid), dim3(QUANT_THREADS), 0,
+                               stream, xs, out, out + pbytes, (int)rows, (int)k, (int)nblk, (int)sld, (int)row_bytes, (int)wpr,
+                               (int)total_ws, ds, topk, (int)row_bytes);
+        else
+            hipLaunchKernelGGL((mx_quant_rows_kernel<FMT, RND, HWCVT, false, false, true>), dim3(grid), dim3(QUANT_THREADS), 0,
+                               stream, xs, out, out + pbytes, (int)rows, (int)k, (int)nblk, (int)sld, (int)row_bytes, (int)wpr,
+                               (int)total_ws, ds, topk, (int)row_bytes);
+        int rc = launch_status("mx_quant_rows_kernel (scatter)");
+        if (rc) return rc;
+    }
+    return CCH_OK;
+}
+
 }  // namespace cch
+
+extern "C" int cch_mx_quant_scatter_packed(const void *x, const int32_t *expanded_row_idx, void *packed_out, int64_t tokens,
+                                           int64_t k, int top_k, int fmt, int rounding, void *stream)
+{
+    using namespace cch;
+    CCH_REQUIRE(tokens >= 0 && k >= 0, "cch_mx_quant_scatter_packed: negative shape tokens=%lld k=%lld", (long long)tokens,
+                (long long)k);
+    CCH_REQUIRE(k < (int64_t)1 << 30, "cch_mx_quant_scatter_packed: k=%lld too large", (long long)k);
+    CCH_REQUIRE(top_k >= 0 && top_k <= QUANT_MAX_TOPK, "cch_mx_quant_scatter_packed: top_k=%d outside 0..%d", top_k,
+                QUANT_MAX_TOPK);
+    CCH_REQUIRE(rounding == CCH_ROUND_RNE || rounding == CCH_ROUND_LUT, "cch_mx_quant_scatter_packed: rounding %d", rounding);
+    if (tokens == 0 || k == 0 || top_k == 0) return CCH_OK;  // as the reference: nothing to do
+    CCH_REQUIRE(x && expanded_row_idx && packed_out, "cch_mx_quant_scatter_packed: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool lut = rounding == CCH_ROUND_LUT;
+    switch (fmt) {
+        case CCH_FMT_E4M3:
+            return lut ? launch_scatter<CCH_FMT_E4M3, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s)
+                       : launch_scatter<CCH_FMT_E4M3, CCH_ROUND_RNE, true>(x, expanded_row_idx, packed_out, tokens, k, top_k, s);
+        case CCH_FMT_E5M2:
+            return lut ? launch_scatter<CCH_FMT_E5M2, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s)
+                       : launch_scatter<CCH_FMT_E5M2, CCH_ROUND_RNE, true>(x, expanded_row_idx, packed_out, tokens, k, top_k, s);
+        case CCH_FMT_E2M1:
+            return lut ? launch_scatter<CCH_FMT_E2M1, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s)
+                       : launch_scatter<CCH_FMT_E2M1, CCH_ROUND_RNE, true>(x, expanded_row_idx, packed_out, tokens, k, top_k, s);
+        default:
+            return fail(CCH_EINVAL, "cch_mx_quant_scatter_packed: unknown format %d", fmt);
+    }
+}
 
 extern "C" int cch_mx_quant_rows(const void *x, void *payload, void *scales, int64_t m, int64_t k, int fmt,
                                  int rounding, void *stream)

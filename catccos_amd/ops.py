@@ -61,6 +61,34 @@ def mx_quant(x, fmt="e4m3", rounding=ROUND_RNE):
     return payload, scales
 
 
+def packed_row_bytes(k, fmt="e4m3"):
+    """Bytes of one packed row of mx_quant_scatter_packed: payload followed by the padded scales."""
+    return ((k + 1) // 2 if _fmt(fmt) == FMT_E2M1 else k) + scale_cols(k)
+
+
+def mx_quant_scatter_packed(x, expanded_row_idx, packed_out, top_k, fmt="e4m3", rounding=ROUND_RNE):
+    """Quantises every row of x (bf16 [tokens, K]) once and writes [payload | scales] to rows
+    expanded_row_idx[t * top_k + r] of packed_out (uint8 [rows, packed_row_bytes(K)]), skipping
+    negative entries.  Rows that no route names keep their contents.  Returns packed_out."""
+    fmt = _fmt(fmt)
+    _require_gpu(x, expanded_row_idx, packed_out)
+    if x.dim() != 2 or x.dtype != torch.bfloat16:
+        raise ValueError("mx_quant_scatter_packed expects a 2-D bfloat16 tensor")
+    tokens, k = x.shape
+    if expanded_row_idx.dtype != torch.int32 or expanded_row_idx.numel() != tokens * top_k:
+        raise ValueError("expanded_row_idx must hold tokens * top_k int32 entries")
+    row_bytes = ((k + 1) // 2 if fmt == FMT_E2M1 else k) + scale_cols(k)
+    if packed_out.dim() != 2 or packed_out.dtype != torch.uint8 or packed_out.shape[1] != row_bytes or not packed_out.is_contiguous():
+        raise ValueError("packed_out must be a contiguous uint8 [rows, %d] tensor" % row_bytes)
+    if top_k and tokens and int(expanded_row_idx.max()) >= packed_out.shape[0]:
+        raise ValueError("expanded_row_idx names a row past packed_out")
+    x = x.contiguous()
+    idx = expanded_row_idx.contiguous()
+    check(_abi.lib().cch_mx_quant_scatter_packed(_ptr(x), _ptr(idx), _ptr(packed_out), tokens, k, int(top_k), fmt, rounding,
+                                                 _stream()))
+    return packed_out
+
+
 def mx_quant_b(b, fmt="e4m3", rounding=ROUND_RNE, trans_b=0):
     """MX quantisation of a right-hand operand b [K,N] (bf16) with blocks running down K.
 

@@ -127,6 +127,21 @@ int cch_mx_gemm(const void *a, const void *sa, const void *b, const void *sb, vo
 int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes, void *out,
                int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, void *stream);
 
+/* ---- MX quantisation scattered to the routed rows, packed (dispatch side of the MoE path) ----
+ * Replaces CommBlockMxQuant::QuantScatterPacked (include/catccos/comm/block/
+ * comm_block_mx_quant.hpp:319-369), called by the dispatch stage of
+ * examples/ascend950_dispatch_ffn_combine/ascend950_dispatch_ffn_combine_device.h: every token
+ * row is quantised once and the same packed row is written to each of its top_k destinations.
+ *   x                 bf16 [tokens, k] row-major
+ *   expanded_row_idx  int32 [tokens * top_k]: destination row of (token, route); negative = skip
+ *   packed_out        bytes [rows, payload_bytes + scale_bytes]: payload_bytes = k (FP8) or
+ *                     ceil(k/2) (FP4), scale_bytes = 2*ceil(k/64) E8M0 bytes (a padding entry is
+ *                     127); rows that no route names are not touched
+ *   top_k             0..8; fmt / rounding as cch_mx_quant_rows
+ * Destination rows must be distinct (two routes writing one row race, as in the reference). */
+int cch_mx_quant_scatter_packed(const void *x, const int32_t *expanded_row_idx, void *packed_out, int64_t tokens,
+                                int64_t k, int top_k, int fmt, int rounding, void *stream);
+
 /* ---- Per-token dynamic int8 quantisation with row gather (feeds config 4) ----
  * Replaces MoeV2GatherDynamicQuant (examples/aux_ops/moe_init_routing_quant_v2/
  * moe_v2_gather_dynamic_quant.h:117-150 Compute, :213-250 the gather loop), without its

@@ -138,6 +138,24 @@ def mx_quant_rows(x_bf16, fmt=E4M3, rounding=RNE):
     return payload, scales
 
 
+def packed_row_bytes(k, fmt=E4M3):
+    """Bytes of one packed row: payload followed by the padded E8M0 scales."""
+    return ((k + 1) // 2 if fmt == E2M1 else k) + scale_cols(k)
+
+
+def mx_quant_scatter_packed(x_bf16, expanded_row_idx, out_rows, top_k, fmt=E4M3, rounding=RNE, fill=0):
+    """Quantise each row of x once and write [payload | scales] to rows expanded_row_idx[t*top_k + r]
+    of a uint8 [out_rows, packed_row_bytes] array (initialised to `fill`); negative entries are skipped."""
+    x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
+    idx = np.ascontiguousarray(expanded_row_idx, dtype=np.int32).reshape(-1)
+    tokens, k = x.shape
+    assert idx.size == tokens * top_k
+    out = np.full((out_rows, packed_row_bytes(k, fmt)), fill, dtype=np.uint8)
+    rc = lib().orc_mx_quant_scatter_packed(_p(x), _p(idx), _i64(tokens), _i64(k), int(top_k), fmt, rounding, _p(out))
+    assert rc == 0
+    return out
+
+
 def mx_quant_b(b_bf16, fmt=E4M3, rounding=RNE, trans_b=0):
     """b_bf16 uint16 [K,N] quantised along K; returns (payload, scales) in the boundary layouts."""
     b = np.ascontiguousarray(b_bf16, dtype=np.uint16)

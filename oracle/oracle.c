@@ -275,6 +275,39 @@ int orc_mx_quant_rows(const uint16_t *x, int64_t M, int64_t K, int fmt, int roun
 }
 
 /*
+ * Quantise each token row once and write the same packed row
+ * [payload | E8M0 scales, padded to an even count] to every routed
+ * destination row (CommBlockMxQuant::QuantScatterPacked,
+ * include/catccos/comm/block/comm_block_mx_quant.hpp:319-369: packedRowBytes =
+ * quantBytes + AlignUp(CeilDiv(N, 32), 2); dstRow = expandedRowIdx[token *
+ * topK + route], a negative dstRow is skipped).  Rows of packed_out that no
+ * route names are left as they were.
+ * pinned by: it is orc_mx_quant_rows (pinned above) followed by row copies;
+ *            the test rebuilds the result from orc_mx_quant_rows with numpy
+ *            indexing and checks untouched rows stay untouched.
+ */
+int orc_mx_quant_scatter_packed(const uint16_t *x, const int32_t *expanded_row_idx, int64_t tokens, int64_t K,
+                                int top_k, int fmt, int rounding, uint8_t *packed_out)
+{
+    const int64_t nblk = (K + 31) / 32;
+    const int64_t sld = ((nblk + 1) / 2) * 2;
+    const int64_t pld = (fmt == ORC_FMT_E2M1) ? (K + 1) / 2 : K;
+    const int64_t row_bytes = pld + sld;
+    uint8_t *row = (uint8_t *)malloc((size_t)row_bytes);
+    if (!row) return -1;
+    for (int64_t t = 0; t < tokens; t++) {
+        orc_mx_quant_rows(x + t * K, 1, K, fmt, rounding, row, row + pld);
+        for (int r = 0; r < top_k; r++) {
+            const int32_t dst = expanded_row_idx[t * top_k + r];
+            if (dst < 0) continue;
+            memcpy(packed_out + (int64_t)dst * row_bytes, row, (size_t)row_bytes);
+        }
+    }
+    free(row);
+    return 0;
+}
+
+/*
  * MX quantisation of a bf16 matrix B [K,N] (row-major) along axis 0, as the
  * reference prepares the right-hand GEMM operand
  * (gen_data_mxfp8_mmrs.py:202-217 = quantise the transpose by rows;
