@@ -256,7 +256,31 @@ def main():
         q_gbs = qbytes / (q_us * 1e-6) / 1e9
         extra["mx_quant_cfg1"] = {"gb_per_s": round(q_gbs, 1), "frac_of_hbm_peak": round(q_gbs / HBM_PEAK_GBS, 4),
                                   "us": round(q_us, 2), "bytes": qbytes, "buffers": "6 rotating input sets (352 MB), 120 queued launches"}
-        del sets
+        # the same rows quantised once and scattered as packed [payload | scales] rows to their top-2 destinations
+        idx1 = torch.randperm(M1 * 2, device=dev).to(torch.int32)
+        packed1 = torch.empty((M1 * 2, cc.packed_row_bytes(K1)), dtype=torch.uint8, device=dev)
+        st1 = torch.cuda.current_stream().cuda_stream
+        from catccos_amd import _abi as abi1
+
+        def sc_launch(i):
+            abi1.check(abi1.lib().cch_mx_quant_scatter_packed(sets[i % len(sets)].data_ptr(), idx1.data_ptr(), packed1.data_ptr(),
+                                                              M1, K1, 2, 0, 0, st1))
+
+        for i in range(600):
+            sc_launch(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(120):
+            sc_launch(i)
+        e1.record()
+        torch.cuda.synchronize()
+        sc_us = e0.elapsed_time(e1) * 1e3 / 120
+        sc_bytes = M1 * K1 * 2 + 2 * M1 * cc.packed_row_bytes(K1)
+        extra["mx_quant_scatter_top2_cfg1_rows"] = {"gb_per_s": round(sc_bytes / sc_us / 1e3, 1),
+                                                    "frac_of_hbm_peak": round(sc_bytes / sc_us / 1e3 / HBM_PEAK_GBS, 4),
+                                                    "us": round(sc_us, 2), "bytes": sc_bytes}
+        del sets, packed1
         # config 2: int8 W8A8 + dequant
         m2, k2, n2 = 8192, 4096, 8192
         a2 = torch.randint(-127, 128, (m2, k2), dtype=torch.int8, device=dev)

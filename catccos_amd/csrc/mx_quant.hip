@@ -305,10 +305,12 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
 // (1024 elements of one row), keeps the next pair's loads in flight while it converts the
 // current one, stores 16 (FP8) or 8 (FP4) payload bytes per lane and writes the 32 scale bytes
 // of the pair as dwords gathered with row shifts.
-template <int FMT>
+// SCATTER: as in mx_quant_rows_kernel, the row goes to rows dst_idx[r*topk + 0 .. topk-1]; `sld`
+// is then the distance between scale rows of the packed output.
+template <int FMT, bool SCATTER = false>
 __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_fast_kernel(
     const uint16_t *__restrict__ x, uint8_t *__restrict__ payload, uint8_t *__restrict__ scales, int K, int sld, int pld,
-    int ppr, int npairs)
+    int ppr, int npairs, const int32_t *__restrict__ dst_idx = nullptr, int topk = 1)
 {
     constexpr bool FP4 = FMT == CCH_FMT_E2M1;
     const int lane = threadIdx.x & 63;
@@ -316,14 +318,21 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_fast_kernel(
     const int stride = (int)gridDim.x * (QUANT_THREADS / 64);
     const bool odd_lane = lane & 1;
 
-    auto fetch = [&](int p, u32x4 (&v)[2]) {
+    struct Dest {
+        int row[SCATTER ? QUANT_MAX_TOPK : 1];
+    };
+    auto fetch = [&](int p, u32x4 (&v)[2], Dest &d) {
         const int r = p / ppr, c = p - r * ppr;  // row, pair within the row (wave-uniform)
         const uint16_t *src = x + (size_t)r * K + (size_t)c * 1024 + lane * 8;
         v[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src));
         v[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 512));
+        if constexpr (SCATTER) {
+#pragma unroll
+            for (int t = 0; t < QUANT_MAX_TOPK; t++) d.row[t] = t < topk ? dst_idx[(size_t)r * topk + t] : -1;
+        }
     };
-    auto convert = [&](int p, const u32x4 (&v)[2]) {
-        const int r = p / ppr, c = p - r * ppr;
+    auto convert = [&](int p, const u32x4 (&v)[2], const Dest &d) {
+        const int r0 = p / ppr, c = p - r0 * ppr;
         uint32_t q[2][2], sdw[2];
 #pragma unroll
         for (int h = 0; h < 2; h++) {
@@ -345,32 +354,38 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_fast_kernel(
         const uint32_t recv1 = FP4 ? 0u : (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send1, 0xB1, 0xF, 0xF, true);
         // element offset inside the row of the first value this lane stores
         const int k = c * 1024 + (odd_lane ? 512 + (lane - 1) * 8 : lane * 8);
-        uint8_t *dst = payload + (size_t)r * pld + (FP4 ? (k >> 1) : k);
-        if (FP4) {
-            const u32x2 o = odd_lane ? (u32x2){recv0, q[1][0]} : (u32x2){q[0][0], recv0};
-            __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(dst));
-        } else {
-            const u32x4 o = odd_lane ? (u32x4){recv0, recv1, q[1][0], q[1][1]} : (u32x4){q[0][0], q[0][1], recv0, recv1};
-            __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(dst));
-        }
-        if ((lane & 15) == 0) {
-            uint32_t *sp = reinterpret_cast<uint32_t *>(scales + (size_t)r * sld + c * 32 + (lane >> 4) * 4);
-            sp[0] = sdw[0];
-            sp[4] = sdw[1];
+#pragma unroll
+        for (int t = 0; t < (SCATTER ? QUANT_MAX_TOPK : 1); t++) {
+            const int r = SCATTER ? d.row[t] : r0;
+            if (r < 0) continue;  // wave-uniform
+            uint8_t *dst = payload + (size_t)r * pld + (FP4 ? (k >> 1) : k);
+            if (FP4) {
+                const u32x2 o = odd_lane ? (u32x2){recv0, q[1][0]} : (u32x2){q[0][0], recv0};
+                __builtin_nontemporal_store(o, reinterpret_cast<u32x2 *>(dst));
+            } else {
+                const u32x4 o = odd_lane ? (u32x4){recv0, recv1, q[1][0], q[1][1]} : (u32x4){q[0][0], q[0][1], recv0, recv1};
+                __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(dst));
+            }
+            if ((lane & 15) == 0) {
+                uint32_t *sp = reinterpret_cast<uint32_t *>(scales + (size_t)r * sld + c * 32 + (lane >> 4) * 4);
+                sp[0] = sdw[0];
+                sp[4] = sdw[1];
+            }
         }
     };
 
     u32x4 v0[2], v1[2];
+    Dest d0, d1;
     int p0 = wave;
     if (p0 >= npairs) return;
-    fetch(p0, v0);
+    fetch(p0, v0, d0);
     for (;;) {
         const int p1 = p0 + stride, p2 = p1 + stride;  // wave-uniform
-        if (p1 < npairs) fetch(p1, v1);
-        convert(p0, v0);
+        if (p1 < npairs) fetch(p1, v1, d1);
+        convert(p0, v0, d0);
         if (p1 >= npairs) break;
-        if (p2 < npairs) fetch(p2, v0);
-        convert(p1, v1);
+        if (p2 < npairs) fetch(p2, v0, d0);
+        convert(p1, v1, d1);
         if (p2 >= npairs) break;
         p0 = p2;
     }
@@ -509,8 +524,17 @@ static int launch_scatter(const void *x, const int32_t *dst_idx, void *packed, i
     CCH_HIP(hipGetDevice(&dev));
     CCH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     const int64_t max_blocks = (int64_t)cus * QUANT_BLOCKS_PER_CU;
-    const int64_t rows_per_launch = std::max<int64_t>(1, (int64_t)(1 << 30) / wpr);
     uint8_t *out = static_cast<uint8_t *>(packed);
+    if (HWCVT && k % 1024 == 0 && aligned(x, 16) && aligned(packed, 16) && row_bytes % 16 == 0 &&
+        tokens * (k / 1024) < ((int64_t)1 << 30)) {
+        const int64_t npairs = tokens * (k / 1024);
+        const unsigned grid = (unsigned)std::min<int64_t>((npairs + QUANT_THREADS / 64 - 1) / (QUANT_THREADS / 64), max_blocks);
+        hipLaunchKernelGGL((mx_quant_rows_fast_kernel<FMT, true>), dim3(grid), dim3(QUANT_THREADS), 0, stream,
+                           static_cast<const uint16_t *>(x), out, out + pbytes, (int)k, (int)row_bytes, (int)row_bytes,
+                           (int)(k / 1024), (int)npairs, dst_idx, topk);
+        return launch_status("mx_quant_rows_fast_kernel (scatter)");
+    }
+    const int64_t rows_per_launch = std::max<int64_t>(1, (int64_t)(1 << 30) / wpr);
     for (int64_t r0 = 0; r0 < tokens; r0 += rows_per_launch) {
         const int64_t rows = std::min(rows_per_launch, tokens - r0);
         const int64_t total_ws = rows * wpr;
