@@ -333,6 +333,31 @@ def main():
         extra["dyn_quant_i8_cfg4_tokens"] = {"gb_per_s": round(dq_bytes / dq_us / 1e3, 1), "frac_of_hbm_peak": round(dq_bytes / dq_us / 1e3 / HBM_PEAK_GBS, 4),
                                              "us": round(dq_us, 2), "bytes": dq_bytes}
         del xs4, q4
+        # combine side: top-2 weighted un-permute of 8192 expert-output rows back to 4096 tokens
+        tok_u, hid_u, topk_u = 4096, 7168, 2
+        ys = [torch.randn(tok_u * topk_u, hid_u, device=dev).to(torch.bfloat16) for _ in range(3)]
+        idx_u = torch.randperm(tok_u * topk_u, device=dev).to(torch.int32)
+        pr_u = torch.rand(tok_u * topk_u, device=dev)
+        out_u = torch.empty((tok_u, hid_u), dtype=torch.bfloat16, device=dev)
+
+        def un_launch(i):
+            _abi.check(_abi.lib().cch_moe_token_unpermute(ys[i % 3].data_ptr(), idx_u.data_ptr(), pr_u.data_ptr(), out_u.data_ptr(),
+                                                          tok_u * topk_u, tok_u, hid_u, topk_u, st4))
+
+        for i in range(600):
+            un_launch(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(60):
+            un_launch(i)
+        e1.record()
+        torch.cuda.synchronize()
+        un_us = e0.elapsed_time(e1) * 1e3 / 60
+        un_bytes = tok_u * topk_u * hid_u * 2 + tok_u * hid_u * 2 + tok_u * topk_u * 8
+        extra["moe_token_unpermute_top2"] = {"gb_per_s": round(un_bytes / un_us / 1e3, 1), "frac_of_hbm_peak": round(un_bytes / un_us / 1e3 / HBM_PEAK_GBS, 4),
+                                             "us": round(un_us, 2), "bytes": un_bytes}
+        del ys, out_u
         # config 5: MXFP4 grouped (same groups as the headline)
         a5, sa5 = cc.mx_quant((torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16), "e2m1")
         b5 = torch.empty((E, K, N // 2), dtype=torch.uint8, device=dev)

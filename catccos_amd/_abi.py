@@ -34,6 +34,7 @@ PROTOTYPES = {
     "cch_mx_quant_rows": [_P, _P, _P, _I64, _I64, _I, _I, _P],
     "cch_mx_quant_b": [_P, _P, _P, _I64, _I64, _I, _I, _I, _P],
     "cch_mx_quant_scatter_packed": [_P, _P, _P, _I64, _I64, _I, _I, _I, _P],
+    "cch_moe_token_unpermute": [_P, _P, _P, _P, _I64, _I64, _I64, _I, _P],
     "cch_dyn_quant_i8_rows": [_P, _P, _P, _P, _I64, _I64, _I64, _I, _I, _P],
     "cch_gemm_i8_dequant": [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I, _P],
     "cch_gmm_i8_dequant_swiglu": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _P],

@@ -141,6 +141,31 @@ def dynamic_quant_i8(x, src_rows=None, topk=1, mode=DQ_DEVICE):
     return q, scale
 
 
+def moe_token_unpermute(permuted_tokens, sorted_indices, probs=None, top_k=1):
+    """out[t] = sum_j permuted_tokens[sorted_indices[t*top_k + j]] * probs[t*top_k + j] (bf16 [tokens, hidden]).
+
+    permuted_tokens bf16 [rows, hidden]; sorted_indices int32 with tokens*top_k entries (entries outside
+    [0, rows) contribute nothing); probs float32 with as many entries, or None for a plain sum."""
+    _require_gpu(permuted_tokens, sorted_indices)
+    if permuted_tokens.dim() != 2 or permuted_tokens.dtype != torch.bfloat16:
+        raise ValueError("permuted_tokens must be a 2-D bfloat16 tensor")
+    if sorted_indices.dtype != torch.int32 or sorted_indices.numel() % top_k != 0:
+        raise ValueError("sorted_indices must hold tokens * top_k int32 entries")
+    x = permuted_tokens.contiguous()
+    idx = sorted_indices.contiguous().reshape(-1)
+    rows, hidden = x.shape
+    tokens = idx.numel() // top_k
+    if probs is not None:
+        _require_gpu(probs)
+        if probs.dtype != torch.float32 or probs.numel() != idx.numel():
+            raise ValueError("probs must hold tokens * top_k float32 entries")
+        probs = probs.contiguous().reshape(-1)
+    out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=x.device)
+    check(_abi.lib().cch_moe_token_unpermute(_ptr(x), _ptr(idx), _ptr(probs) if probs is not None else None, _ptr(out), rows,
+                                             tokens, hidden, int(top_k), _stream()))
+    return out
+
+
 def set_option(name, value):
     """Library switch (see cch_set_option in include/catccos_hip.h)."""
     check(_abi.lib().cch_set_option(name.encode(), int(value)))

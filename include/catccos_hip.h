@@ -142,6 +142,21 @@ int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, con
 int cch_mx_quant_scatter_packed(const void *x, const int32_t *expanded_row_idx, void *packed_out, int64_t tokens,
                                 int64_t k, int top_k, int fmt, int rounding, void *stream);
 
+/* ---- MoE token un-permute (combine side of the MoE path) ----
+ * Replaces KernelMoeTokenUnpermute (examples/aux_ops/moe_token_unpermute/
+ * moe_token_unpermute.h:235-355), the last stage of DispatchFFNCombine
+ * (examples/dispatch_ffn_combine/dispatch_ffn_combine_device.h:886-898).
+ *   permuted_tokens  bf16 [rows, hidden]: expert outputs in the expert-sorted row order
+ *   sorted_indices   int32 [tokens * top_k]: row of permuted_tokens that holds route j of token t;
+ *                    an entry outside [0, rows) contributes nothing
+ *   probs            fp32 [tokens * top_k] routing weights, or NULL for an unweighted sum
+ *   out              bf16 [tokens, hidden] = sum_j permuted[sorted_indices[t,j]] * probs[t,j]: fp32,
+ *                    each product rounded before it is added, routes in order, route 0 assigns;
+ *                    rounded to nearest even
+ *   top_k            1..8 */
+int cch_moe_token_unpermute(const void *permuted_tokens, const int32_t *sorted_indices, const float *probs, void *out,
+                            int64_t rows, int64_t tokens, int64_t hidden, int top_k, void *stream);
+
 /* ---- Per-token dynamic int8 quantisation with row gather (feeds config 4) ----
  * Replaces MoeV2GatherDynamicQuant (examples/aux_ops/moe_init_routing_quant_v2/
  * moe_v2_gather_dynamic_quant.h:117-150 Compute, :213-250 the gather loop), without its

@@ -304,3 +304,18 @@ def compare(d, g, rtol=2.0 ** -7):
     m = np.zeros(5, dtype=np.float64)
     lib().orc_compare(_p(d), _p(g), _i64(d.size), ctypes.c_float(rtol), _p(m))
     return {"max_rel_floor1": m[0], "max_rel_floor_rms": m[1], "eb": m[2], "rms_golden": m[3], "frac_bad": m[4]}
+
+
+def moe_token_unpermute(permuted_bf16, sorted_indices, probs, top_k):
+    """permuted uint16 [rows, hidden] (bf16 bits), sorted_indices int32 [tokens*top_k], probs float32
+    [tokens*top_k] or None -> uint16 [tokens, hidden]."""
+    x = np.ascontiguousarray(permuted_bf16, dtype=np.uint16)
+    idx = np.ascontiguousarray(sorted_indices, dtype=np.int32).reshape(-1)
+    rows, hidden = x.shape
+    tokens = idx.size // top_k
+    pr = None if probs is None else np.ascontiguousarray(probs, dtype=np.float32).reshape(-1)
+    out = np.empty((tokens, hidden), dtype=np.uint16)
+    rc = lib().orc_moe_token_unpermute(_p(x), _p(idx), _p(pr) if pr is not None else None, _i64(rows), _i64(tokens),
+                                       _i64(hidden), int(top_k), _p(out))
+    assert rc == 0
+    return out

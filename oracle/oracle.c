@@ -804,3 +804,41 @@ int orc_num_threads(void)
     return 1;
 #endif
 }
+
+/*
+ * MoE token un-permute: out[t] = sum over the top_k routes of token t of
+ * permuted[sorted_indices[t*top_k + j]] * probs[t*top_k + j], as the reference
+ * kernel computes it (examples/aux_ops/moe_token_unpermute/moe_token_unpermute.h:
+ * 235-279): fp32 throughout, the product of each route rounded on its own
+ * (Muls, :315 / :330) before it is added (Add, :333), route 0 assigns (or the
+ * sum starts at zero when its index is not below `rows`, :247-258), routes
+ * with an index outside [0, rows) are skipped, and the result is cast with
+ * CAST_RINT (:353) = round to nearest even.  probs may be NULL (no weighting).
+ * The reference's Python fallback (gen_data_moe.py:60-70) accumulates in the
+ * token dtype instead and takes the inverse permutation as its index; it is not
+ * what this function follows.
+ * pinned by: a torch restatement with one separately rounded fp32 op per step,
+ *            gather special case (top_k = 1, probs = 1), linearity in probs by
+ *            powers of two.
+ */
+__attribute__((optimize("fp-contract=off")))
+int orc_moe_token_unpermute(const uint16_t *permuted, const int32_t *sorted_indices, const float *probs,
+                            int64_t rows, int64_t tokens, int64_t hidden, int top_k, uint16_t *out)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t t = 0; t < tokens; t++) {
+        for (int64_t h = 0; h < hidden; h++) {
+            float acc = 0.0f;
+            for (int j = 0; j < top_k; j++) {
+                const int64_t idx = sorted_indices[t * top_k + j];
+                if (idx < 0 || idx >= rows) continue;
+                volatile float v = orc_bf16_to_f32(permuted[idx * hidden + h]);
+                if (probs) v = v * probs[t * top_k + j];
+                if (j == 0) acc = v;
+                else acc = acc + v;
+            }
+            out[t * hidden + h] = orc_f32_to_bf16(acc);
+        }
+    }
+    return 0;
+}
