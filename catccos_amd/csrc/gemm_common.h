@@ -21,7 +21,9 @@ struct GemmProblem {
     const uint8_t *sb;       // MX: per expert trans_b ? [N, sld] : [sld/2, N, 2]
     const float *per_tok;    // int8: [T]
     const float *per_ch;     // int8: [E, N]
-    uint16_t *out;           // bf16 [T, n_out]
+    uint16_t *out;           // bf16 [T, n_out] (with out_row_map: [out_rows, n_out])
+    const int32_t *out_row_map;  // device int32[T] or nullptr: row of `out` that receives row i (negative: dropped)
+    int64_t out_rows;        // rows of `out` when out_row_map is given
     const int32_t *group_sizes;  // device int32[E] or nullptr (dense, E = 1)
     int num_groups;
     int T, N, K;             // K in elements

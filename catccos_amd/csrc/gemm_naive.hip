@@ -75,6 +75,12 @@ __global__ __launch_bounds__(256) void gemm_naive_kernel(GemmProblem p)
     const int row = blockIdx.y;
     if (col >= p.n_out) return;
     const int e = find_group(tab, p.num_groups, row);  // bm = 1: tile rows are rows
+    size_t out_row = (size_t)row;
+    if (p.out_row_map) {
+        // mapped output: rows of no group and rows mapped to a negative index are not written
+        if (e >= p.num_groups || p.out_row_map[row] < 0) return;
+        out_row = (size_t)p.out_row_map[row];
+    }
     float v = 0.0f;
     if (e < p.num_groups) {
         if (EPI == EPI_DEQUANT_SWIGLU) {
@@ -89,7 +95,7 @@ __global__ __launch_bounds__(256) void gemm_naive_kernel(GemmProblem p)
             v = dot_column<KIND>(p, row, e, col);
         }
     }
-    p.out[(size_t)row * p.n_out + col] = (uint16_t)f32_to_bf16_bits(v);
+    p.out[out_row * p.n_out + col] = (uint16_t)f32_to_bf16_bits(v);
 }
 
 template <int KIND, int EPI>

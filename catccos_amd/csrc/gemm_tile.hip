@@ -249,7 +249,8 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     // Rows that belong to no group are written as zeros (the reference's golden pads them,
     // examples/utils/gen_data_fp4_mx_alltoallv_gmm.py:788-790): all workgroups share the range,
     // 16 bytes per thread and pass; usually it is empty.
-    if (p.group_sizes) {
+    const bool has_map = EPI == EPI_PLAIN && p.out_row_map != nullptr;   // rows go where the map says
+    if (p.group_sizes && !has_map) {
         const size_t begin = (size_t)uniform(tab.row_start[p.num_groups]) * p.n_out / 8, end = (size_t)p.T * p.n_out / 8;
         v4u *o16 = reinterpret_cast<v4u *>(p.out);
         for (size_t i = begin + (size_t)blockIdx.x * TILE_THREADS + threadIdx.x; i < end; i += (size_t)gridDim.x * TILE_THREADS)
@@ -359,6 +360,12 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             if (SWIGLU) col = ((idx >> 5) & 1) * p.n_out + min(c.j0 + (idx >> 6) * 32 + (idx & 31), p.n_out - 1);
             else col = min(c.j0 + idx, p.N - 1);
             load4_to_lds(make_rsrc(p.per_ch + (size_t)c.e * p.N, c.lim), (uint32_t)col * 4u, 0u, dst + 1024u);
+        } else {
+            // destination rows of the tile's 256 rows, where the per-token scales of the other
+            // epilogues go; without a map the descriptor is empty and nothing is fetched
+            const int idx = (wave & 3) * 64 + lane;
+            const uint32_t dst = lds_base + (uint32_t)(PARAM_OFF + parity * PARAM_SET) + (uint32_t)(wave & 3) * 256u;
+            load4_to_lds(make_rsrc(p.out_row_map + c.m0, has_map ? c.lim : 0u), (uint32_t)min(idx, c.m_end - 1 - c.m0) * 4u, 0u, dst);
         }
         issue_scales(1, c, 0, gi & 1);
         gi++;
@@ -613,7 +620,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             int lane_e = lane;
             asm volatile("" : "+v"(lane_e));
             const __amdgpu_buffer_rsrc_t rs_out =
-                __builtin_amdgcn_make_buffer_rsrc(p.out + (size_t)cur.m0 * p.n_out, 0, 0x7FFFFFFF, 0x00020000);
+                __builtin_amdgcn_make_buffer_rsrc(p.out + (has_map ? (size_t)0 : (size_t)cur.m0 * p.n_out), 0, 0x7FFFFFFF, 0x00020000);
             float chs[NT];
             if (EPI != EPI_PLAIN) {
 #pragma unroll
@@ -666,8 +673,14 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                     const v4i val = lds_read16(epi + (uint32_t)(lrow * ROWB + chunk * 16));
                     const int row = wm * WM + i * 32 + ps * PASS_ROWS + lrow;  // relative to m0
                     const int col = cur.j0 + wn * WN_OUT + chunk * 8;
-                    const bool ok = (cur.m0 + row < cur.m_end) && (col + 8 <= p.n_out);
-                    const uint32_t off = ok ? ((uint32_t)row * (uint32_t)p.n_out + (uint32_t)col) * 2u : 0xFFFFFFF0u;
+                    bool ok = (cur.m0 + row < cur.m_end) && (col + 8 <= p.n_out);
+                    uint32_t out_row = (uint32_t)row;
+                    if constexpr (EPI == EPI_PLAIN) {
+                        const int mapped = (int)lds_read4(prm + (uint32_t)row * 4u);
+                        ok = ok && (!has_map || mapped >= 0);
+                        out_row = has_map ? (uint32_t)mapped : out_row;
+                    }
+                    const uint32_t off = ok ? (out_row * (uint32_t)p.n_out + (uint32_t)col) * 2u : 0xFFFFFFF0u;
                     __builtin_amdgcn_raw_buffer_store_b128((v4u){(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]},
                                                            rs_out, (int)off, 0, 0);
                 }
@@ -708,6 +721,8 @@ bool gemm_tile_supports(const GemmProblem &p, int kind, int epi)
     if (p.K < 2 * BKB * epb || p.K % (BKB * epb) != 0) return false;
     if (p.n_out % 8 != 0 || !aligned(p.out, 16)) return false;
     if ((int64_t)BM * p.n_out * 2 >= ((int64_t)1 << 31)) return false;
+    // mapped output rows are addressed from the start of `out` with 32-bit offsets
+    if (p.out_row_map && (epi != EPI_PLAIN || p.out_rows * p.n_out * 2 >= ((int64_t)1 << 31) || !aligned(p.out_row_map, 4))) return false;
     if (p.num_groups > MAX_GROUPS) return false;
     if ((int64_t)p.N * (p.K / epb) >= ((int64_t)1 << 31)) return false;  // 32-bit source offsets
     if (!aligned(p.a, 16) || !aligned(p.b, 16) || p.b_stride % 16 != 0) return false;

@@ -127,6 +127,21 @@ int cch_mx_gemm(const void *a, const void *sa, const void *b, const void *sb, vo
 int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes, void *out,
                int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, void *stream);
 
+/* ---- MXFP8 / MXFP4 grouped matmul with mapped output rows (down projection, config-5 twin) ----
+ * Replaces the matmul half of GroupedMatmulAllToAllV for MX operands
+ * (include/catccos/dgemm/kernel/grouped_matmul_alltoallv_mx.hpp:250 with the scheduler's RemapperC,
+ * include/catccos/dgemm/block/block_scheduler_reducescatter_alltoallv.hpp:237-256; launched by
+ * LaunchAscend950Fp8MxGroupedMatmulAllToAllVFP16, tests/dynamic_tiling/impl/kernel_fp16_ascend950.cpp:446):
+ * the result rows leave in the order of the send buffer (by destination rank, then expert) instead of
+ * the order of the tokens (by expert, then source rank).  Operands as cch_mx_gmm, plus
+ *   out_row_map  int32 [t]: row of `out` that receives the result of row i of a; negative = dropped.
+ *                Entries of rows past sum(group_sizes) are ignored (those rows produce nothing).
+ *   out          bf16 [out_rows, n]; rows that the map does not name are not written
+ * Destination rows must be distinct. */
+int cch_mx_gmm_mapped(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes,
+                      const int32_t *out_row_map, void *out, int64_t out_rows, int64_t num_experts, int64_t t, int64_t n,
+                      int64_t k, int fmt, int trans_b, void *stream);
+
 /* ---- MX quantisation scattered to the routed rows, packed (dispatch side of the MoE path) ----
  * Replaces CommBlockMxQuant::QuantScatterPacked (include/catccos/comm/block/
  * comm_block_mx_quant.hpp:319-369), called by the dispatch stage of

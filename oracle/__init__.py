@@ -319,3 +319,38 @@ def moe_token_unpermute(permuted_bf16, sorted_indices, probs, top_k):
                                        _i64(hidden), int(top_k), _p(out))
     assert rc == 0
     return out
+
+
+def send_buffer_row_map(global_tokens_per_local_expert, rank_rows=None):
+    """Destination row of every result row of the down-projection grouped matmul.
+
+    Tokens arrive grouped by local expert and, inside an expert, by the rank they came from
+    (chunk (e, r) holds global_tokens_per_local_expert[r, e] rows); results leave grouped by
+    destination rank and, inside a rank, by expert (the reference's RemapperC,
+    include/catccos/dgemm/block/block_scheduler_reducescatter_alltoallv.hpp:237-256, and the golden's
+    simulate_all_to_all_v_with_unpermute, examples/utils/gen_data_gmm_alltoallv_fp8_mx.py:720-737).
+    Rank r's region starts at row r * rank_rows (default: directly after rank r-1's rows).
+    Pure index arithmetic, pinned by a brute-force rebuild in the tests."""
+    g = np.asarray(global_tokens_per_local_expert, dtype=np.int64)
+    ranks, experts = g.shape
+    per_rank = g.sum(axis=1)
+    starts = np.arange(ranks) * rank_rows if rank_rows is not None else np.concatenate([[0], np.cumsum(per_rank)[:-1]])
+    out = np.empty(int(g.sum()), dtype=np.int32)
+    src = 0
+    for e in range(experts):
+        for r in range(ranks):
+            n = int(g[r, e])
+            dst = starts[r] + int(g[r, :e].sum())
+            out[src:src + n] = np.arange(dst, dst + n)
+            src += n
+    return out
+
+
+def scatter_rows(values, row_map, out_rows, fill=0):
+    """out[row_map[i]] = values[i] for row_map[i] >= 0; other rows hold `fill`."""
+    values = np.asarray(values)
+    out = np.full((out_rows,) + values.shape[1:], fill, dtype=values.dtype)
+    m = np.asarray(row_map)
+    keep = m >= 0
+    out[m[keep]] = values[: m.size][keep]
+    return out

@@ -244,3 +244,45 @@ def test_mx_gmm_tiled(fmt, cfg, trans_b, tiled_only):
     want = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], trans_b, group_sizes=gs)
     got = out_f32(cc.mx_grouped_matmul(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), fmt, trans_b))
     assert_close(got, want, ("mx gmm tiled", fmt, cfg[:4], trans_b))
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e2m1"])
+@pytest.mark.parametrize("trans_b", [0, 1])
+@pytest.mark.parametrize("tiled", [True, False])
+def test_mx_gmm_mapped_rows(fmt, trans_b, tiled):
+    """Down-projection form: result rows leave in send-buffer order (by destination rank, then
+    expert); dropped rows and rows of no group are not written."""
+    ranks, e, k, n = 3, 5, 1024, 416
+    rng = np.random.default_rng(77 + trans_b)
+    g = rng.integers(0, 260, (ranks, e)).astype(np.int32)
+    g[:, 2] = 0                                                  # an expert nobody routed to
+    gs = g.sum(axis=0).astype(np.int32)
+    used = int(gs.sum())
+    t = used + 19                                                # rows past the groups
+    rank_rows = int(g.sum(axis=1).max()) + 5
+    row_map = np.full(t, -1, np.int32)
+    row_map[:used] = orc.send_buffer_row_map(g, rank_rows)
+    row_map[7] = -1                                              # a dropped row
+    sigma = 0.02 if fmt == "e2m1" else 1.0
+    pa, sa = orc.mx_quant_rows(rand_bf16(rng, (t, k), sigma), FMT[fmt])
+    pbs, sbs = [], []
+    for _ in range(e):
+        pb, sb = orc.mx_quant_b(rand_bf16(rng, (k, n), sigma), FMT[fmt], orc.RNE, trans_b)
+        pbs.append(pb)
+        sbs.append(sb)
+    pb, sb = np.stack(pbs), np.stack(sbs)
+    gold = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], trans_b, group_sizes=gs)
+    want = orc.scatter_rows(gold[:used], row_map[:used], ranks * rank_rows, fill=np.float32(-3.0))
+    cc.set_option("require_tiled_gemm", 1 if tiled else 0)
+    cc.set_option("force_generic_gemm", 0 if tiled else 1)
+    try:
+        out = torch.full((ranks * rank_rows, n), -3.0, dtype=torch.bfloat16, device="cuda")
+        cc.mx_grouped_matmul_mapped(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), dev(row_map), out, fmt, trans_b)
+        got = out_f32(out)
+    finally:
+        cc.set_option("require_tiled_gemm", 0)
+        cc.set_option("force_generic_gemm", 0)
+    untouched = np.ones(ranks * rank_rows, bool)
+    untouched[row_map[:used][row_map[:used] >= 0]] = False
+    assert (got[untouched] == -3.0).all()
+    assert_close(got[~untouched], want[~untouched], ("mx gmm mapped", fmt, trans_b, tiled))

@@ -54,3 +54,33 @@ def test_tile_order_serpentine_small_case():
     want_rows = [0, 0, 0, 1, 1, 1, 2, 2, 2, 3, 3, 3, 4, 4, 4]
     assert list(rec[:, 3]) == want_cols and list(rec[:, 2]) == want_rows
     assert list(rec[:, 0]) == [i % 2 for i in range(15)]
+
+
+def test_send_buffer_row_map_against_brute_force():
+    # rebuild the golden's reordering literally: split the expert-major rows into (expert, rank)
+    # chunks, then concatenate per destination rank in expert order
+    # (gen_data_gmm_alltoallv_fp8_mx.py:720-737 with one expert-parallel rank)
+    rng = np.random.default_rng(0)
+    for ranks, experts in [(1, 4), (2, 3), (4, 8), (3, 1)]:
+        g = rng.integers(0, 6, (ranks, experts))
+        g[rng.integers(0, ranks), rng.integers(0, experts)] = 0
+        total = int(g.sum())
+        rows = np.arange(total)
+        chunks = np.split(rows, np.cumsum(g.T.reshape(-1))[:-1])            # [expert][rank]
+        want_order = np.concatenate([np.concatenate([chunks[e * ranks + r] for e in range(experts)] or [rows[:0]])
+                                     for r in range(ranks)] or [rows[:0]])
+        m = orc.send_buffer_row_map(g)
+        assert sorted(m.tolist()) == list(range(total))
+        assert np.array_equal(want_order[m], rows)                           # row i lands where the golden puts it
+        padded = orc.send_buffer_row_map(g, rank_rows=total + 3)
+        per_rank = g.sum(axis=1)
+        for r in range(ranks):
+            sel = (padded >= r * (total + 3)) & (padded < (r + 1) * (total + 3))
+            assert sel.sum() == per_rank[r]
+
+
+def test_scatter_rows_places_and_drops():
+    vals = np.arange(12, dtype=np.float32).reshape(4, 3)
+    out = orc.scatter_rows(vals, np.array([2, -1, 0, 5], np.int32), 6, fill=-7)
+    assert np.array_equal(out[2], vals[0]) and np.array_equal(out[0], vals[2]) and np.array_equal(out[5], vals[3])
+    assert (out[[1, 3, 4]] == -7).all()
