@@ -3,6 +3,7 @@
 // communication stage of the reference operator is dropped, so rankSize only selects file names
 // and output offsets.  File names follow the reference's <op>_host.h files (cited per class);
 // all files are raw little-endian arrays without header.
+#include <algorithm>
 #include <cstdlib>
 #include <vector>
 
@@ -239,6 +240,75 @@ public:
 using Ascend950Fp4MxAllToAllVGroupedMatmulOperator = MxAllToAllVGroupedMatmulOperator<true, ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL>;
 using Ascend950Fp8MxAllToAllVGroupedMatmulOperator = MxAllToAllVGroupedMatmulOperator<false, ASCEND950_FP8_MX_ALLTOALLV_GROUPED_MATMUL>;
 
+// ---------------------------------------------------------------------------------------------
+// MX grouped matmul whose results leave in send-buffer order, FP8 and FP4 payload (reference
+// examples/ascend950_fp8_mx_grouped_matmul_alltoallv/ascend950_fp8_mx_grouped_matmul_alltoallv_host.h:
+// 16-160 and its fp4 twin): the down projection of the MoE layer.  ptrA = tokens grouped by local
+// expert and, inside an expert, by the rank they came from (m rows), ptrB = W [E,...], ptrC = out
+// bf16 [rankSize * m, n] zero-filled, region r holding the rows that go back to rank r in expert
+// order; custom[0] = scaleA, custom[1] = scaleB, custom[2] = local_tokens_per_expert (unused on one
+// rank), custom[3] = global_tokens_per_local_expert int32 [rankSize, E].  Derived here, as the
+// reference's scheduler derives them on the device (block_scheduler_reducescatter_alltoallv.hpp:
+// 211-256): custom[4] = rows per expert, custom[5] = destination row of every row of A.
+// The reference registers this operator for fp16 output; this build's GEMM epilogue writes bf16.
+template <bool FP4, CocCommType KIND> class MxGroupedMatmulAllToAllVOperator : public CatccosOperator {
+public:
+    void AllocateDeviceSpace(KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        const size_t m = t.m, k = t.k, n = t.n, ranks = t.rankSize ? t.rankSize : 1, sc = ScaleCols(k), pack = FP4 ? 2 : 1;
+        const size_t e = t.expertNum / (t.epSize ? t.epSize : 1);
+        const int one = FP4 ? 0x22 : 0x38;  // payload 1.0 in either format
+        uint8_t *a = LoadOrFill(m * k / pack, dataFile, "a_gm_" + R(rankId) + ".bin", one);
+        uint8_t *b = LoadOrFill(e * k * n / pack, dataFile, "b_gm_" + R(rankId) + ".bin", one);
+        uint8_t *sa = LoadOrFill(m * sc, dataFile, "a_scale_" + R(rankId) + ".bin", 127);
+        uint8_t *sb = LoadOrFill(e * n * sc, dataFile, "b_scale_" + R(rankId) + ".bin", 127);
+        const size_t outBytes = ranks * m * n * 2;
+        uint8_t *d = DeviceAlloc(outBytes);
+        CCH_CHECK(cch_memset(d, 0, outBytes));
+        std::vector<int32_t> local(t.expertNum, 0), global(ranks * e, 0);
+        for (size_t r = 0; r < ranks; r++)
+            for (size_t i = 0; i < e; i++) global[r * e + i] = static_cast<int32_t>(m / (ranks * e));
+        if (!dataFile.empty()) {
+            ReadFile(dataFile + "/local_tokens_per_expert_" + R(rankId) + ".bin", local.data(), local.size() * 4);
+            ReadFile(dataFile + "/global_tokens_per_local_expert_" + R(rankId) + ".bin", global.data(), global.size() * 4);
+        }
+        // rows per expert, and where each row goes: chunk (expert i, rank r) of A -> region r, after
+        // the chunks of experts 0..i-1 for that rank
+        std::vector<int32_t> groups(e, 0), rowMap(m, -1);
+        size_t src = 0;
+        for (size_t i = 0; i < e; i++) {
+            for (size_t r = 0; r < ranks; r++) {
+                const int64_t cnt = std::max<int32_t>(global[r * e + i], 0);
+                int64_t dst = static_cast<int64_t>(r * m);
+                for (size_t j = 0; j < i; j++) dst += std::max<int32_t>(global[r * e + j], 0);
+                for (int64_t x = 0; x < cnt && src < m; x++) rowMap[src++] = static_cast<int32_t>(dst + x);
+                groups[i] += static_cast<int32_t>(cnt);
+            }
+        }
+        uint8_t *localDev = DeviceAlloc(local.size() * 4), *globalDev = DeviceAlloc(global.size() * 4);
+        uint8_t *grpDev = DeviceAlloc(e * 4), *mapDev = DeviceAlloc(m * 4);
+        CCH_CHECK(cch_memcpy_h2d(localDev, local.data(), local.size() * 4));
+        CCH_CHECK(cch_memcpy_h2d(globalDev, global.data(), global.size() * 4));
+        CCH_CHECK(cch_memcpy_h2d(grpDev, groups.data(), e * 4));
+        CCH_CHECK(cch_memcpy_h2d(mapDev, rowMap.data(), m * 4));
+        params.SetKernelParams(a, b, d, sa, sb, localDev, globalDev, grpDev, mapDev);
+    }
+    void WriteResultFile(const KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        const size_t ranks = t.rankSize ? t.rankSize : 1;
+        DumpDevice(params.ptrC, ranks * t.m * static_cast<size_t>(t.n) * 2, dataFile + "/output_" + R(rankId) + ".bin");
+    }
+    size_t GetWorkspaceSize(const CocTilingParams &) override { return 0; }
+    CocCommType GetActualKernelType(const CocTilingParams &) override { return KIND; }
+    bool CheckCocTilingParams(uint32_t, const CocTilingParams &t) override
+    {
+        return t.m > 0 && t.k > 0 && t.n > 0 && t.k % 64 == 0 && t.expertNum > 0 && (!FP4 || t.n % 2 == 0) &&
+               static_cast<uint64_t>(t.rankSize ? t.rankSize : 1) * t.m < (1ull << 31);
+    }
+};
+using Ascend950Fp8MxGroupedMatmulAllToAllVOperator = MxGroupedMatmulAllToAllVOperator<false, ASCEND950_FP8_MX_GROUPED_MATMUL_ALLTOALLV>;
+using Ascend950Fp4MxGroupedMatmulAllToAllVOperator = MxGroupedMatmulAllToAllVOperator<true, ASCEND950_FP4_MX_GROUPED_MATMUL_ALLTOALLV>;
+
 }  // namespace
 
 REGISTER_OPERATOR("MxQuantAllGather", MxQuantAllGatherOperator)
@@ -247,3 +317,5 @@ REGISTER_OPERATOR("Ascend950MxFp8MatmulReduceScatter", Ascend950MxFp8MatmulReduc
 REGISTER_OPERATOR("DispatchGmmDequantSwiglu", DispatchGmmDequantSwigluOperator)
 REGISTER_OPERATOR("Ascend950Fp4MxAllToAllVGroupedMatmul", Ascend950Fp4MxAllToAllVGroupedMatmulOperator)
 REGISTER_OPERATOR("Ascend950Fp8MxAllToAllVGroupedMatmul", Ascend950Fp8MxAllToAllVGroupedMatmulOperator)
+REGISTER_OPERATOR("Ascend950Fp8MxGroupedMatmulAllToAllV", Ascend950Fp8MxGroupedMatmulAllToAllVOperator)
+REGISTER_OPERATOR("Ascend950Fp4MxGroupedMatmulAllToAllV", Ascend950Fp4MxGroupedMatmulAllToAllVOperator)

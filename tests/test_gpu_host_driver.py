@@ -102,3 +102,26 @@ def test_mx_grouped_files(tmp_path, kernel, fmt):
     gs.tofile(tmp_path / "global_tokens_per_local_expert_0.bin")
     drive(tmp_path, kernel, t, k, n, tmp_path, "--experts", e, "--iters", 1, "--warmup", 0)
     assert_close(bf16_file(tmp_path / "output_0.bin", (t, n)), orc.mx_gmm(pa, sa, pb, sb, n, k, fmt, 0, group_sizes=gs))
+
+
+@pytest.mark.parametrize("kernel,fmt", [("a5fp4gmmata", orc.E2M1), ("a5fp8gmmata", orc.E4M3)])
+def test_mx_grouped_down_projection_files(tmp_path, kernel, fmt):
+    """Down projection with two source ranks: rows arrive by (expert, rank) and leave by (rank, expert),
+    rank r's rows in region r of the output (file names of ascend950_fp8_mx_grouped_matmul_alltoallv_host.h)."""
+    ranks, e, t, k, n = 2, 4, 1024, 256, 256
+    rng = np.random.default_rng(6)
+    g = rng.multinomial(t - 24, np.ones(ranks * e) / (ranks * e)).reshape(ranks, e).astype(np.int32)
+    g[1, 2] = 0
+    gs = g.sum(axis=0).astype(np.int32)
+    used = int(gs.sum())
+    pa, sa = orc.mx_quant_rows(rand_bf16(rng, (t, k), 0.5), fmt)
+    pbs, sbs = zip(*[orc.mx_quant_b(rand_bf16(rng, (k, n), 0.5), fmt, orc.RNE, 0) for _ in range(e)])
+    pb, sb = np.stack(pbs), np.stack(sbs)
+    pa.tofile(tmp_path / "a_gm_0.bin"); pb.tofile(tmp_path / "b_gm_0.bin")
+    sa.tofile(tmp_path / "a_scale_0.bin"); sb.tofile(tmp_path / "b_scale_0.bin")
+    g.tofile(tmp_path / "global_tokens_per_local_expert_0.bin")
+    np.zeros(e, np.int32).tofile(tmp_path / "local_tokens_per_expert_0.bin")
+    drive(tmp_path, kernel, t, k, n, tmp_path, "--experts", e, "--ranks", ranks, "--iters", 1, "--warmup", 0)
+    gold = orc.mx_gmm(pa, sa, pb, sb, n, k, fmt, 0, group_sizes=gs)
+    want = orc.scatter_rows(gold[:used], orc.send_buffer_row_map(g, rank_rows=t), ranks * t, fill=np.float32(0))
+    assert_close(bf16_file(tmp_path / "output_0.bin", (ranks * t, n)), want)
