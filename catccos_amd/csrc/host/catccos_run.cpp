@@ -3,7 +3,7 @@
 //   registry -> CheckCocTilingParams -> AllocateDeviceSpace -> launcher (warm-up + timed loop)
 //   -> WriteResultFile -> FreeDeviceSpace.
 //
-//   catccos_run <kernel> <m> <k> <n> <data_dir|-> [--transB 0|1] [--experts E] [--rank R] [--ranks S]
+//   catccos_run <kernel> <m> <k> <n> <data_dir|-> [--transB 0|1] [--experts E] [--rank R] [--ranks S] [--topk T]
 //               [--warmup W] [--iters I]
 //   catccos_run --list            registry names and dispatch keys, no device needed
 // <kernel> is a short name of CommTypeMap (mxqtag, agmmdq, a5mxfp8mmrs, dgds, a5fp4mxatavgmm,
@@ -37,7 +37,7 @@ int main(int argc, char **argv)
         return 0;
     }
     if (argc < 6) {
-        ERROR_LOG("usage: %s <kernel> <m> <k> <n> <data_dir|-> [--transB 0|1] [--experts E] [--rank R] [--ranks S] [--warmup W] [--iters I]", argv[0]);
+        ERROR_LOG("usage: %s <kernel> <m> <k> <n> <data_dir|-> [--transB 0|1] [--experts E] [--rank R] [--ranks S] [--topk T] [--warmup W] [--iters I]", argv[0]);
         return -1;
     }
     const std::string kernelName = argv[1];
@@ -58,6 +58,7 @@ int main(int argc, char **argv)
         else if (key == "--experts") tiling.expertNum = val;
         else if (key == "--rank") rank = val;
         else if (key == "--ranks") tiling.rankSize = val ? val : 1;
+        else if (key == "--topk") tiling.topK = val ? val : 1;
         else if (key == "--warmup") warmup = val;
         else if (key == "--iters") iters = val;
         else { ERROR_LOG("unknown option %s", key.c_str()); return -1; }

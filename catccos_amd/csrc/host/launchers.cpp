@@ -40,6 +40,19 @@ void LaunchAscend950MxFp8MatmulReduceScatterFP8E4M3FN(void *stream, uint32_t, ui
 void LaunchDispatchGmmDequantSwigluINT8(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
                                         CocTilingParams &t, uint32_t, uint32_t transB)
 {
+    if (p.customCount >= 6) {
+        // from bf16 tokens: dynamic int8 quantisation with the expert-sorted gather, then the grouped matmul
+        const int64_t topK = t.topK ? t.topK : 1, rows = (int64_t)t.m * topK;
+        int rc = cch_dyn_quant_i8_rows(p.ptrA, reinterpret_cast<const int32_t *>(p.customPtrs[4]), p.customPtrs[5],
+                                       reinterpret_cast<float *>(p.customPtrs[2]), t.m, rows, t.k, (int)topK, CCH_DQ_DEVICE, stream);
+        if (rc == CCH_OK)
+            rc = cch_gmm_i8_dequant_swiglu(p.customPtrs[5], p.ptrB, reinterpret_cast<const int32_t *>(p.customPtrs[3]),
+                                           reinterpret_cast<const float *>(p.customPtrs[2]),
+                                           reinterpret_cast<const float *>(p.customPtrs[0]), p.ptrC, t.expertNum, rows, t.n, t.k,
+                                           (int)transB, stream);
+        Finish(rc, stream, "DispatchGmmDequantSwiglu");
+        return;
+    }
     Finish(cch_gmm_i8_dequant_swiglu(p.ptrA, p.ptrB, reinterpret_cast<const int32_t *>(p.customPtrs[1]),
                                      reinterpret_cast<const float *>(p.customPtrs[2]),
                                      reinterpret_cast<const float *>(p.customPtrs[0]), p.ptrC, t.expertNum, t.m, t.n, t.k,

@@ -161,43 +161,97 @@ public:
 
 // ---------------------------------------------------------------------------------------------
 // MoE grouped int8 matmul + dequant + SwiGLU (reference examples/dispatch_gmm_dequant_swiglu/
-// dispatch_gmm_dequant_swiglu_host.h:15-119).  The routing / dispatch stage is dropped: a_gm_<r>.bin
-// holds the int8 tokens this rank received, grouped by local expert ([m,k], m = rows received);
-// group_list_<r>.bin int32[expertNum] their counts; pertoken_scale_<r>.bin fp32[m].
-// ptrA = tokens, ptrB = W int8 [E,k,n] (transB: [E,n,k]), ptrC = out bf16 [m,n/2],
-// custom[0] = per-channel fp32 [E,n], custom[1] = group list, custom[2] = per-token fp32 [m].
+// dispatch_gmm_dequant_swiglu_host.h:15-119), two file sets:
+//  * the reference's own (expert_idx_<r>.bin present): a_gm_<r>.bin bf16 tokens [m,k], expert_idx_<r>.bin
+//    int32 [m,topK], scale_gm_<r>.bin per-channel scales as 64-bit fix-pipe words (low 32 bits = fp32,
+//    gen_data_dispatch_gmm_dequant_swiglu.py:75-76) or plain fp32.  The routing is done here on the host
+//    (stable sort of the flat expert indices, as moe_init_routing does), the dynamic int8 quantisation
+//    with the expert-sorted row gather and the grouped matmul on the device, over m * topK rows.
+//    ptrA = tokens, ptrB = W, ptrC = out bf16 [m*topK, n/2], custom[0] = per-channel fp32 [E,n],
+//    custom[1] = expert idx (as in the reference), then derived: custom[2] = per-token fp32 [m*topK],
+//    custom[3] = rows per expert, custom[4] = sorted expanded-row index [m*topK], custom[5] = int8 rows.
+//  * after the dispatch (no expert_idx file): a_gm_<r>.bin holds the int8 tokens this rank received,
+//    grouped by local expert ([m,k]); group_list_<r>.bin int32[expertNum] their counts;
+//    pertoken_scale_<r>.bin fp32[m].  ptrA = tokens, ptrB = W int8 [E,k,n] (transB: [E,n,k]),
+//    ptrC = out bf16 [m,n/2], custom[0] = per-channel fp32 [E,n], custom[1] = group list,
+//    custom[2] = per-token fp32 [m].
 class DispatchGmmDequantSwigluOperator : public CatccosOperator {
 public:
     void AllocateDeviceSpace(KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
     {
-        const size_t m = t.m, k = t.k, n = t.n, e = t.expertNum;
-        uint8_t *a = LoadOrFill(m * k, dataFile, "a_gm_" + R(rankId) + ".bin", 1);
+        const size_t m = t.m, k = t.k, n = t.n, e = t.expertNum, topK = t.topK ? t.topK : 1;
+        struct stat st;
+        const std::string idxFile = dataFile + "/expert_idx_" + R(rankId) + ".bin";
+        fromTokens_ = !dataFile.empty() && stat(idxFile.c_str(), &st) == 0;
         uint8_t *b = LoadOrFill(e * k * n, dataFile, "b_gm_" + R(rankId) + ".bin", 1);
+        std::vector<float> perCh(e * n, 1.0f);
+        if (!dataFile.empty()) {
+            std::vector<uint64_t> raw(e * n, 0);
+            size_t got = 0;
+            if (ReadFile(dataFile + "/scale_gm_" + R(rankId) + ".bin", raw.data(), e * n * 8, &got)) {
+                if (got == e * n * 8) {
+                    for (size_t i = 0; i < e * n; i++) {
+                        const uint32_t lo = static_cast<uint32_t>(raw[i]);
+                        memcpy(&perCh[i], &lo, 4);
+                    }
+                } else if (got == e * n * 4) {
+                    memcpy(perCh.data(), raw.data(), e * n * 4);
+                } else {
+                    ERROR_LOG("scale_gm_%u.bin has %zu bytes, expected %zu or %zu", rankId, got, e * n * 4, e * n * 8);
+                }
+            }
+        }
+        uint8_t *chDev = DeviceAlloc(e * n * 4);
+        CCH_CHECK(cch_memcpy_h2d(chDev, perCh.data(), e * n * 4));
+        if (fromTokens_) {
+            const size_t rows = m * topK;
+            uint8_t *x = LoadOrFill(m * k * 2, dataFile, "a_gm_" + R(rankId) + ".bin", 0);
+            std::vector<int32_t> expertIdx(rows, 0), groups(e, 0), sorted(rows, -1);
+            ReadFile(idxFile, expertIdx.data(), rows * 4);
+            // stable counting sort of the flat (token, route) list by expert: position -> flat index
+            for (size_t i = 0; i < rows; i++)
+                if (expertIdx[i] >= 0 && static_cast<size_t>(expertIdx[i]) < e) groups[expertIdx[i]]++;
+            std::vector<size_t> next(e, 0);
+            for (size_t i = 1; i < e; i++) next[i] = next[i - 1] + groups[i - 1];
+            for (size_t i = 0; i < rows; i++)
+                if (expertIdx[i] >= 0 && static_cast<size_t>(expertIdx[i]) < e) sorted[next[expertIdx[i]]++] = static_cast<int32_t>(i);
+            uint8_t *idxDev = DeviceAlloc(rows * 4), *tokDev = DeviceAlloc(rows * 4), *grpDev = DeviceAlloc(e * 4);
+            uint8_t *srcDev = DeviceAlloc(rows * 4), *q = DeviceAlloc(rows * k), *d = DeviceAlloc(rows * (n / 2) * 2);
+            CCH_CHECK(cch_memcpy_h2d(idxDev, expertIdx.data(), rows * 4));
+            CCH_CHECK(cch_memcpy_h2d(grpDev, groups.data(), e * 4));
+            CCH_CHECK(cch_memcpy_h2d(srcDev, sorted.data(), rows * 4));
+            params.SetKernelParams(x, b, d, chDev, idxDev, tokDev, grpDev, srcDev, q);
+            return;
+        }
+        uint8_t *a = LoadOrFill(m * k, dataFile, "a_gm_" + R(rankId) + ".bin", 1);
         uint8_t *d = DeviceAlloc(m * (n / 2) * 2);
-        std::vector<float> perCh(e * n, 1.0f), perTok(m, 1.0f);
+        std::vector<float> perTok(m, 1.0f);
         std::vector<int32_t> groups(e, 0);
         for (size_t i = 0; i < e; i++) groups[i] = static_cast<int32_t>(m / e + (i < m % e ? 1 : 0));
         if (!dataFile.empty()) {
-            ReadFile(dataFile + "/scale_gm_" + R(rankId) + ".bin", perCh.data(), e * n * 4);
             ReadFile(dataFile + "/pertoken_scale_" + R(rankId) + ".bin", perTok.data(), m * 4);
             ReadFile(dataFile + "/group_list_" + R(rankId) + ".bin", groups.data(), e * 4);
         }
-        uint8_t *chDev = DeviceAlloc(e * n * 4), *tokDev = DeviceAlloc(m * 4), *grpDev = DeviceAlloc(e * 4);
-        CCH_CHECK(cch_memcpy_h2d(chDev, perCh.data(), e * n * 4));
+        uint8_t *tokDev = DeviceAlloc(m * 4), *grpDev = DeviceAlloc(e * 4);
         CCH_CHECK(cch_memcpy_h2d(tokDev, perTok.data(), m * 4));
         CCH_CHECK(cch_memcpy_h2d(grpDev, groups.data(), e * 4));
         params.SetKernelParams(a, b, d, chDev, grpDev, tokDev);
     }
     void WriteResultFile(const KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
     {
-        DumpDevice(params.ptrC, static_cast<size_t>(t.m) * (t.n / 2) * 2, dataFile + "/output_" + R(rankId) + ".bin");
+        const size_t rows = static_cast<size_t>(t.m) * (fromTokens_ ? (t.topK ? t.topK : 1) : 1);
+        DumpDevice(params.ptrC, rows * (t.n / 2) * 2, dataFile + "/output_" + R(rankId) + ".bin");
     }
     size_t GetWorkspaceSize(const CocTilingParams &) override { return 0; }
     CocCommType GetActualKernelType(const CocTilingParams &) override { return DISPATCH_GMM_DEQUANT_SWIGLU; }
     bool CheckCocTilingParams(uint32_t, const CocTilingParams &t) override
     {
-        return t.m > 0 && t.k > 0 && t.n > 0 && t.n % 2 == 0 && t.expertNum > 0;
+        return t.m > 0 && t.k > 0 && t.n > 0 && t.n % 2 == 0 && t.expertNum > 0 &&
+               static_cast<uint64_t>(t.m) * (t.topK ? t.topK : 1) < (1ull << 31);
     }
+
+private:
+    bool fromTokens_ = false;
 };
 
 // ---------------------------------------------------------------------------------------------

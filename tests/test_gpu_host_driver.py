@@ -125,3 +125,31 @@ def test_mx_grouped_down_projection_files(tmp_path, kernel, fmt):
     gold = orc.mx_gmm(pa, sa, pb, sb, n, k, fmt, 0, group_sizes=gs)
     want = orc.scatter_rows(gold[:used], orc.send_buffer_row_map(g, rank_rows=t), ranks * t, fill=np.float32(0))
     assert_close(bf16_file(tmp_path / "output_0.bin", (ranks * t, n)), want)
+
+
+@pytest.mark.parametrize("words", [True, False])
+def test_dispatch_gmm_swiglu_from_bf16_tokens(tmp_path, words):
+    """The reference's own file set for this operator: bf16 tokens + expert_idx [m, topK] + per-channel
+    scales as 64-bit fix-pipe words (dispatch_gmm_dequant_swiglu_host.h:21-71).  Routing on the host,
+    dynamic int8 quantisation with the expert-sorted gather and the grouped matmul on the device."""
+    e, m, topk, k, n = 8, 300, 2, 512, 512
+    rng = np.random.default_rng(8)
+    xb = rand_bf16(rng, (m, k), 1.5)
+    expert_idx = rng.integers(0, e, (m, topk)).astype(np.int32)
+    expert_idx[expert_idx == 5] = 4                                   # an expert nobody routes to
+    w = rng.integers(-16, 16, (e, k, n)).astype(np.int8)
+    pc = rng.uniform(0.001, 0.02, (e, n)).astype(np.float32)
+    xb.tofile(tmp_path / "a_gm_0.bin"); w.tofile(tmp_path / "b_gm_0.bin"); expert_idx.tofile(tmp_path / "expert_idx_0.bin")
+    if words:
+        raw = np.zeros((e, n), np.uint64)
+        raw[:] = pc.view(np.uint32)
+        raw.tofile(tmp_path / "scale_gm_0.bin")
+    else:
+        pc.tofile(tmp_path / "scale_gm_0.bin")
+    drive(tmp_path, "dgds", m, k, n, tmp_path, "--experts", e, "--topk", topk, "--iters", 1, "--warmup", 0)
+    flat = expert_idx.reshape(-1)
+    order = np.argsort(flat, kind="stable").astype(np.int32)          # moe_init_routing: sorted position -> flat index
+    gs = np.bincount(flat, minlength=e).astype(np.int32)
+    q, s = orc.dyn_quant_i8_rows(xb, order, topk, orc.DQ_DEVICE)
+    want = orc.gmm_i8_dequant_swiglu(q, w, gs, s, pc)
+    assert_close(bf16_file(tmp_path / "output_0.bin", (m * topk, n // 2)), want)
