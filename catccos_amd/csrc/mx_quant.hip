@@ -14,7 +14,7 @@ namespace cch {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int QUANT_THREADS = 256;
+constexpr int QUANT_THREADS = 512;        // large workgroups: the dispatcher places 512 blocks of 256 threads noticeably slower
 #ifndef QUANT_UNROLL_V
 #define QUANT_UNROLL_V 2
 #endif

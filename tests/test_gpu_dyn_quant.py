@@ -19,7 +19,8 @@ def dev_bf16(bits):
 
 
 @pytest.mark.parametrize("mode", [cc.DQ_DEVICE, cc.DQ_GOLDEN])
-@pytest.mark.parametrize("shape", [(64, 512), (300, 7168), (17, 1000), (5, 8200), (3, 12288), (9, 8), (2, 7)])
+@pytest.mark.parametrize("shape", [(64, 512), (300, 7168), (17, 1000), (5, 8200), (3, 12288), (9, 8), (2, 7),
+                                   (10, 4096), (7, 3000), (5, 2048), (3, 16384), (2, 20000), (1, 7168)])
 def test_dyn_quant_bit_exact(shape, mode):
     rows, k = shape
     rng = np.random.default_rng(rows * 131 + k + mode)
