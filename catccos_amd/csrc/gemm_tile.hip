@@ -231,7 +231,9 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     const uint32_t sb_sel = (r & 1) ? 0x07060302u : 0x05040100u;   // TB = 0: which half of the dwords holds this column
     // TB = 0 fragment reads: lane (q = lane / 16, i = lane % 16) addresses K-row 16*(q/2) + i/2 of
     // the substep part and the 8-byte half (i & 1) of 16-byte chunk wn*4 + j*2 + (q & 1), whose
-    // position in the row is swizzled by the row's low bits (i / 2)
+    // position in the row is swizzled by twice the row's low bits (i / 2): the 32 lanes of one pass
+    // of the load address 8 K-rows x 2 neighbouring chunks, and chunk ^ 2*(row & 7) puts those 16
+    // pieces on 16 different chunk positions of the 256-byte row, i.e. on all 64 banks once
     // For FP4 the panel has 256 K-rows of 128 bytes (two columns per byte) and the 4-bit form of
     // the load is a 16 x 16 nibble transpose: lane i addresses K-row i at 16 columns (8 bytes) and
     // lane j receives 16 consecutive K nibbles of column j; the chunk swizzle uses row bits 1..3.
@@ -244,7 +246,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     const uint32_t rd_bt = FP4K ? (uint32_t)PANEL_BYTES + (uint32_t)(32 * (tq >> 1) + ti) * 128u +
                                       ((uint32_t)((wn * 2) ^ (ti >> 1)) << 4) + (uint32_t)(tq & 1) * 8u
                                 : (uint32_t)PANEL_BYTES + (uint32_t)(16 * (tq >> 1) + (ti >> 1)) * 256u +
-                                      ((uint32_t)((wn * 4 + (tq & 1)) ^ (ti >> 1)) << 4) + (uint32_t)(ti & 1) * 8u;
+                                      ((uint32_t)((wn * 4 + (tq & 1)) ^ ((ti >> 1) << 1)) << 4) + (uint32_t)(ti & 1) * 8u;
     const int ldb = TB ? lda : p.N / EPB;   // bytes between consecutive rows of B as stored
     // Rows that belong to no group are written as zeros (the reference's golden pads them,
     // examples/utils/gen_data_fp4_mx_alltoallv_gmm.py:788-790): all workgroups share the range,
@@ -296,9 +298,9 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             } else {
                 // Instruction j fills K-rows (wave*NJ + j)*4 .. +3 of the panel, 256 bytes each;
                 // lane l lands at row l/16, chunk position l%16 and fetches tile chunk
-                // (l%16) ^ (row & 7): 16 tile columns, clamped to stay inside the row of B.
+                // (l%16) ^ 2*(row & 7): 16 tile columns, clamped to stay inside the row of B.
                 const int kr = (wave * NJ + j) * BRPI + lane / BCPR;
-                const int tc = (lane % BCPR) ^ (FP4K ? (kr >> 1) & 7 : kr & 7);
+                const int tc = (lane % BCPR) ^ (FP4K ? (kr >> 1) & 7 : (kr & 7) << 1);
                 constexpr int CPC = 16 * EPB;  // columns per chunk
                 int col;
                 if (SWIGLU) col = ((tc >> 1) & 1) * p.n_out + min(c.j0 + (tc >> 2) * 32 + (tc & 1) * 16, p.n_out - 16);
