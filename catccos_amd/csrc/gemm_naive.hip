@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void gemm_naive_kernel(GemmProblem p)
     size_t out_row = (size_t)row;
     if (p.out_row_map) {
         // mapped output: rows of no group and rows mapped to a negative index are not written
-        if (e >= p.num_groups || p.out_row_map[row] < 0) return;
+        if (e >= p.num_groups || p.out_row_map[row] < 0 || p.out_row_map[row] >= p.out_rows) return;
         out_row = (size_t)p.out_row_map[row];
     }
     float v = 0.0f;

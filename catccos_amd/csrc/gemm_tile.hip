@@ -679,7 +679,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                     uint32_t out_row = (uint32_t)row;
                     if constexpr (EPI == EPI_PLAIN) {
                         const int mapped = (int)lds_read4(prm + (uint32_t)row * 4u);
-                        ok = ok && (!has_map || mapped >= 0);
+                        ok = ok && (!has_map || (mapped >= 0 && mapped < (int)p.out_rows));   // dropped or out of range: not written
                         out_row = has_map ? (uint32_t)mapped : out_row;
                     }
                     const uint32_t off = ok ? (out_row * (uint32_t)p.n_out + (uint32_t)col) * 2u : 0xFFFFFFF0u;

@@ -134,7 +134,8 @@ int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, con
  * LaunchAscend950Fp8MxGroupedMatmulAllToAllVFP16, tests/dynamic_tiling/impl/kernel_fp16_ascend950.cpp:446):
  * the result rows leave in the order of the send buffer (by destination rank, then expert) instead of
  * the order of the tokens (by expert, then source rank).  Operands as cch_mx_gmm, plus
- *   out_row_map  int32 [t]: row of `out` that receives the result of row i of a; negative = dropped.
+ *   out_row_map  int32 [t]: row of `out` that receives the result of row i of a; negative or
+ *                >= out_rows = dropped.
  *                Entries of rows past sum(group_sizes) are ignored (those rows produce nothing).
  *   out          bf16 [out_rows, n]; rows that the map does not name are not written
  * Destination rows must be distinct. */

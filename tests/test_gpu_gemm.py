@@ -263,6 +263,7 @@ def test_mx_gmm_mapped_rows(fmt, trans_b, tiled):
     row_map = np.full(t, -1, np.int32)
     row_map[:used] = orc.send_buffer_row_map(g, rank_rows)
     row_map[7] = -1                                              # a dropped row
+    row_map[9] = ranks * rank_rows + 3                           # past the end of out: dropped as well
     sigma = 0.02 if fmt == "e2m1" else 1.0
     pa, sa = orc.mx_quant_rows(rand_bf16(rng, (t, k), sigma), FMT[fmt])
     pbs, sbs = [], []
@@ -272,7 +273,8 @@ def test_mx_gmm_mapped_rows(fmt, trans_b, tiled):
         sbs.append(sb)
     pb, sb = np.stack(pbs), np.stack(sbs)
     gold = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], trans_b, group_sizes=gs)
-    want = orc.scatter_rows(gold[:used], row_map[:used], ranks * rank_rows, fill=np.float32(-3.0))
+    kept = np.where(row_map[:used] < ranks * rank_rows, row_map[:used], -1)
+    want = orc.scatter_rows(gold[:used], kept, ranks * rank_rows, fill=np.float32(-3.0))
     cc.set_option("require_tiled_gemm", 1 if tiled else 0)
     cc.set_option("force_generic_gemm", 0 if tiled else 1)
     try:
@@ -283,6 +285,6 @@ def test_mx_gmm_mapped_rows(fmt, trans_b, tiled):
         cc.set_option("require_tiled_gemm", 0)
         cc.set_option("force_generic_gemm", 0)
     untouched = np.ones(ranks * rank_rows, bool)
-    untouched[row_map[:used][row_map[:used] >= 0]] = False
+    untouched[kept[kept >= 0]] = False
     assert (got[untouched] == -3.0).all()
     assert_close(got[~untouched], want[~untouched], ("mx gmm mapped", fmt, trans_b, tiled))
