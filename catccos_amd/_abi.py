@@ -40,7 +40,7 @@ PROTOTYPES = {
     "cch_gmm_i8_dequant_swiglu": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _P],
     "cch_mx_gemm": [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I, _I, _P],
     "cch_mx_gmm": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _I, _P],
-    "cch_mx_gmm_mapped": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I, _I, _P],
+    "cch_mx_gmm_mapped": [_P, _P, _P, _P, _P, _P, _P, _I64, _I, _I64, _I64, _I64, _I64, _I, _I, _P],
     "cch_set_option": [c.c_char_p, _I],
 }
 _RESTYPE = {"cch_last_error": c.c_char_p}

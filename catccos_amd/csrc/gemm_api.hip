@@ -145,18 +145,20 @@ int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, con
 }
 
 int cch_mx_gmm_mapped(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes,
-                      const int32_t *out_row_map, void *out, int64_t out_rows, int64_t num_experts, int64_t t, int64_t n,
-                      int64_t k, int fmt, int trans_b, void *stream)
+                      const int32_t *out_row_map, void *out, int64_t out_rows, int out_dtype, int64_t num_experts, int64_t t,
+                      int64_t n, int64_t k, int fmt, int trans_b, void *stream)
 {
     GemmProblem p{};
     int kind = 0;
     CCH_REQUIRE(group_sizes != nullptr || t == 0, "cch_mx_gmm_mapped: null group_sizes");
     CCH_REQUIRE(out_row_map != nullptr || t == 0, "cch_mx_gmm_mapped: null out_row_map");
     CCH_REQUIRE(out_rows >= 0 && out_rows < ((int64_t)1 << 31), "cch_mx_gmm_mapped: out_rows=%lld", (long long)out_rows);
+    CCH_REQUIRE(out_dtype == CCH_OUT_BF16 || out_dtype == CCH_OUT_FP16, "cch_mx_gmm_mapped: out_dtype %d", out_dtype);
     int rc = mx_problem("cch_mx_gmm_mapped", p, a, sa, b, sb, group_sizes, out, num_experts, t, n, k, fmt, trans_b, &kind);
     if (rc) return rc;
     p.out_row_map = out_row_map;
     p.out_rows = out_rows;
+    p.out_fp16 = out_dtype == CCH_OUT_FP16;
     return run(p, kind, EPI_PLAIN, static_cast<hipStream_t>(stream));
 }
 

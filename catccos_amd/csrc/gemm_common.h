@@ -24,6 +24,7 @@ struct GemmProblem {
     uint16_t *out;           // bf16 [T, n_out] (with out_row_map: [out_rows, n_out])
     const int32_t *out_row_map;  // device int32[T] or nullptr: row of `out` that receives row i (negative: dropped)
     int64_t out_rows;        // rows of `out` when out_row_map is given
+    int out_fp16;            // output elements are IEEE half instead of bf16 (both rounded to nearest even)
     const int32_t *group_sizes;  // device int32[E] or nullptr (dense, E = 1)
     int num_groups;
     int T, N, K;             // K in elements

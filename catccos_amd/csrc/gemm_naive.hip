@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void gemm_naive_kernel(GemmProblem p)
             v = dot_column<KIND>(p, row, e, col);
         }
     }
-    p.out[out_row * p.n_out + col] = (uint16_t)f32_to_bf16_bits(v);
+    p.out[out_row * p.n_out + col] = p.out_fp16 ? __builtin_bit_cast(uint16_t, (_Float16)v) : (uint16_t)f32_to_bf16_bits(v);
 }
 
 template <int KIND, int EPI>

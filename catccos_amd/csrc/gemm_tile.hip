@@ -46,6 +46,7 @@ typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int BM = 256, BN = 256;        // output tile
 constexpr int BKB = 128;                 // bytes of K per step (per row) = one L2 line
@@ -663,7 +664,9 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                                 // hardware RNE to bf16, both rows in one dword; then the neighbour's dword
                                 // and one byte permute: even lanes keep the low halves (row x), odd lanes
                                 // the high halves (row x+1), own column in its place
-                                const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){v[0], v[1]}, bf16x2));
+                                const uint32_t pk_bf = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){v[0], v[1]}, bf16x2));
+                                const uint32_t pk_h = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){v[0], v[1]}, f16x2));
+                                const uint32_t pk = p.out_fp16 ? pk_h : pk_bf;   // wave-uniform choice of the output type
                                 const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, true);
                                 const uint32_t packed = __builtin_amdgcn_perm(nb, pk, odd ? 0x03020706u : 0x05040100u);
                                 const int lrow = qq * 8 + g * 4 + xr + (odd ? 1 : 0);

@@ -3,7 +3,7 @@
 //   registry -> CheckCocTilingParams -> AllocateDeviceSpace -> launcher (warm-up + timed loop)
 //   -> WriteResultFile -> FreeDeviceSpace.
 //
-//   catccos_run <kernel> <m> <k> <n> <data_dir|-> [--transB 0|1] [--experts E] [--rank R] [--ranks S] [--topk T]
+//   catccos_run <kernel> <m> <k> <n> <data_dir|-> [--transB 0|1] [--experts E] [--rank R] [--ranks S] [--topk T] [--fp16 0|1]
 //               [--warmup W] [--iters I]
 //   catccos_run --list            registry names and dispatch keys, no device needed
 // <kernel> is a short name of CommTypeMap (mxqtag, agmmdq, a5mxfp8mmrs, dgds, a5fp4mxatavgmm,
@@ -37,7 +37,7 @@ int main(int argc, char **argv)
         return 0;
     }
     if (argc < 6) {
-        ERROR_LOG("usage: %s <kernel> <m> <k> <n> <data_dir|-> [--transB 0|1] [--experts E] [--rank R] [--ranks S] [--topk T] [--warmup W] [--iters I]", argv[0]);
+        ERROR_LOG("usage: %s <kernel> <m> <k> <n> <data_dir|-> [--transB 0|1] [--experts E] [--rank R] [--ranks S] [--topk T] [--fp16 0|1] [--warmup W] [--iters I]", argv[0]);
         return -1;
     }
     const std::string kernelName = argv[1];
@@ -50,7 +50,7 @@ int main(int argc, char **argv)
     tiling.rankSize = 1;
     tiling.epSize = 1;
     tiling.expertNum = 1;
-    uint32_t rank = 0, warmup = WARM_UP_TIMES, iters = PERF_TEST_CYCLE_TIMES;
+    uint32_t rank = 0, warmup = WARM_UP_TIMES, iters = PERF_TEST_CYCLE_TIMES, fp16Out = 0;
     for (int i = 6; i + 1 < argc; i += 2) {
         const std::string key = argv[i];
         const uint32_t val = (uint32_t)atoll(argv[i + 1]);
@@ -59,6 +59,7 @@ int main(int argc, char **argv)
         else if (key == "--rank") rank = val;
         else if (key == "--ranks") tiling.rankSize = val ? val : 1;
         else if (key == "--topk") tiling.topK = val ? val : 1;
+        else if (key == "--fp16") fp16Out = val;
         else if (key == "--warmup") warmup = val;
         else if (key == "--iters") iters = val;
         else { ERROR_LOG("unknown option %s", key.c_str()); return -1; }
@@ -89,7 +90,8 @@ int main(int argc, char **argv)
     KernelParams params;
     op->AllocateDeviceSpace(params, tiling, rank, dataDir);
     const CocCommType actual = op->GetActualKernelType(tiling);
-    KernelFuncPtr fn = KernelDispatcher::GetKernelFunc(actual, DataTypeOf(actual));
+    // --fp16 1 asks for the half-precision launcher of an operator that has one
+    KernelFuncPtr fn = KernelDispatcher::GetKernelFunc(actual, fp16Out ? FP16 : DataTypeOf(actual));
     if (!fn) {
         ERROR_LOG("no launcher for kernel type %d", (int)actual);
         return -1;

@@ -76,28 +76,41 @@ void LaunchAscend950Fp8MxAllToAllVGroupedMatmulBF16(void *stream, uint32_t, uint
            stream, "Ascend950Fp8MxAllToAllVGroupedMatmul");
 }
 
-// Down projection: the reference's launchers for these two operators are registered for fp16 output
-// (tests/dynamic_tiling/impl/kernel_fp16_ascend950.cpp:446-485, launch_map.h:98-99); this build
-// writes bf16 and registers them accordingly.
-static void MxGroupedMatmulAllToAllV(void *stream, KernelParams &p, CocTilingParams &t, uint32_t transB, int fmt, const char *what)
+// Down projection.  The reference registers these two operators for fp16 output only
+// (tests/dynamic_tiling/impl/kernel_fp16_ascend950.cpp:446-485, launch_map.h:98-99); this build has
+// that launcher and a bf16 twin, which the driver uses by default like for every other operator.
+static void MxGroupedMatmulAllToAllV(void *stream, KernelParams &p, CocTilingParams &t, uint32_t transB, int fmt, int outDtype,
+                                     const char *what)
 {
     const int64_t ranks = t.rankSize ? t.rankSize : 1, experts = t.expertNum / (t.epSize ? t.epSize : 1);
     Finish(cch_mx_gmm_mapped(p.ptrA, p.customPtrs[0], p.ptrB, p.customPtrs[1], reinterpret_cast<const int32_t *>(p.customPtrs[4]),
-                             reinterpret_cast<const int32_t *>(p.customPtrs[5]), p.ptrC, ranks * t.m, experts, t.m, t.n, t.k, fmt,
-                             (int)transB, stream),
+                             reinterpret_cast<const int32_t *>(p.customPtrs[5]), p.ptrC, ranks * t.m, outDtype, experts, t.m, t.n,
+                             t.k, fmt, (int)transB, stream),
            stream, what);
 }
 
 void LaunchAscend950Fp8MxGroupedMatmulAllToAllVBF16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
                                                     CocTilingParams &t, uint32_t, uint32_t transB)
 {
-    MxGroupedMatmulAllToAllV(stream, p, t, transB, CCH_FMT_E4M3, "Ascend950Fp8MxGroupedMatmulAllToAllV");
+    MxGroupedMatmulAllToAllV(stream, p, t, transB, CCH_FMT_E4M3, CCH_OUT_BF16, "Ascend950Fp8MxGroupedMatmulAllToAllV");
 }
 
 void LaunchAscend950Fp4MxGroupedMatmulAllToAllVBF16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
                                                     CocTilingParams &t, uint32_t, uint32_t transB)
 {
-    MxGroupedMatmulAllToAllV(stream, p, t, transB, CCH_FMT_E2M1, "Ascend950Fp4MxGroupedMatmulAllToAllV");
+    MxGroupedMatmulAllToAllV(stream, p, t, transB, CCH_FMT_E2M1, CCH_OUT_BF16, "Ascend950Fp4MxGroupedMatmulAllToAllV");
+}
+
+void LaunchAscend950Fp8MxGroupedMatmulAllToAllVFP16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
+                                                    CocTilingParams &t, uint32_t, uint32_t transB)
+{
+    MxGroupedMatmulAllToAllV(stream, p, t, transB, CCH_FMT_E4M3, CCH_OUT_FP16, "Ascend950Fp8MxGroupedMatmulAllToAllV");
+}
+
+void LaunchAscend950Fp4MxGroupedMatmulAllToAllVFP16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
+                                                    CocTilingParams &t, uint32_t, uint32_t transB)
+{
+    MxGroupedMatmulAllToAllV(stream, p, t, transB, CCH_FMT_E2M1, CCH_OUT_FP16, "Ascend950Fp4MxGroupedMatmulAllToAllV");
 }
 
 static AutoRegister s_reg0(MX_QUANT_ALLGATHER, FP8E4M3FN, &LaunchAscend950BF16QuantAllGatherFP8E4M3FN);
@@ -108,3 +121,5 @@ static AutoRegister s_reg4(ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL, BF16, &Lau
 static AutoRegister s_reg5(ASCEND950_FP8_MX_ALLTOALLV_GROUPED_MATMUL, BF16, &LaunchAscend950Fp8MxAllToAllVGroupedMatmulBF16);
 static AutoRegister s_reg6(ASCEND950_FP8_MX_GROUPED_MATMUL_ALLTOALLV, BF16, &LaunchAscend950Fp8MxGroupedMatmulAllToAllVBF16);
 static AutoRegister s_reg7(ASCEND950_FP4_MX_GROUPED_MATMUL_ALLTOALLV, BF16, &LaunchAscend950Fp4MxGroupedMatmulAllToAllVBF16);
+static AutoRegister s_reg8(ASCEND950_FP8_MX_GROUPED_MATMUL_ALLTOALLV, FP16, &LaunchAscend950Fp8MxGroupedMatmulAllToAllVFP16);
+static AutoRegister s_reg9(ASCEND950_FP4_MX_GROUPED_MATMUL_ALLTOALLV, FP16, &LaunchAscend950Fp4MxGroupedMatmulAllToAllVFP16);

@@ -304,7 +304,8 @@ using Ascend950Fp8MxAllToAllVGroupedMatmulOperator = MxAllToAllVGroupedMatmulOpe
 // rank), custom[3] = global_tokens_per_local_expert int32 [rankSize, E].  Derived here, as the
 // reference's scheduler derives them on the device (block_scheduler_reducescatter_alltoallv.hpp:
 // 211-256): custom[4] = rows per expert, custom[5] = destination row of every row of A.
-// The reference registers this operator for fp16 output; this build's GEMM epilogue writes bf16.
+// The output is bf16 or, through the FP16 launchers (the type the reference registers this operator
+// for), IEEE half; both are two bytes per element.
 template <bool FP4, CocCommType KIND> class MxGroupedMatmulAllToAllVOperator : public CatccosOperator {
 public:
     void AllocateDeviceSpace(KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override

@@ -274,7 +274,7 @@ def mx_grouped_matmul(a, sa, b, sb, group_sizes, fmt="e4m3", trans_b=0):
 def mx_grouped_matmul_mapped(a, sa, b, sb, group_sizes, out_row_map, out, fmt="e4m3", trans_b=0):
     """MX grouped GEMM whose result row i is written to out[out_row_map[i]] (entries that are negative
     or past the end of `out` are dropped; rows of `out` that the map does not name keep their contents).  `out` is a contiguous
-    bf16 [rows, N] tensor supplied by the caller; returns it."""
+    bfloat16 or float16 [rows, N] tensor supplied by the caller (its dtype selects the output type); returns it."""
     _require_gpu(a, sa, b, sb, group_sizes, out_row_map, out)
     if group_sizes.dtype != torch.int32 or group_sizes.dim() != 1:
         raise ValueError("group_sizes must be a 1-D int32 tensor")
@@ -284,8 +284,9 @@ def mx_grouped_matmul_mapped(a, sa, b, sb, group_sizes, out_row_map, out, fmt="e
         raise ValueError("group_sizes must have one entry per expert")
     if out_row_map.dtype != torch.int32 or out_row_map.numel() != t:
         raise ValueError("out_row_map must hold one int32 entry per row of a")
-    if out.dim() != 2 or out.dtype != torch.bfloat16 or out.shape[1] != n or not out.is_contiguous():
-        raise ValueError("out must be a contiguous bfloat16 [rows, %d] tensor" % n)
+    if out.dim() != 2 or out.dtype not in (torch.bfloat16, torch.float16) or out.shape[1] != n or not out.is_contiguous():
+        raise ValueError("out must be a contiguous bfloat16 or float16 [rows, %d] tensor" % n)
     check(_abi.lib().cch_mx_gmm_mapped(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(group_sizes), _ptr(out_row_map.contiguous()),
-                                       _ptr(out), out.shape[0], e, t, n, k, fmt, int(trans_b), _stream()))
+                                       _ptr(out), out.shape[0], 1 if out.dtype == torch.float16 else 0, e, t, n, k, fmt,
+                                       int(trans_b), _stream()))
     return out

@@ -137,11 +137,15 @@ int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, con
  *   out_row_map  int32 [t]: row of `out` that receives the result of row i of a; negative or
  *                >= out_rows = dropped.
  *                Entries of rows past sum(group_sizes) are ignored (those rows produce nothing).
- *   out          bf16 [out_rows, n]; rows that the map does not name are not written
+ *   out          [out_rows, n] of out_dtype; rows that the map does not name are not written
+ *   out_dtype    CCH_OUT_BF16, or CCH_OUT_FP16 (IEEE half, the type the reference registers these
+ *                operators for); fp32 accumulators are rounded to nearest even either way
  * Destination rows must be distinct. */
+#define CCH_OUT_BF16 0
+#define CCH_OUT_FP16 1
 int cch_mx_gmm_mapped(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes,
-                      const int32_t *out_row_map, void *out, int64_t out_rows, int64_t num_experts, int64_t t, int64_t n,
-                      int64_t k, int fmt, int trans_b, void *stream);
+                      const int32_t *out_row_map, void *out, int64_t out_rows, int out_dtype, int64_t num_experts, int64_t t,
+                      int64_t n, int64_t k, int fmt, int trans_b, void *stream);
 
 /* ---- MX quantisation scattered to the routed rows, packed (dispatch side of the MoE path) ----
  * Replaces CommBlockMxQuant::QuantScatterPacked (include/catccos/comm/block/

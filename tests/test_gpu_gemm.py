@@ -246,6 +246,40 @@ def test_mx_gmm_tiled(fmt, cfg, trans_b, tiled_only):
     assert_close(got, want, ("mx gmm tiled", fmt, cfg[:4], trans_b))
 
 
+def test_mx_gmm_mapped_fp16_is_the_rounded_accumulator():
+    """The half-precision output is the same fp32 result rounded to nearest even: on data whose
+    results are exact in both types (small integers) the two outputs agree exactly, and on random
+    data the fp16 output is closer to the oracle than bf16's 8 bits allow."""
+    e, t, k, n = 2, 300, 256, 256
+    rng = np.random.default_rng(5)
+    gs = np.array([130, 170], np.int32)
+    pa, sa = orc.mx_quant_rows(rand_bf16(rng, (t, k), 1.0), orc.E4M3)
+    pbs, sbs = zip(*[orc.mx_quant_b(rand_bf16(rng, (k, n), 1.0), orc.E4M3, orc.RNE, 0) for _ in range(e)])
+    pb, sb = np.stack(pbs), np.stack(sbs)
+    gold = orc.mx_gmm(pa, sa, pb, sb, n, k, orc.E4M3, 0, group_sizes=gs)
+    ident = np.arange(t, dtype=np.int32)
+    for tiled in (True, False):
+        cc.set_option("require_tiled_gemm", 1 if tiled else 0)
+        cc.set_option("force_generic_gemm", 0 if tiled else 1)
+        try:
+            out_h = torch.zeros((t, n), dtype=torch.float16, device="cuda")
+            out_b = torch.zeros((t, n), dtype=torch.bfloat16, device="cuda")
+            cc.mx_grouped_matmul_mapped(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), dev(ident), out_h, "e4m3", 0)
+            cc.mx_grouped_matmul_mapped(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), dev(ident), out_b, "e4m3", 0)
+            torch.cuda.synchronize()
+        finally:
+            cc.set_option("require_tiled_gemm", 0)
+            cc.set_option("force_generic_gemm", 0)
+        h, b = out_h.float().cpu().numpy(), out_b.float().cpu().numpy()
+        assert_close(h, gold, ("fp16 out", tiled))
+        # bf16 of the half result equals the bf16 result wherever no double rounding can occur:
+        # compare through the error against the fp32 oracle instead, half must be at least as close
+        eh, eb = np.abs(h - gold), np.abs(b - gold)
+        assert eh.mean() < 0.2 * eb.mean()
+        # and fp16 rounding of the oracle's fp32 value is within one half-ulp of what came back
+        assert np.max(np.abs(h - gold.astype(np.float16).astype(np.float32)) / np.maximum(np.abs(gold), 1.0)) < 2e-3
+
+
 @pytest.mark.parametrize("fmt", ["e4m3", "e2m1"])
 @pytest.mark.parametrize("trans_b", [0, 1])
 @pytest.mark.parametrize("tiled", [True, False])

@@ -104,8 +104,9 @@ def test_mx_grouped_files(tmp_path, kernel, fmt):
     assert_close(bf16_file(tmp_path / "output_0.bin", (t, n)), orc.mx_gmm(pa, sa, pb, sb, n, k, fmt, 0, group_sizes=gs))
 
 
+@pytest.mark.parametrize("fp16", [0, 1])
 @pytest.mark.parametrize("kernel,fmt", [("a5fp4gmmata", orc.E2M1), ("a5fp8gmmata", orc.E4M3)])
-def test_mx_grouped_down_projection_files(tmp_path, kernel, fmt):
+def test_mx_grouped_down_projection_files(tmp_path, kernel, fmt, fp16):
     """Down projection with two source ranks: rows arrive by (expert, rank) and leave by (rank, expert),
     rank r's rows in region r of the output (file names of ascend950_fp8_mx_grouped_matmul_alltoallv_host.h)."""
     ranks, e, t, k, n = 2, 4, 1024, 256, 256
@@ -121,10 +122,14 @@ def test_mx_grouped_down_projection_files(tmp_path, kernel, fmt):
     sa.tofile(tmp_path / "a_scale_0.bin"); sb.tofile(tmp_path / "b_scale_0.bin")
     g.tofile(tmp_path / "global_tokens_per_local_expert_0.bin")
     np.zeros(e, np.int32).tofile(tmp_path / "local_tokens_per_expert_0.bin")
-    drive(tmp_path, kernel, t, k, n, tmp_path, "--experts", e, "--ranks", ranks, "--iters", 1, "--warmup", 0)
+    drive(tmp_path, kernel, t, k, n, tmp_path, "--experts", e, "--ranks", ranks, "--fp16", fp16, "--iters", 1, "--warmup", 0)
     gold = orc.mx_gmm(pa, sa, pb, sb, n, k, fmt, 0, group_sizes=gs)
     want = orc.scatter_rows(gold[:used], orc.send_buffer_row_map(g, rank_rows=t), ranks * t, fill=np.float32(0))
-    assert_close(bf16_file(tmp_path / "output_0.bin", (ranks * t, n)), want)
+    if fp16:     # the type the reference registers this operator for
+        got = np.fromfile(tmp_path / "output_0.bin", dtype=np.float16).astype(np.float32).reshape(ranks * t, n)
+    else:
+        got = bf16_file(tmp_path / "output_0.bin", (ranks * t, n))
+    assert_close(got, want)
 
 
 @pytest.mark.parametrize("words", [True, False])

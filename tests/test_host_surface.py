@@ -16,7 +16,7 @@ EXPECT = {
     "a5fp4mxatavgmm": ("Ascend950Fp4MxAllToAllVGroupedMatmul", 28, 27),
     "a5fp8mxatavgmm": ("Ascend950Fp8MxAllToAllVGroupedMatmul", 27, 27),
     # down projection: the reference registers these two for fp16 output (launch_map.h:98-99);
-    # this build writes bf16 and registers them under BF16
+    # this build has those launchers (keys (25 << 8) | 1, (26 << 8) | 1) and bf16 twins, which --list shows
     "a5fp8gmmata": ("Ascend950Fp8MxGroupedMatmulAllToAllV", 25, 27),
     "a5fp4gmmata": ("Ascend950Fp4MxGroupedMatmulAllToAllV", 26, 27),
 }
