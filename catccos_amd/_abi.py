@@ -10,7 +10,7 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "libcatccos_hip.so")
 
 OK, EINVAL, EHIP, ENODEV, ENOSUP = 0, -1, -2, -3, -4
-FMT_E4M3, FMT_E5M2, FMT_E2M1 = 0, 1, 2
+FMT_E4M3, FMT_E5M2, FMT_E2M1, FMT_E1M2 = 0, 1, 2, 3
 ROUND_RNE, ROUND_LUT = 0, 1
 
 c = ctypes

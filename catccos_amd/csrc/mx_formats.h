@@ -1,4 +1,4 @@
-// Device-side number formats of the MX path: bf16, E4M3 / E5M2 / E2M1 payload codes,
+// Device-side number formats of the MX path: bf16, E4M3 / E5M2 / E2M1 / E1M2 payload codes,
 // E8M0 block scales.  Arithmetic is integer-exact so that results are bit-identical
 // to the CPU golden of the reference (examples/utils/gen_mx_quant_allgather_data.py).
 #pragma once
@@ -26,6 +26,15 @@ template <> struct FmtTraits<CCH_FMT_E2M1> {
     static constexpr float MAXV = 6.0f;
     static constexpr uint32_t SIGN = 0x8u, NANCODE = 0x7u;
 };
+
+// E1M2 (examples/utils/gen_mx_quant_allgather_data.py:65-72): subnormals m/4, normals 1 + m/4.
+template <> struct FmtTraits<CCH_FMT_E1M2> {
+    static constexpr int MB = 2, BIAS = 1, EMAX = 0;
+    static constexpr float MAXV = 1.75f;
+    static constexpr uint32_t SIGN = 0x8u, NANCODE = 0x7u;
+};
+// The two 4-bit formats share the packing: two codes per byte, element 2j in the low nibble.
+template <int FMT> constexpr bool is_fp4_v = FMT == CCH_FMT_E2M1 || FMT == CCH_FMT_E1M2;
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 

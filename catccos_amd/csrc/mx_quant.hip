@@ -1,4 +1,4 @@
-// MX block quantiser: bf16 -> FP8 (E4M3/E5M2) or FP4 (E2M1) payload + one E8M0 scale per
+// MX block quantiser: bf16 -> FP8 (E4M3/E5M2) or FP4 (E2M1/E1M2) payload + one E8M0 scale per
 // 32 elements.  Streaming, HBM-bound kernel: every lane owns 8 consecutive elements (one
 // 16-byte load), four neighbouring lanes own one MX block and reduce its maximum with two
 // DPP quad permutes; payload leaves as one 8-byte (FP8) or 4-byte (FP4) store per lane.
@@ -33,14 +33,16 @@ template <int FMT, int RND>
 __device__ __forceinline__ void quant8_soft(const uint32_t (&w)[4], int e, bool is_nan, uint32_t (&out)[2])
 {
     using T = FmtTraits<FMT>;
-    const float inv = pow2i(-e);
+    // 2^-e in two exact factors: 2^-127 (a format whose largest exponent is 0 meets a block
+    // maximum of 2^127) is no normal float
+    const float inv = pow2i(-min(e, 126)), inv2 = e > 126 ? 0.5f : 1.0f;
     float y[8];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        y[2 * i] = __uint_as_float(w[i] << 16) * inv;
-        y[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u) * inv;
+        y[2 * i] = __uint_as_float(w[i] << 16) * inv * inv2;
+        y[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u) * inv * inv2;
     }
-    if constexpr (FMT == CCH_FMT_E2M1) {
+    if constexpr (is_fp4_v<FMT>) {
         uint32_t r = 0;
 #pragma unroll
         for (int i = 0; i < 8; i++) r |= (is_nan ? T::NANCODE : encode_small<FMT, RND>(y[i])) << (4 * i);
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
 {
     static_assert(!(SCATTER && PAIR), "the scatter variant stores one wave-step at a time");
     if (!SCATTER) sstride = sld;
-    constexpr bool FP4 = FMT == CCH_FMT_E2M1;
+    constexpr bool FP4 = is_fp4_v<FMT>;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (QUANT_THREADS / 64) + (threadIdx.x >> 6)));
     const int stride = (int)gridDim.x * (QUANT_THREADS / 64) * QUANT_UNROLL;
@@ -312,7 +314,7 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_fast_kernel(
     const uint16_t *__restrict__ x, uint8_t *__restrict__ payload, uint8_t *__restrict__ scales, int K, int sld, int pld,
     int ppr, int npairs, const int32_t *__restrict__ dst_idx = nullptr, int topk = 1)
 {
-    constexpr bool FP4 = FMT == CCH_FMT_E2M1;
+    constexpr bool FP4 = is_fp4_v<FMT>;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (QUANT_THREADS / 64) + (threadIdx.x >> 6)));
     const int stride = (int)gridDim.x * (QUANT_THREADS / 64);
@@ -394,7 +396,7 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_fast_kernel(
 template <int FMT, int RND, bool HWCVT>
 static int launch_rows(const void *x, void *payload, void *scales, int64_t m, int64_t k, hipStream_t stream)
 {
-    const bool fp4 = FMT == CCH_FMT_E2M1;
+    const bool fp4 = is_fp4_v<FMT>;
     const int64_t nblk = (k + 31) / 32, sld = 2 * ((nblk + 1) / 2), pld = fp4 ? (k + 1) / 2 : k;
     const int64_t wpr = (nblk * 4 + 63) / 64;
     const bool vec = (k % 8 == 0) && aligned(x, 16) && aligned(payload, 8);
@@ -403,7 +405,8 @@ static int launch_rows(const void *x, void *payload, void *scales, int64_t m, in
     CCH_HIP(hipGetDevice(&dev));
     CCH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     const int64_t max_blocks = (int64_t)cus * QUANT_BLOCKS_PER_CU;
-    if (HWCVT && k % 1024 == 0 && aligned(x, 16) && aligned(payload, 16) && aligned(scales, 4) && m * (k / 1024) < ((int64_t)1 << 30)) {
+    if constexpr (HWCVT)
+    if (k % 1024 == 0 && aligned(x, 16) && aligned(payload, 16) && aligned(scales, 4) && m * (k / 1024) < ((int64_t)1 << 30)) {
         const int64_t npairs = m * (k / 1024);
         const unsigned grid = (unsigned)std::min<int64_t>((npairs + QUANT_THREADS / 64 - 1) / (QUANT_THREADS / 64), max_blocks);
         hipLaunchKernelGGL((mx_quant_rows_fast_kernel<FMT>), dim3(grid), dim3(QUANT_THREADS), 0, stream,
@@ -445,7 +448,7 @@ __global__ __launch_bounds__(256) void mx_quant_b_kernel(const uint32_t *__restr
                                                          uint8_t *__restrict__ scales, int K, int N, int trans_b)
 {
     using T = FmtTraits<FMT>;
-    constexpr bool FP4 = FMT == CCH_FMT_E2M1;
+    constexpr bool FP4 = is_fp4_v<FMT>;
     const int np = blockIdx.x * 256 + threadIdx.x;  // column pair
     const int kb = blockIdx.y;
     if (np * 2 >= N) return;
@@ -461,12 +464,14 @@ __global__ __launch_bounds__(256) void mx_quant_b_kernel(const uint32_t *__restr
     int e0, e1;
     bool n0, n1;
     const uint32_t s0 = shared_exp_byte<FMT>(m0, e0, n0), s1 = shared_exp_byte<FMT>(m1, e1, n1);
-    const float i0 = pow2i(-e0), i1 = pow2i(-e1);
+    // 2^-e in two exact factors (2^-127 is no normal float)
+    const float i0 = pow2i(-min(e0, 126)), i1 = pow2i(-min(e1, 126));
+    const float j0 = e0 > 126 ? 0.5f : 1.0f, j1 = e1 > 126 ? 0.5f : 1.0f;
     uint32_t q0[32], q1[32];
 #pragma unroll
     for (int i = 0; i < 32; i++) {
-        q0[i] = n0 ? T::NANCODE : encode_small<FMT, RND>(__uint_as_float(w[i] << 16) * i0);
-        q1[i] = n1 ? T::NANCODE : encode_small<FMT, RND>(__uint_as_float(w[i] & 0xFFFF0000u) * i1);
+        q0[i] = n0 ? T::NANCODE : encode_small<FMT, RND>(__uint_as_float(w[i] << 16) * i0 * j0);
+        q1[i] = n1 ? T::NANCODE : encode_small<FMT, RND>(__uint_as_float(w[i] & 0xFFFF0000u) * i1 * j1);
     }
     const int n = np * 2;
     if (!trans_b) {
@@ -515,7 +520,7 @@ template <int FMT, int RND, bool HWCVT>
 static int launch_scatter(const void *x, const int32_t *dst_idx, void *packed, int64_t tokens, int64_t k, int topk,
                           hipStream_t stream)
 {
-    const bool fp4 = FMT == CCH_FMT_E2M1;
+    const bool fp4 = is_fp4_v<FMT>;
     const int64_t nblk = (k + 31) / 32, sld = 2 * ((nblk + 1) / 2), pbytes = fp4 ? (k + 1) / 2 : k;
     const int64_t row_bytes = pbytes + sld;
     const int64_t wpr = (nblk * 4 + 63) / 64;
@@ -525,7 +530,8 @@ static int launch_scatter(const void *x, const int32_t *dst_idx, void *packed, i
     CCH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     const int64_t max_blocks = (int64_t)cus * QUANT_BLOCKS_PER_CU;
     uint8_t *out = static_cast<uint8_t *>(packed);
-    if (HWCVT && k % 1024 == 0 && aligned(x, 16) && aligned(packed, 16) && row_bytes % 16 == 0 &&
+    if constexpr (HWCVT)
+    if (k % 1024 == 0 && aligned(x, 16) && aligned(packed, 16) && row_bytes % 16 == 0 &&
         tokens * (k / 1024) < ((int64_t)1 << 30)) {
         const int64_t npairs = tokens * (k / 1024);
         const unsigned grid = (unsigned)std::min<int64_t>((npairs + QUANT_THREADS / 64 - 1) / (QUANT_THREADS / 64), max_blocks);
@@ -582,6 +588,9 @@ extern "C" int cch_mx_quant_scatter_packed(const void *x, const int32_t *expande
         case CCH_FMT_E2M1:
             return lut ? launch_scatter<CCH_FMT_E2M1, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s)
                        : launch_scatter<CCH_FMT_E2M1, CCH_ROUND_RNE, true>(x, expanded_row_idx, packed_out, tokens, k, top_k, s);
+        case CCH_FMT_E1M2:  // no hardware conversion for this format: integer encoder for both rules
+            return lut ? launch_scatter<CCH_FMT_E1M2, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s)
+                       : launch_scatter<CCH_FMT_E1M2, CCH_ROUND_RNE, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s);
         default:
             return fail(CCH_EINVAL, "cch_mx_quant_scatter_packed: unknown format %d", fmt);
     }
@@ -608,6 +617,9 @@ extern "C" int cch_mx_quant_rows(const void *x, void *payload, void *scales, int
         case CCH_FMT_E2M1:
             return lut ? launch_rows<CCH_FMT_E2M1, CCH_ROUND_LUT, false>(x, payload, scales, m, k, s)
                        : launch_rows<CCH_FMT_E2M1, CCH_ROUND_RNE, true>(x, payload, scales, m, k, s);
+        case CCH_FMT_E1M2:  // no hardware conversion for this format: integer encoder for both rules
+            return lut ? launch_rows<CCH_FMT_E1M2, CCH_ROUND_LUT, false>(x, payload, scales, m, k, s)
+                       : launch_rows<CCH_FMT_E1M2, CCH_ROUND_RNE, false>(x, payload, scales, m, k, s);
         default:
             return fail(CCH_EINVAL, "cch_mx_quant_rows: unknown format %d", fmt);
     }
@@ -649,6 +661,9 @@ extern "C" int cch_mx_quant_b(const void *b, void *payload, void *scales, int64_
         case CCH_FMT_E2M1:
             return lut ? launch_b<CCH_FMT_E2M1, CCH_ROUND_LUT>(b, payload, scales, k, n, trans_b, s)
                        : launch_b<CCH_FMT_E2M1, CCH_ROUND_RNE>(b, payload, scales, k, n, trans_b, s);
+        case CCH_FMT_E1M2:
+            return lut ? launch_b<CCH_FMT_E1M2, CCH_ROUND_LUT>(b, payload, scales, k, n, trans_b, s)
+                       : launch_b<CCH_FMT_E1M2, CCH_ROUND_RNE>(b, payload, scales, k, n, trans_b, s);
         default:
             return fail(CCH_EINVAL, "cch_mx_quant_b: unknown format %d", fmt);
     }

@@ -7,9 +7,10 @@ torch is used for device memory and streams only; all arithmetic happens in the 
 import torch
 
 from . import _abi
-from ._abi import FMT_E2M1, FMT_E4M3, FMT_E5M2, ROUND_LUT, ROUND_RNE, check
+from ._abi import FMT_E1M2, FMT_E2M1, FMT_E4M3, FMT_E5M2, ROUND_LUT, ROUND_RNE, check
 
-_FMT_NAMES = {"e4m3": FMT_E4M3, "e5m2": FMT_E5M2, "e2m1": FMT_E2M1, "fp8": FMT_E4M3, "fp4": FMT_E2M1}
+_FMT_NAMES = {"e4m3": FMT_E4M3, "e5m2": FMT_E5M2, "e2m1": FMT_E2M1, "e1m2": FMT_E1M2, "fp8": FMT_E4M3, "fp4": FMT_E2M1}
+_FP4 = (FMT_E2M1, FMT_E1M2)   # two codes per byte; E1M2 exists for the quantiser only
 
 
 def _fmt(fmt):
@@ -17,7 +18,7 @@ def _fmt(fmt):
         if fmt.lower() not in _FMT_NAMES:
             raise ValueError("unknown MX payload format %r" % fmt)
         return _FMT_NAMES[fmt.lower()]
-    if fmt not in (FMT_E4M3, FMT_E5M2, FMT_E2M1):
+    if fmt not in (FMT_E4M3, FMT_E5M2, FMT_E2M1, FMT_E1M2):
         raise ValueError("unknown MX payload format %r" % (fmt,))
     return fmt
 
@@ -54,7 +55,7 @@ def mx_quant(x, fmt="e4m3", rounding=ROUND_RNE):
         raise ValueError("mx_quant expects a 2-D bfloat16 tensor")
     x = x.contiguous()
     m, k = x.shape
-    pld = (k + 1) // 2 if fmt == FMT_E2M1 else k
+    pld = (k + 1) // 2 if fmt in _FP4 else k
     payload = torch.empty((m, pld), dtype=torch.uint8, device=x.device)
     scales = torch.empty((m, scale_cols(k)), dtype=torch.uint8, device=x.device)
     check(_abi.lib().cch_mx_quant_rows(_ptr(x), _ptr(payload), _ptr(scales), m, k, fmt, rounding, _stream()))
@@ -63,7 +64,7 @@ def mx_quant(x, fmt="e4m3", rounding=ROUND_RNE):
 
 def packed_row_bytes(k, fmt="e4m3"):
     """Bytes of one packed row of mx_quant_scatter_packed: payload followed by the padded scales."""
-    return ((k + 1) // 2 if _fmt(fmt) == FMT_E2M1 else k) + scale_cols(k)
+    return ((k + 1) // 2 if _fmt(fmt) in _FP4 else k) + scale_cols(k)
 
 
 def mx_quant_scatter_packed(x, expanded_row_idx, packed_out, top_k, fmt="e4m3", rounding=ROUND_RNE):
@@ -77,7 +78,7 @@ def mx_quant_scatter_packed(x, expanded_row_idx, packed_out, top_k, fmt="e4m3", 
     tokens, k = x.shape
     if expanded_row_idx.dtype != torch.int32 or expanded_row_idx.numel() != tokens * top_k:
         raise ValueError("expanded_row_idx must hold tokens * top_k int32 entries")
-    row_bytes = ((k + 1) // 2 if fmt == FMT_E2M1 else k) + scale_cols(k)
+    row_bytes = ((k + 1) // 2 if fmt in _FP4 else k) + scale_cols(k)
     if packed_out.dim() != 2 or packed_out.dtype != torch.uint8 or packed_out.shape[1] != row_bytes or not packed_out.is_contiguous():
         raise ValueError("packed_out must be a contiguous uint8 [rows, %d] tensor" % row_bytes)
     if top_k and tokens and int(expanded_row_idx.max()) >= packed_out.shape[0]:
@@ -101,7 +102,7 @@ def mx_quant_b(b, fmt="e4m3", rounding=ROUND_RNE, trans_b=0):
         raise ValueError("mx_quant_b expects a 2-D bfloat16 tensor [K,N]")
     b = b.contiguous()
     k, n = b.shape
-    fp4 = fmt == FMT_E2M1
+    fp4 = fmt in _FP4
     if trans_b:
         payload = torch.empty((n, k // 2 if fp4 else k), dtype=torch.uint8, device=b.device)
         scales = torch.empty((n, k // 32), dtype=torch.uint8, device=b.device)
@@ -223,6 +224,8 @@ def gmm_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, trans_b=0):
 
 def _mx_shapes(a, sa, b, sb, fmt, trans_b, grouped):
     fmt = _fmt(fmt)
+    if fmt == FMT_E1M2:
+        raise ValueError("E1M2 is a quantiser format only: the matrix instructions have no such operand type")
     fp4 = fmt == FMT_E2M1
     _check_2d("a", a, torch.uint8)
     _check_2d("sa", sa, torch.uint8)

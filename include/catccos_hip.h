@@ -32,6 +32,7 @@ extern "C" {
 #define CCH_FMT_E4M3 0
 #define CCH_FMT_E5M2 1
 #define CCH_FMT_E2M1 2
+#define CCH_FMT_E1M2 3 /* FP4 with one exponent and two mantissa bits (0, .25 ... 1.75): quantiser only */
 
 /* payload rounding: 0 = round to nearest even, sign of zero kept (the device
  * cast, include/catccos/comm/block/comm_block_mx_quant.hpp:596-642);
@@ -70,7 +71,9 @@ int cch_stream_destroy(void *stream);
  *   payload  FP8: [m,k] bytes; FP4: [m,ceil(k/2)], element 2j in the low nibble
  *   scales   E8M0 [m, 2*ceil(k/64)]; entries past ceil(k/32) are 127 (=1.0)
  * One scale per 32 consecutive elements of a row; a ragged last block is
- * treated as zero padded. */
+ * treated as zero padded.  fmt: any CCH_FMT_* — the four output types of the
+ * reference's example (examples/ascend950_mx_quant_allgather/main.cpp:24-37,
+ * MX_QUANT_DTYPE 0..3 = fp8_e4m3, fp8_e5m2, fp4_e2m1, fp4_e1m2). */
 int cch_mx_quant_rows(const void *x, void *payload, void *scales, int64_t m, int64_t k, int fmt, int rounding,
                       void *stream);
 

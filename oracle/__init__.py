@@ -16,7 +16,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
-E4M3, E5M2, E2M1 = 0, 1, 2
+E4M3, E5M2, E2M1, E1M2 = 0, 1, 2, 3
+FP4_FORMATS = (E2M1, E1M2)
 RNE, LUT = 0, 1
 
 _lib = None
@@ -40,7 +41,7 @@ def lib():
         L.orc_bf16_to_f32.argtypes = [c.c_uint16]
         L.orc_f32_to_bf16.restype = c.c_uint16
         L.orc_f32_to_bf16.argtypes = [c.c_float]
-        for name in ("orc_e4m3_decode", "orc_e5m2_decode", "orc_e2m1_decode", "orc_e8m0_decode"):
+        for name in ("orc_e4m3_decode", "orc_e5m2_decode", "orc_e2m1_decode", "orc_e1m2_decode", "orc_e8m0_decode"):
             getattr(L, name).restype = c.c_float
             getattr(L, name).argtypes = [c.c_uint8]
         L.orc_encode.restype = c.c_uint8
@@ -100,7 +101,7 @@ def bf16_to_f32(h):
 
 
 def decode_table(fmt):
-    n = 16 if fmt == E2M1 else 256
+    n = 16 if fmt in FP4_FORMATS else 256
     return np.array([lib().orc_decode(i, fmt) for i in range(n)], dtype=np.float32)
 
 
@@ -131,7 +132,7 @@ def mx_quant_rows(x_bf16, fmt=E4M3, rounding=RNE):
     """x_bf16 uint16 [M,K] -> (payload uint8 [M,K or ceil(K/2)], scales uint8 [M,scale_cols(K)])."""
     x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
     m, k = x.shape
-    pld = (k + 1) // 2 if fmt == E2M1 else k
+    pld = (k + 1) // 2 if fmt in FP4_FORMATS else k
     payload = np.empty((m, pld), dtype=np.uint8)
     scales = np.empty((m, scale_cols(k)), dtype=np.uint8)
     lib().orc_mx_quant_rows(_p(x), _i64(m), _i64(k), fmt, rounding, _p(payload), _p(scales))
@@ -140,7 +141,7 @@ def mx_quant_rows(x_bf16, fmt=E4M3, rounding=RNE):
 
 def packed_row_bytes(k, fmt=E4M3):
     """Bytes of one packed row: payload followed by the padded E8M0 scales."""
-    return ((k + 1) // 2 if fmt == E2M1 else k) + scale_cols(k)
+    return ((k + 1) // 2 if fmt in FP4_FORMATS else k) + scale_cols(k)
 
 
 def mx_quant_scatter_packed(x_bf16, expanded_row_idx, out_rows, top_k, fmt=E4M3, rounding=RNE, fill=0):
@@ -160,7 +161,7 @@ def mx_quant_b(b_bf16, fmt=E4M3, rounding=RNE, trans_b=0):
     """b_bf16 uint16 [K,N] quantised along K; returns (payload, scales) in the boundary layouts."""
     b = np.ascontiguousarray(b_bf16, dtype=np.uint16)
     k, n = b.shape
-    fp4 = fmt == E2M1
+    fp4 = fmt in FP4_FORMATS
     if trans_b:
         payload = np.empty((n, (k + 1) // 2 if fp4 else k), dtype=np.uint8)
         scales = np.empty((n, scale_cols(k)), dtype=np.uint8)

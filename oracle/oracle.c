@@ -41,6 +41,8 @@
 #define ORC_FMT_E4M3 0
 #define ORC_FMT_E5M2 1
 #define ORC_FMT_E2M1 2
+#define ORC_FMT_E1M2 3
+#define ORC_IS_FP4(fmt) ((fmt) == ORC_FMT_E2M1 || (fmt) == ORC_FMT_E1M2)
 /* rounding rule of the payload cast */
 #define ORC_ROUND_RNE 0 /* nearest, ties to even code, sign of zero kept      */
 #define ORC_ROUND_LUT 1 /* nearest, ties to the smaller magnitude, zero is +0 */
@@ -106,6 +108,16 @@ float orc_e2m1_decode(uint8_t nib)
     return (nib & 8u) ? -v : v;
 }
 
+/* E1M2 nibble: magnitudes {0,.25,.5,.75,1,1.25,1.5,1.75}
+ * (gen_mx_quant_allgather_data.py:65-72 with the table builder :352-375: one exponent bit,
+ * two mantissa bits, bias 1).
+ * pinned by: the closed list above, spelled out in the test */
+float orc_e1m2_decode(uint8_t nib)
+{
+    float v = small_decode(nib & 7u, 1, 2, 1);
+    return (nib & 8u) ? -v : v;
+}
+
 /* E8M0: 2^(b-127); 0xFF is NaN.  pinned by: torch.float8_e8m0fnu, 256 codes */
 float orc_e8m0_decode(uint8_t b)
 {
@@ -124,7 +136,7 @@ typedef struct {
     uint8_t nan_code;
 } fmt_table;
 
-static fmt_table g_tab[3];
+static fmt_table g_tab[4];
 static int g_tab_ready = 0;
 
 static void build_tables(void)
@@ -142,6 +154,10 @@ static void build_tables(void)
     t->ncodes = 8;
     for (int i = 0; i < 8; i++) t->val[i] = small_decode((uint32_t)i, 2, 1, 1);
     t->maxv = 6.0f; t->emax = 2; t->signbit = 0x8u; t->nan_code = 0x7u; /* E2M1 has no NaN */
+    t = &g_tab[ORC_FMT_E1M2];
+    t->ncodes = 8;
+    for (int i = 0; i < 8; i++) t->val[i] = small_decode((uint32_t)i, 1, 2, 1);
+    t->maxv = 1.75f; t->emax = 0; t->signbit = 0x8u; t->nan_code = 0x7u; /* no NaN either */
 #pragma omp flush
     g_tab_ready = 1;
 }
@@ -188,6 +204,7 @@ float orc_decode(uint8_t c, int fmt)
 {
     if (fmt == ORC_FMT_E4M3) return orc_e4m3_decode(c);
     if (fmt == ORC_FMT_E5M2) return orc_e5m2_decode(c);
+    if (fmt == ORC_FMT_E1M2) return orc_e1m2_decode(c);
     return orc_e2m1_decode(c);
 }
 
@@ -235,14 +252,14 @@ int orc_mx_quant_rows(const uint16_t *x, int64_t M, int64_t K, int fmt, int roun
     build_tables();
     const int64_t nblk = (K + 31) / 32;
     const int64_t sld = ((nblk + 1) / 2) * 2;
-    const int64_t pld = (fmt == ORC_FMT_E2M1) ? (K + 1) / 2 : K;
+    const int64_t pld = ORC_IS_FP4(fmt) ? (K + 1) / 2 : K;
     const int emax = fmt_emax(fmt);
 #pragma omp parallel for schedule(static)
     for (int64_t m = 0; m < M; m++) {
         const uint16_t *xr = x + m * K;
         uint8_t *pr = payload + m * pld;
         uint8_t *sr = scales + m * sld;
-        if (fmt == ORC_FMT_E2M1) memset(pr, 0, (size_t)pld);
+        if (ORC_IS_FP4(fmt)) memset(pr, 0, (size_t)pld);
         for (int64_t b = 0; b < sld; b++) {
             if (b >= nblk) { sr[b] = 127; continue; }
             int64_t k0 = b * 32, k1 = k0 + 32 < K ? k0 + 32 : K;
@@ -266,7 +283,7 @@ int orc_mx_quant_rows(const uint16_t *x, int64_t M, int64_t K, int fmt, int roun
                 /* division by 2^e is exact in fp32 unless the quotient is subnormal */
                 float y = is_nan ? NAN : ldexpf(v, -e);
                 uint8_t q = orc_encode(y, fmt, rounding);
-                if (fmt == ORC_FMT_E2M1) pr[k >> 1] |= (uint8_t)(q << ((k & 1) * 4));
+                if (ORC_IS_FP4(fmt)) pr[k >> 1] |= (uint8_t)(q << ((k & 1) * 4));
                 else pr[k] = q;
             }
         }
@@ -291,7 +308,7 @@ int orc_mx_quant_scatter_packed(const uint16_t *x, const int32_t *expanded_row_i
 {
     const int64_t nblk = (K + 31) / 32;
     const int64_t sld = ((nblk + 1) / 2) * 2;
-    const int64_t pld = (fmt == ORC_FMT_E2M1) ? (K + 1) / 2 : K;
+    const int64_t pld = ORC_IS_FP4(fmt) ? (K + 1) / 2 : K;
     const int64_t row_bytes = pld + sld;
     uint8_t *row = (uint8_t *)malloc((size_t)row_bytes);
     if (!row) return -1;
@@ -322,7 +339,7 @@ int orc_mx_quant_b(const uint16_t *b, int64_t K, int64_t N, int fmt, int roundin
 {
     const int64_t nblk = (K + 31) / 32;
     const int64_t sld = ((nblk + 1) / 2) * 2;
-    const int fp4 = fmt == ORC_FMT_E2M1;
+    const int fp4 = ORC_IS_FP4(fmt);
     const int64_t pldT = fp4 ? (K + 1) / 2 : K;
     uint16_t *bt = (uint16_t *)malloc((size_t)(N * K) * 2);
     uint8_t *pt = (uint8_t *)malloc((size_t)(N * pldT));
@@ -364,11 +381,11 @@ void orc_mx_dequant_rows(const uint8_t *payload, const uint8_t *scales, int64_t 
 {
     const int64_t nblk = (K + 31) / 32;
     const int64_t sld = ((nblk + 1) / 2) * 2;
-    const int64_t pld = (fmt == ORC_FMT_E2M1) ? (K + 1) / 2 : K;
+    const int64_t pld = ORC_IS_FP4(fmt) ? (K + 1) / 2 : K;
 #pragma omp parallel for schedule(static)
     for (int64_t m = 0; m < M; m++)
         for (int64_t k = 0; k < K; k++) {
-            uint8_t q = (fmt == ORC_FMT_E2M1) ? (payload[m * pld + (k >> 1)] >> ((k & 1) * 4)) & 0xF
+            uint8_t q = ORC_IS_FP4(fmt) ? (payload[m * pld + (k >> 1)] >> ((k & 1) * 4)) & 0xF
                                               : payload[m * pld + k];
             out[m * K + k] = orc_decode(q, fmt) * orc_e8m0_decode(scales[m * sld + k / 32]);
         }

@@ -9,7 +9,7 @@ from catccos_amd import _abi
 
 pytestmark = pytest.mark.gpu
 
-FMTS = [(orc.E4M3, cc.FMT_E4M3), (orc.E5M2, cc.FMT_E5M2), (orc.E2M1, cc.FMT_E2M1)]
+FMTS = [(orc.E4M3, cc.FMT_E4M3), (orc.E5M2, cc.FMT_E5M2), (orc.E2M1, cc.FMT_E2M1), (orc.E1M2, cc.FMT_E1M2)]
 
 
 def to_dev(bits_u16):

@@ -9,7 +9,7 @@ import catccos_amd as cc
 
 pytestmark = pytest.mark.gpu
 
-FMTS = {"e4m3": orc.E4M3, "e5m2": orc.E5M2, "e2m1": orc.E2M1}
+FMTS = {"e4m3": orc.E4M3, "e5m2": orc.E5M2, "e2m1": orc.E2M1, "e1m2": orc.E1M2}
 
 
 def rand_rows(rng, rows, k, sigma=1.0):
@@ -36,7 +36,7 @@ def run_case(tokens, k, topk, fmt, rounding, seed, drop=2):
     assert np.array_equal(packed.cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1", "e1m2"])
 @pytest.mark.parametrize("shape", [(64, 7168, 2), (33, 1024, 8), (7, 256, 1), (19, 4096, 4)])
 def test_scatter_vector_path(shape, fmt):
     tokens, k, topk = shape
@@ -51,7 +51,7 @@ def test_scatter_byte_path_and_ragged_k(shape, fmt):
     run_case(tokens, k, topk, fmt, cc.ROUND_RNE, tokens * 3 + k)
 
 
-@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1", "e1m2"])
 def test_scatter_lut_rounding(fmt):
     run_case(40, 2048, 2, fmt, cc.ROUND_LUT, 5)
 

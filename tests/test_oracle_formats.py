@@ -45,6 +45,24 @@ def test_e2m1_table_closed_form():
     assert np.signbit(t[8])
 
 
+def test_e1m2_table_closed_form():
+    # one exponent bit, two mantissa bits, bias 1 (gen_mx_quant_allgather_data.py:65-72, :352-375):
+    # subnormals m/4, normals 1 + m/4
+    t = orc.decode_table(orc.E1M2)
+    mags = [0.0, 0.25, 0.5, 0.75, 1.0, 1.25, 1.5, 1.75]
+    assert list(t[:8]) == mags
+    assert list(t[8:]) == [-m for m in mags]
+    assert np.signbit(t[8])
+
+
+def test_e1m2_ties_and_saturation():
+    x = np.array([0.125, 0.375, 0.625, 0.875, 1.125, 1.375, 1.625, 1.8, 9.0, -0.125, -0.375, -1.625, -0.05, -0.0], dtype=np.float32)
+    want_rne = [0, 2, 2, 4, 4, 6, 6, 7, 7, 8, 10, 14, 8, 8]
+    want_lut = [0, 1, 2, 3, 4, 5, 6, 7, 7, 0, 9, 14, 0, 0]
+    assert list(orc.encode(x, orc.E1M2, orc.RNE)) == want_rne
+    assert list(orc.encode(x, orc.E1M2, orc.LUT)) == want_lut
+
+
 def test_bf16_rounding_matches_torch():
     rng = np.random.default_rng(0)
     x = np.concatenate([
@@ -89,14 +107,14 @@ def test_fp8_rne_encode_matches_torch(fmt, dtype, maxv):
                           torch.from_numpy(np.clip(y, -maxv, maxv)).to(dtype).view(torch.uint8).numpy())
 
 
-@pytest.mark.parametrize("fmt", [orc.E4M3, orc.E5M2, orc.E2M1])
+@pytest.mark.parametrize("fmt", [orc.E4M3, orc.E5M2, orc.E2M1, orc.E1M2])
 def test_lut_encode_is_first_argmin_over_full_table(fmt):
     """The reference's table rule: argmin |LUT - v| over the full signed table, first index wins
     (gen_mx_quant_allgather_data.py:198-247; gen_data_fp4_mx_alltoallv_gmm.py:216-217)."""
     tab = orc.decode_table(fmt).astype(np.float64)
     n = tab.size
     half = n // 2
-    maxv = {orc.E4M3: 448.0, orc.E5M2: 57344.0, orc.E2M1: 6.0}[fmt]
+    maxv = {orc.E4M3: 448.0, orc.E5M2: 57344.0, orc.E2M1: 6.0, orc.E1M2: 1.75}[fmt]
     lut = tab.copy()
     bad = ~np.isfinite(lut)
     lut[bad] = np.where(np.arange(n)[bad] < half, maxv, -maxv)  # reference maps NaN/Inf codes to +-max
@@ -108,7 +126,7 @@ def test_lut_encode_is_first_argmin_over_full_table(fmt):
     assert np.array_equal(ours, brute)
 
 
-@pytest.mark.parametrize("fmt", [orc.E4M3, orc.E5M2, orc.E2M1])
+@pytest.mark.parametrize("fmt", [orc.E4M3, orc.E5M2, orc.E2M1, orc.E1M2])
 @pytest.mark.parametrize("rounding", [orc.RNE, orc.LUT])
 def test_encode_decode_identity(fmt, rounding):
     tab = orc.decode_table(fmt)
@@ -133,7 +151,7 @@ def test_shared_exponent_invariant_all_bf16_maxima():
     """2^e <= amax / 2^emax < 2^(e+1) for every positive normal bf16 block maximum."""
     bits = np.arange(0x0080, 0x7F80, dtype=np.uint16)
     vals = orc.bf16_to_f32(bits)
-    for emax in (8, 15, 2):
+    for emax in (8, 15, 2, 0):
         for v in vals[::37]:
             if v < 1e-12:
                 continue

@@ -7,8 +7,8 @@ import torch
 
 import oracle as orc
 
-MAXV = {orc.E4M3: 448.0, orc.E5M2: 57344.0, orc.E2M1: 6.0}
-EMAX = {orc.E4M3: 8, orc.E5M2: 15, orc.E2M1: 2}
+MAXV = {orc.E4M3: 448.0, orc.E5M2: 57344.0, orc.E2M1: 6.0, orc.E1M2: 1.75}
+EMAX = {orc.E4M3: 8, orc.E5M2: 15, orc.E2M1: 2, orc.E1M2: 0}
 
 
 def make_input(m, k, seed, outliers=True, scale=1.0):
@@ -54,16 +54,17 @@ def test_fp8_rows_match_independent_recipe(fmt, shape):
     assert np.array_equal(q, qi)
 
 
-def test_fp4_rows_match_bruteforce():
+@pytest.mark.parametrize("fmt", [orc.E2M1, orc.E1M2])
+def test_fp4_rows_match_bruteforce(fmt):
     x = make_input(48, 256, seed=4, scale=0.02)
-    p, s = orc.mx_quant_rows(x, orc.E2M1, orc.RNE)
+    p, s = orc.mx_quant_rows(x, fmt, orc.RNE)
     q = unpack_fp4(p, 256)
     xf = orc.bf16_to_f32(x).astype(np.float64).reshape(48, 8, 32)
     amax = np.abs(xf).max(-1)
-    e = np.floor(np.log2(amax)) - 2
+    e = np.floor(np.log2(amax)) - EMAX[fmt]
     assert np.array_equal(s, (e + 127).astype(np.uint8))
-    y = np.clip(xf / np.exp2(e)[..., None], -6, 6).reshape(48, 256)
-    tab = orc.decode_table(orc.E2M1).astype(np.float64)
+    y = np.clip(xf / np.exp2(e)[..., None], -MAXV[fmt], MAXV[fmt]).reshape(48, 256)
+    tab = orc.decode_table(fmt).astype(np.float64)
     d = np.abs(y[..., None] - tab[None, None, :])
     best = d.min(-1)
     # the chosen code is a nearest one, and among ties it has an even mantissa bit
@@ -75,7 +76,7 @@ def test_fp4_rows_match_bruteforce():
     assert np.array_equal((q & 8) != 0, neg)  # RNE rule keeps the sign, also on zero results
 
 
-@pytest.mark.parametrize("fmt", [orc.E4M3, orc.E5M2, orc.E2M1])
+@pytest.mark.parametrize("fmt", [orc.E4M3, orc.E5M2, orc.E2M1, orc.E1M2])
 @pytest.mark.parametrize("rounding", [orc.RNE, orc.LUT])
 def test_requantising_dequantised_data_is_identity(fmt, rounding):
     """The check the reference's own run.sh performs: its inputs are dequantised values
@@ -95,7 +96,7 @@ def test_requantising_dequantised_data_is_identity(fmt, rounding):
     assert np.array_equal(s, s2)
 
 
-@pytest.mark.parametrize("fmt", [orc.E4M3, orc.E2M1])
+@pytest.mark.parametrize("fmt", [orc.E4M3, orc.E2M1, orc.E1M2])
 def test_power_of_two_scaling_shifts_only_the_scale(fmt):
     x = make_input(16, 256, seed=6)
     p, s = orc.mx_quant_rows(x, fmt)
