@@ -322,3 +322,57 @@ def test_mx_gmm_mapped_rows(fmt, trans_b, tiled):
     untouched[kept[kept >= 0]] = False
     assert (got[untouched] == -3.0).all()
     assert_close(got[~untouched], want[~untouched], ("mx gmm mapped", fmt, trans_b, tiled))
+
+
+def _both_paths(fn):
+    """fn() on the tiled kernels (a fall-back would be an error) and on the generic ones."""
+    outs = []
+    for tiled in (True, False):
+        cc.set_option("require_tiled_gemm", 1 if tiled else 0)
+        cc.set_option("force_generic_gemm", 0 if tiled else 1)
+        try:
+            outs.append(out_f32(fn()))
+        finally:
+            cc.set_option("require_tiled_gemm", 0)
+            cc.set_option("force_generic_gemm", 0)
+    return outs
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_tiled_matches_generic_on_random_groups(seed):
+    """Random expert counts, group sizes (empty, one-row, many-tile groups, rows of no group), K-step
+    counts, widths and both weight layouts: the tiled kernels against the one-thread-per-output
+    kernels on the device.  Both accumulate the same products in fp32 (int32 for int8), so they may
+    differ only by summation order and one final rounding."""
+    rng = np.random.default_rng(1000 + seed)
+    e = int(rng.integers(1, 13))
+    sizes = rng.choice([0, 1, 31, 33, 100, 129, 255, 256, 257, 300, 600, 1100], e).astype(np.int32)
+    used = int(sizes.sum())
+    t = used + int(rng.choice([0, 0, 5, 260]))
+    if t == 0:
+        t, sizes[0] = 40, 40
+    kind = ["i8", "e4m3", "e5m2", "e2m1"][seed % 4]
+    k = int(rng.choice([256, 384, 640, 1024])) * (2 if kind == "e2m1" else 1)    # whole 128-byte K-steps, at least two
+    n = int(rng.choice([64, 160, 256, 416, 512, 672]))
+    trans_b = int(rng.integers(0, 2))
+    gs = dev(sizes)
+    if kind == "i8":
+        x = dev(rng.integers(-127, 128, (t, k)).astype(np.int8))
+        w = dev(rng.integers(-127, 128, (e, n, k) if trans_b else (e, k, n)).astype(np.int8))
+        pt = dev(rng.uniform(0.001, 0.02, t).astype(np.float32))
+        pc = dev(rng.uniform(0.001, 0.02, (e, n)).astype(np.float32))
+        a, b = _both_paths(lambda: cc.gmm_dequant_swiglu(x, w, gs, pt, pc, trans_b))
+    else:
+        pack = 2 if kind == "e2m1" else 1
+        mask = 0x77 if kind != "e5m2" else 0x7B                       # finite codes only
+        pa = dev((rng.integers(0, 256, (t, k // pack)) & (mask | 0x80 if pack == 1 else 0xFF)).astype(np.uint8))
+        pb = dev((rng.integers(0, 256, ((e, n, k // pack) if trans_b else (e, k, n // pack))) & (mask | 0x80 if pack == 1 else 0xFF)).astype(np.uint8))
+        sa = dev(rng.integers(120, 132, (t, k // 32)).astype(np.uint8))
+        sb = dev(rng.integers(120, 132, ((e, n, k // 32) if trans_b else (e, k // 64, n, 2))).astype(np.uint8))
+        a, b = _both_paths(lambda: cc.mx_grouped_matmul(pa, sa, pb, sb, gs, kind, trans_b))
+    assert np.isfinite(a).all() and np.isfinite(b).all()
+    assert (a[used:] == 0).all() and (b[used:] == 0).all()               # rows of no group
+    # one bf16 unit in the last place of the element itself, plus summation-order noise relative to the typical size
+    scale = max(float(np.sqrt(np.mean(b[:used].astype(np.float64) ** 2))), 1e-30) if used else 1.0
+    excess = np.abs(a - b) - (2.0 ** -7 * np.abs(b) + 1e-3 * scale)
+    assert excess.max() <= 0, (seed, e, sizes.tolist(), t, k, n, trans_b, kind, float(excess.max()), scale)
