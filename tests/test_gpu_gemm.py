@@ -129,6 +129,43 @@ def test_mx_gemm(fmt, shape, trans_b, path):
     assert_close(got, want)
 
 
+def _reference_shapes(op, limit=4e10):
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_shapes.json")
+    return [tuple(s) for s in json.load(open(path))[op] if 2.0 * s[0] * s[1] * s[2] <= limit]
+
+
+@pytest.mark.parametrize("shape", _reference_shapes("ascend950_mxfp8_matmul_reduce_scatter"))
+def test_mx_gemm_reference_shape_list(shape):
+    """Every (M, K, N) of the reference's own list for the MXFP8 operator
+    (examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/test_shapes.csv, kept as the fixture
+    golden/reference_shapes.json), in the layout its run uses (transB = 1)."""
+    m, k, n = shape
+    rng = np.random.default_rng(m + k + n)
+    pa, sa, pb, sb = mx_operands(rng, m, n, k, "e4m3", 1)
+    want = orc.mx_gmm(pa, sa, pb, sb, n, k, orc.E4M3, 1)
+    got = out_f32(cc.mx_matmul(dev(pa), dev(sa), dev(pb), dev(sb), "e4m3", 1))
+    assert_close(got, want, shape)
+
+
+@pytest.mark.parametrize("op,fmt", [("ascend950_fp8_mx_grouped_matmul_alltoallv", "e4m3"), ("ascend950_fp4_mx_grouped_matmul_alltoallv", "e2m1"),
+                                    ("ascend950_fp8_mx_alltoallv_grouped_matmul", "e4m3"), ("ascend950_fp4_mx_alltoallv_grouped_matmul", "e2m1")])
+def test_mx_gmm_reference_shape_lists(op, fmt):
+    """The grouped operators' own shapes (their scripts/test_shapes.csv), 8 experts as their run.sh defaults to."""
+    for (m, k, n) in _reference_shapes(op):
+        e = 8
+        rng = np.random.default_rng(m + k + n)
+        gs = zipf_groups(rng, m, e)
+        sigma = 0.02 if fmt == "e2m1" else 1.0
+        pa, sa = orc.mx_quant_rows(rand_bf16(rng, (m, k), sigma), FMT[fmt])
+        pbs, sbs = zip(*[orc.mx_quant_b(rand_bf16(rng, (k, n), sigma), FMT[fmt], orc.RNE, 0) for _ in range(e)])
+        pb, sb = np.stack(pbs), np.stack(sbs)
+        want = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], 0, group_sizes=gs)
+        got = out_f32(cc.mx_grouped_matmul(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), fmt, 0))
+        assert_close(got, want, (op, m, k, n))
+
+
 def test_mx_gemm_scale_extremes():
     """Scale bytes far from 127 on both operands, incl. products that leave the fp32 normal range."""
     rng = np.random.default_rng(5)

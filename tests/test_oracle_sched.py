@@ -1,15 +1,22 @@
 """Scheduler arithmetic: the reference's only numeric known-answer test, plus partition invariants."""
+import json
+import os
+
 import numpy as np
 
 import oracle as orc
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 
 def test_reference_unit_test_vector():
     """tests/comm_block_scheduler_alltoallv_gmm/test_comm_block_scheduler_alltoallv_gmm.cpp:37-102:
     rank=2, EP=4, expertPerRank=2, tokenData[i]=i+1; expected 16 ints (entries 2,3 are the
-    freshly reset context)."""
+    freshly reset context).  The expected vector is the committed fixture golden/scheduler_kat.json."""
+    kat = json.load(open(os.path.join(GOLDEN, "scheduler_kat.json")))
     tok = np.arange(1, 33, dtype=np.int32)
-    rank, ep, epr = 2, 4, 2
+    rank, ep, epr = kat["rank"], kat["ep"], kat["expert_per_rank"]
+    assert [(q["core"], q["num"]) for q in kat["queries"]] == [(1, 3), (4, 6), (0, 3)]
     got = []
     core, num = 1, 3
     got += [core, num, 0, 0, orc.sched_src_prev_sum(tok, rank, ep, epr, core), orc.sched_comm_loops(ep, core, num),
@@ -20,7 +27,7 @@ def test_reference_unit_test_vector():
     core, num = 0, 3
     got += [core, orc.sched_src_prev_sum(tok, rank, ep, epr, core), orc.sched_comm_loops(ep, core, num),
             orc.sched_block_offset_row(core, num, 1)]
-    assert got == [1, 3, 0, 0, 42, 1, 1, 4, 4, 0, 0, 4, 0, 10, 2, 3]
+    assert got == kat["expected"] == [1, 3, 0, 0, 42, 1, 1, 4, 4, 0, 0, 4, 0, 10, 2, 3]
 
 
 def test_cumsum_mm_is_column_cumsum():
