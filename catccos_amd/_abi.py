@@ -35,6 +35,8 @@ PROTOTYPES = {
     "cch_mx_quant_b": [_P, _P, _P, _I64, _I64, _I, _I, _I, _P],
     "cch_mx_quant_scatter_packed": [_P, _P, _P, _I64, _I64, _I, _I, _I, _P],
     "cch_moe_token_unpermute": [_P, _P, _P, _P, _I64, _I64, _I64, _I, _P],
+    "cch_moe_init_routing_workspace_bytes": [_I64, _I],
+    "cch_moe_init_routing": [_P, _I64, _I, _P, _P, _P, _I, _P, _I64, _P],
     "cch_dyn_quant_i8_rows": [_P, _P, _P, _P, _I64, _I64, _I64, _I, _I, _P],
     "cch_gemm_i8_dequant": [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I, _P],
     "cch_gmm_i8_dequant_swiglu": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _P],
@@ -43,7 +45,7 @@ PROTOTYPES = {
     "cch_mx_gmm_mapped": [_P, _P, _P, _P, _P, _P, _P, _I64, _I, _I64, _I64, _I64, _I64, _I, _I, _P],
     "cch_set_option": [c.c_char_p, _I],
 }
-_RESTYPE = {"cch_last_error": c.c_char_p}
+_RESTYPE = {"cch_last_error": c.c_char_p, "cch_moe_init_routing_workspace_bytes": _I64}
 
 _lib = None
 

@@ -41,9 +41,14 @@ void LaunchDispatchGmmDequantSwigluINT8(void *stream, uint32_t, uint64_t, Kernel
                                         CocTilingParams &t, uint32_t, uint32_t transB)
 {
     if (p.customCount >= 6) {
-        // from bf16 tokens: dynamic int8 quantisation with the expert-sorted gather, then the grouped matmul
+        // from bf16 tokens: routing sort, dynamic int8 quantisation with the expert-sorted gather, grouped matmul
         const int64_t topK = t.topK ? t.topK : 1, rows = (int64_t)t.m * topK;
-        int rc = cch_dyn_quant_i8_rows(p.ptrA, reinterpret_cast<const int32_t *>(p.customPtrs[4]), p.customPtrs[5],
+        int rc = cch_moe_init_routing(reinterpret_cast<const int32_t *>(p.customPtrs[1]), rows, (int)t.expertNum,
+                                      reinterpret_cast<int32_t *>(p.customPtrs[4]), reinterpret_cast<int32_t *>(p.customPtrs[6]),
+                                      reinterpret_cast<int32_t *>(p.customPtrs[3]), 0, p.customPtrs[7],
+                                      cch_moe_init_routing_workspace_bytes(rows, (int)t.expertNum), stream);
+        if (rc == CCH_OK)
+            rc = cch_dyn_quant_i8_rows(p.ptrA, reinterpret_cast<const int32_t *>(p.customPtrs[4]), p.customPtrs[5],
                                        reinterpret_cast<float *>(p.customPtrs[2]), t.m, rows, t.k, (int)topK, CCH_DQ_DEVICE, stream);
         if (rc == CCH_OK)
             rc = cch_gmm_i8_dequant_swiglu(p.customPtrs[5], p.ptrB, reinterpret_cast<const int32_t *>(p.customPtrs[3]),

@@ -164,12 +164,13 @@ public:
 // dispatch_gmm_dequant_swiglu_host.h:15-119), two file sets:
 //  * the reference's own (expert_idx_<r>.bin present): a_gm_<r>.bin bf16 tokens [m,k], expert_idx_<r>.bin
 //    int32 [m,topK], scale_gm_<r>.bin per-channel scales as 64-bit fix-pipe words (low 32 bits = fp32,
-//    gen_data_dispatch_gmm_dequant_swiglu.py:75-76) or plain fp32.  The routing is done here on the host
-//    (stable sort of the flat expert indices, as moe_init_routing does), the dynamic int8 quantisation
-//    with the expert-sorted row gather and the grouped matmul on the device, over m * topK rows.
+//    gen_data_dispatch_gmm_dequant_swiglu.py:75-76) or plain fp32.  Routing (stable sort of the flat
+//    expert indices, as moe_init_routing does), dynamic int8 quantisation with the expert-sorted row
+//    gather and the grouped matmul all run on the device, over m * topK rows.
 //    ptrA = tokens, ptrB = W, ptrC = out bf16 [m*topK, n/2], custom[0] = per-channel fp32 [E,n],
 //    custom[1] = expert idx (as in the reference), then derived: custom[2] = per-token fp32 [m*topK],
-//    custom[3] = rows per expert, custom[4] = sorted expanded-row index [m*topK], custom[5] = int8 rows.
+//    custom[3] = rows per expert, custom[4] = flat entry at each sorted position [m*topK], custom[5] = int8
+//    rows, custom[6] = sorted position of each flat entry, custom[7] = routing workspace.
 //  * after the dispatch (no expert_idx file): a_gm_<r>.bin holds the int8 tokens this rank received,
 //    grouped by local expert ([m,k]); group_list_<r>.bin int32[expertNum] their counts;
 //    pertoken_scale_<r>.bin fp32[m].  ptrA = tokens, ptrB = W int8 [E,k,n] (transB: [E,n,k]),
@@ -206,21 +207,15 @@ public:
         if (fromTokens_) {
             const size_t rows = m * topK;
             uint8_t *x = LoadOrFill(m * k * 2, dataFile, "a_gm_" + R(rankId) + ".bin", 0);
-            std::vector<int32_t> expertIdx(rows, 0), groups(e, 0), sorted(rows, -1);
+            std::vector<int32_t> expertIdx(rows, 0);
             ReadFile(idxFile, expertIdx.data(), rows * 4);
-            // stable counting sort of the flat (token, route) list by expert: position -> flat index
-            for (size_t i = 0; i < rows; i++)
-                if (expertIdx[i] >= 0 && static_cast<size_t>(expertIdx[i]) < e) groups[expertIdx[i]]++;
-            std::vector<size_t> next(e, 0);
-            for (size_t i = 1; i < e; i++) next[i] = next[i - 1] + groups[i - 1];
-            for (size_t i = 0; i < rows; i++)
-                if (expertIdx[i] >= 0 && static_cast<size_t>(expertIdx[i]) < e) sorted[next[expertIdx[i]]++] = static_cast<int32_t>(i);
+            // buffers of the device-side routing (stable sort by expert), filled by the launcher
+            const size_t wsBytes = static_cast<size_t>(cch_moe_init_routing_workspace_bytes(static_cast<int64_t>(rows), static_cast<int>(e)));
             uint8_t *idxDev = DeviceAlloc(rows * 4), *tokDev = DeviceAlloc(rows * 4), *grpDev = DeviceAlloc(e * 4);
             uint8_t *srcDev = DeviceAlloc(rows * 4), *q = DeviceAlloc(rows * k), *d = DeviceAlloc(rows * (n / 2) * 2);
+            uint8_t *posDev = DeviceAlloc(rows * 4), *wsDev = DeviceAlloc(wsBytes);
             CCH_CHECK(cch_memcpy_h2d(idxDev, expertIdx.data(), rows * 4));
-            CCH_CHECK(cch_memcpy_h2d(grpDev, groups.data(), e * 4));
-            CCH_CHECK(cch_memcpy_h2d(srcDev, sorted.data(), rows * 4));
-            params.SetKernelParams(x, b, d, chDev, idxDev, tokDev, grpDev, srcDev, q);
+            params.SetKernelParams(x, b, d, chDev, idxDev, tokDev, grpDev, srcDev, q, posDev, wsDev);
             return;
         }
         uint8_t *a = LoadOrFill(m * k, dataFile, "a_gm_" + R(rankId) + ".bin", 1);

@@ -142,6 +142,28 @@ def dynamic_quant_i8(x, src_rows=None, topk=1, mode=DQ_DEVICE):
     return q, scale
 
 
+def moe_init_routing(expert_idx, num_experts, cumsum=False):
+    """Stable sort of the flat (token, route) list by expert.
+
+    expert_idx: int32 tensor (any shape, read flat); entries outside [0, num_experts) are dropped.
+    Returns (dst_to_src, src_to_dst, expert_tokens): the flat entry at every sorted position (-1 past
+    the routed entries), the sorted position of every flat entry (-1 if dropped), and the entries
+    per expert (their running sum with cumsum=True)."""
+    _require_gpu(expert_idx)
+    if expert_idx.dtype != torch.int32:
+        raise ValueError("expert_idx must be an int32 tensor")
+    idx = expert_idx.contiguous().reshape(-1)
+    rows = idx.numel()
+    dst_to_src = torch.empty(rows, dtype=torch.int32, device=idx.device)
+    src_to_dst = torch.empty(rows, dtype=torch.int32, device=idx.device)
+    tokens = torch.empty(num_experts, dtype=torch.int32, device=idx.device)
+    nbytes = _abi.lib().cch_moe_init_routing_workspace_bytes(rows, int(num_experts))
+    ws = torch.empty(max(int(nbytes), 4), dtype=torch.uint8, device=idx.device)
+    check(_abi.lib().cch_moe_init_routing(_ptr(idx), rows, int(num_experts), _ptr(dst_to_src), _ptr(src_to_dst), _ptr(tokens),
+                                          1 if cumsum else 0, _ptr(ws), ws.numel(), _stream()))
+    return dst_to_src, src_to_dst, tokens
+
+
 def moe_token_unpermute(permuted_tokens, sorted_indices, probs=None, top_k=1):
     """out[t] = sum_j permuted_tokens[sorted_indices[t*top_k + j]] * probs[t*top_k + j] (bf16 [tokens, hidden]).
 

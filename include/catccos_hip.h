@@ -180,6 +180,24 @@ int cch_mx_quant_scatter_packed(const void *x, const int32_t *expanded_row_idx, 
 int cch_moe_token_unpermute(const void *permuted_tokens, const int32_t *sorted_indices, const float *probs, void *out,
                             int64_t rows, int64_t tokens, int64_t hidden, int top_k, void *stream);
 
+/* ---- MoE routing: stable sort of the (token, route) list by expert ----
+ * Replaces the sort stage of moe_init_routing_quant_v2 (examples/aux_ops/moe_init_routing_quant_v2/
+ * moe_init_routing_quant_v2.h:70-110 with moe_v2_src_to_dst_op.h and moe_v2_expert_token_out.h;
+ * CPU stand-in examples/utils/gen_data_moe.py:48-57).
+ *   expert_idx     int32 [rows]: expert of flat entry token * top_k + route; an entry outside
+ *                  [0, num_experts) is dropped
+ *   dst_to_src     int32 [rows]: flat entry at sorted position i (experts ascending, ties in flat
+ *                  order), -1 past the routed entries; this is the src_rows of cch_dyn_quant_i8_rows
+ *   src_to_dst     int32 [rows]: sorted position of flat entry i, -1 if dropped; this is the
+ *                  sorted_indices of cch_moe_token_unpermute and the expanded_row_idx the reference's
+ *                  operator returns
+ *   expert_tokens  int32 [num_experts]: entries per expert, or their running sum with cumsum != 0
+ *   workspace      device memory of at least cch_moe_init_routing_workspace_bytes(rows, num_experts)
+ * num_experts <= 1024. */
+int64_t cch_moe_init_routing_workspace_bytes(int64_t rows, int num_experts);
+int cch_moe_init_routing(const int32_t *expert_idx, int64_t rows, int num_experts, int32_t *dst_to_src, int32_t *src_to_dst,
+                         int32_t *expert_tokens, int cumsum, void *workspace, int64_t workspace_bytes, void *stream);
+
 /* ---- Per-token dynamic int8 quantisation with row gather (feeds config 4) ----
  * Replaces MoeV2GatherDynamicQuant (examples/aux_ops/moe_init_routing_quant_v2/
  * moe_v2_gather_dynamic_quant.h:117-150 Compute, :213-250 the gather loop), without its

@@ -355,3 +355,20 @@ def scatter_rows(values, row_map, out_rows, fill=0):
     keep = m >= 0
     out[m[keep]] = values[: m.size][keep]
     return out
+
+
+def moe_init_routing(expert_idx, num_experts, cumsum=False):
+    """Stable sort of the flat (token, route) list by expert, as the reference's CPU stand-in does it
+    (examples/utils/gen_data_moe.py:48-57: argsort(stable=True) of the flat expert indices and a
+    bincount); entries outside [0, num_experts) are dropped (-1 in both maps).  Returns
+    (dst_to_src, src_to_dst, expert_tokens).  Pinned in the tests by torch.argsort / torch.bincount."""
+    flat = np.asarray(expert_idx, dtype=np.int64).reshape(-1)
+    ok = (flat >= 0) & (flat < num_experts)
+    order = np.argsort(np.where(ok, flat, num_experts), kind="stable")
+    n_ok = int(ok.sum())
+    dst_to_src = np.full(flat.size, -1, np.int32)
+    dst_to_src[:n_ok] = order[:n_ok]
+    src_to_dst = np.full(flat.size, -1, np.int32)
+    src_to_dst[order[:n_ok]] = np.arange(n_ok, dtype=np.int32)
+    counts = np.bincount(flat[ok], minlength=num_experts).astype(np.int32)
+    return dst_to_src, src_to_dst, (np.cumsum(counts).astype(np.int32) if cumsum else counts)
