@@ -30,9 +30,12 @@ int main(int argc, char **argv)
     if (argc >= 2 && std::string(argv[1]) == "--list") {
         for (auto &name : OperatorRegistry::Instance().Names()) printf("operator %s\n", name.c_str());
         for (auto &kv : CommTypeMap) {
-            if (KernelDispatcher::GetKernelFunc(kv.second, DataTypeOf(kv.second)))
-                printf("launcher %s type=%d dtype=%d key=%d name=%s\n", kv.first.c_str(), (int)kv.second, (int)DataTypeOf(kv.second),
-                       ((int)kv.second << 8) | (int)DataTypeOf(kv.second), CommTypeOpNameMap.at(kv.second).c_str());
+            for (CocDataType dt : {FP16, INT8, BF16, FP8E4M3FN}) {
+                if (KernelDispatcher::GetKernelFunc(kv.second, dt))
+                    printf("launcher %s type=%d dtype=%d key=%d name=%s%s\n", kv.first.c_str(), (int)kv.second, (int)dt,
+                           ((int)kv.second << 8) | (int)dt, CommTypeOpNameMap.at(kv.second).c_str(),
+                           dt == DataTypeOf(kv.second) ? "" : " (--fp16 1)");
+            }
         }
         return 0;
     }

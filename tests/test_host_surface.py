@@ -39,10 +39,14 @@ def test_registry_and_dispatch_keys_match_reference():
     for l in out.stdout.splitlines():
         if l.startswith("launcher "):
             f = l.split()
-            kv = dict(x.split("=") for x in f[2:])
-            seen[f[1]] = (kv["name"], int(kv["type"]), int(kv["dtype"]), int(kv["key"]))
+            kv = dict(x.split("=") for x in f[2:6])
+            seen.setdefault(f[1], []).append((kv["name"], int(kv["type"]), int(kv["dtype"]), int(kv["key"])))
     for short, (name, ctype, dtype) in EXPECT.items():
-        assert seen[short] == (name, ctype, dtype, (ctype << 8) | dtype)
+        assert (name, ctype, dtype, (ctype << 8) | dtype) in seen[short]
+    # the two down-projection operators also have the half-precision launchers the reference registers (dtype FP16 = 1)
+    for short, ctype in (("a5fp8gmmata", 25), ("a5fp4gmmata", 26)):
+        assert any(e[1:] == (ctype, 1, (ctype << 8) | 1) for e in seen[short])
+    assert sum(len(v) for v in seen.values()) == 10
 
 
 def test_unknown_kernel_and_bad_shape_fail_like_the_reference_main():
