@@ -94,6 +94,29 @@ int cch_gmm_i8_dequant_swiglu(const void *x, const void *w, const int32_t *group
     return run(p, KIND_I8, EPI_DEQUANT_SWIGLU, static_cast<hipStream_t>(stream));
 }
 
+int cch_gmm_i8_dequant(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok, const float *per_ch,
+                       void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k, int trans_b, void *stream)
+{
+    int rc = check_shape("cch_gmm_i8_dequant", t, n, k);
+    if (rc) return rc;
+    CCH_REQUIRE(trans_b == 0 || trans_b == 1, "cch_gmm_i8_dequant: trans_b %d", trans_b);
+    CCH_REQUIRE(num_experts >= 1 && num_experts <= 65535, "cch_gmm_i8_dequant: num_experts=%lld", (long long)num_experts);
+    if (t == 0 || n == 0) return CCH_OK;
+    CCH_REQUIRE(out && per_tok && per_ch && group_sizes && (k == 0 || (x && w)), "cch_gmm_i8_dequant: null pointer");
+    GemmProblem p{};
+    p.a = static_cast<const uint8_t *>(x);
+    p.b = static_cast<const uint8_t *>(w);
+    p.per_tok = per_tok;
+    p.per_ch = per_ch;
+    p.out = static_cast<uint16_t *>(out);
+    p.group_sizes = group_sizes;
+    p.num_groups = (int)num_experts;
+    p.T = (int)t; p.N = (int)n; p.K = (int)k; p.n_out = (int)n;
+    p.trans_b = trans_b;
+    p.b_stride = n * k;
+    return run(p, KIND_I8, EPI_DEQUANT, static_cast<hipStream_t>(stream));
+}
+
 static int mx_problem(const char *who, GemmProblem &p, const void *a, const void *sa, const void *b, const void *sb,
                       const int32_t *group_sizes, void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k,
                       int fmt, int trans_b, int *kind)

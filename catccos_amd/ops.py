@@ -219,9 +219,18 @@ def w8a8_matmul_dequant(a, b, per_tok, per_ch, trans_b=0):
     return out
 
 
+def gmm_dequant(x, w, group_sizes, per_tok, per_ch, trans_b=0):
+    """Grouped int8 matmul + per-token x per-channel dequant (no activation); returns bf16 [T, N]."""
+    return _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, False)
+
+
 def gmm_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, trans_b=0):
     """Grouped int8 matmul + dequant + SwiGLU: x int8 [T,K] grouped by expert, w int8 [E,K,N]
     (or [E,N,K]), group_sizes int32 [E] on the device; returns bf16 [T, N/2]."""
+    return _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, True)
+
+
+def _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, swiglu):
     _require_gpu(x, w, group_sizes, per_tok, per_ch)
     _check_2d("x", x, torch.int8)
     if w.dim() != 3 or w.dtype != torch.int8:
@@ -238,9 +247,9 @@ def gmm_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, trans_b=0):
     per_ch = per_ch.contiguous().float()
     if per_tok.numel() != t or tuple(per_ch.shape) != (e, n):
         raise ValueError("per_tok must be [T] and per_ch [E,N]")
-    out = torch.empty((t, n // 2), dtype=torch.bfloat16, device=x.device)
-    check(_abi.lib().cch_gmm_i8_dequant_swiglu(_ptr(x), _ptr(w), _ptr(group_sizes), _ptr(per_tok), _ptr(per_ch),
-                                               _ptr(out), e, t, n, k, int(trans_b), _stream()))
+    out = torch.empty((t, n // 2 if swiglu else n), dtype=torch.bfloat16, device=x.device)
+    fn = _abi.lib().cch_gmm_i8_dequant_swiglu if swiglu else _abi.lib().cch_gmm_i8_dequant
+    check(fn(_ptr(x), _ptr(w), _ptr(group_sizes), _ptr(per_tok), _ptr(per_ch), _ptr(out), e, t, n, k, int(trans_b), _stream()))
     return out
 
 

@@ -97,6 +97,16 @@ int cch_mx_quant_b(const void *b, void *payload, void *scales, int64_t k, int64_
 int cch_gemm_i8_dequant(const void *a, const void *b, const float *per_tok, const float *per_ch, void *out, int64_t m,
                         int64_t n, int64_t k, int trans_b, void *stream);
 
+/* ---- MoE grouped W8A8 matmul + dequant, without the activation ----------------
+ * The grouped GEMM and per-token dequantisation of AlltoallvGmmDequantKernel
+ * (include/catccos/dgemm/kernel/alltoallv_gmm_dequant_v2.hpp:164-244 with
+ * include/catccos/epilogue/block/block_epilogue_per_token_dequant.hpp:247-266) on their own, i.e.
+ * cch_gmm_i8_dequant_swiglu before its SwiGLU:
+ *   out[r,j] = bf16( float(acc) * per_ch[e,j] * per_tok[r] ), out bf16 [t,n];
+ * operands and grouping as below.  Rows past sum(group_sizes) are written as zeros. */
+int cch_gmm_i8_dequant(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok, const float *per_ch,
+                       void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k, int trans_b, void *stream);
+
 /* ---- MoE grouped W8A8 matmul + dequant + SwiGLU (config 4) -------------------
  * Replaces the grouped GEMM of AlltoallvGmmDequantKernel::operator()<AIC>
  * (include/catccos/dgemm/kernel/alltoallv_gmm_dequant_v2.hpp:164-244) and DequantSwigluKernel

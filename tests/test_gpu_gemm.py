@@ -413,3 +413,33 @@ def test_tiled_matches_generic_on_random_groups(seed):
     scale = max(float(np.sqrt(np.mean(b[:used].astype(np.float64) ** 2))), 1e-30) if used else 1.0
     excess = np.abs(a - b) - (2.0 ** -7 * np.abs(b) + 1e-3 * scale)
     assert excess.max() <= 0, (seed, e, sizes.tolist(), t, k, n, trans_b, kind, float(excess.max()), scale)
+
+
+@pytest.mark.parametrize("trans_b", [0, 1])
+@pytest.mark.parametrize("tiled", [True, False])
+def test_gmm_i8_dequant_without_activation(trans_b, tiled):
+    """Grouped int8 matmul + per-token x per-channel dequant: every group is the dense golden of its rows."""
+    e, t, k, n = 5, 900, 512, 384
+    rng = np.random.default_rng(31 + trans_b)
+    gs = np.array([0, 300, 1, 420, 150], np.int32)            # 29 rows belong to no group
+    x = rng.integers(-127, 128, (t, k)).astype(np.int8)
+    w = rng.integers(-127, 128, (e, k, n)).astype(np.int8)
+    pt = rng.uniform(0.001, 0.02, t).astype(np.float32)
+    pc = rng.uniform(0.001, 0.02, (e, n)).astype(np.float32)
+    want = np.zeros((t, n), np.float32)
+    r0 = 0
+    for g in range(e):
+        r1 = r0 + int(gs[g])
+        if r1 > r0:
+            want[r0:r1] = orc.gemm_i8_dequant(x[r0:r1], w[g], pt[r0:r1], pc[g])
+        r0 = r1
+    ww = np.ascontiguousarray(w.transpose(0, 2, 1)) if trans_b else w
+    cc.set_option("require_tiled_gemm", 1 if tiled else 0)
+    cc.set_option("force_generic_gemm", 0 if tiled else 1)
+    try:
+        got = out_f32(cc.gmm_dequant(dev(x), dev(ww), dev(gs), dev(pt), dev(pc), trans_b))
+    finally:
+        cc.set_option("require_tiled_gemm", 0)
+        cc.set_option("force_generic_gemm", 0)
+    assert (got[r0:] == 0).all()
+    assert_close(got, want, ("gmm i8 dequant", trans_b, tiled))
