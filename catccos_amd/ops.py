@@ -116,11 +116,13 @@ def mx_quant_b(b, fmt="e4m3", rounding=ROUND_RNE, trans_b=0):
 DQ_DEVICE, DQ_GOLDEN = 0, 1
 
 
-def dynamic_quant_i8(x, src_rows=None, topk=1, mode=DQ_DEVICE):
+def dynamic_quant_i8(x, src_rows=None, topk=1, mode=DQ_DEVICE, smooth=None, smooth_rows=None):
     """Per-token dynamic int8 quantisation of a 2-D bf16 tensor, optionally gathering rows.
 
-    Output row i quantises x[src_rows[i] // topk] (x[i] without a row map).  Returns
-    (q int8 [T, K], scale float32 [T]) with scale = amax(row) / 127.
+    Output row i quantises x[src_rows[i] // topk] (x[i] without a row map).  With `smooth`
+    (float32 [S, K] or [K]) every element is first multiplied by its column's entry of vector
+    smooth_rows[i] (vector 0 without `smooth_rows`).  Returns (q int8 [T, K], scale float32 [T])
+    with scale = amax(row) / 127.
     """
     _require_gpu(x)
     if x.dim() != 2 or x.dtype != torch.bfloat16:
@@ -135,10 +137,27 @@ def dynamic_quant_i8(x, src_rows=None, topk=1, mode=DQ_DEVICE):
         t = src_rows.shape[0]
     else:
         t = rows_in
+    if smooth is None and smooth_rows is not None:
+        raise ValueError("smooth_rows needs smooth")
+    if smooth is not None:
+        _require_gpu(smooth)
+        if smooth.dtype != torch.float32 or smooth.dim() not in (1, 2) or smooth.shape[-1] != k:
+            raise ValueError("smooth must be float32 [S, K] or [K]")
+        smooth = smooth.contiguous().view(-1, k)
+        if smooth_rows is not None:
+            _require_gpu(smooth_rows)
+            if smooth_rows.dtype != torch.int32 or smooth_rows.shape != (t,):
+                raise ValueError("smooth_rows must be int32 [T]")
+            smooth_rows = smooth_rows.contiguous()
     q = torch.empty((t, k), dtype=torch.int8, device=x.device)
     scale = torch.empty((t,), dtype=torch.float32, device=x.device)
-    check(_abi.lib().cch_dyn_quant_i8_rows(_ptr(x), _ptr(src_rows) if src_rows is not None else None, _ptr(q), _ptr(scale),
-                                           rows_in, t, k, int(topk), int(mode), _stream()))
+    src_p = _ptr(src_rows) if src_rows is not None else None
+    if smooth is None:
+        check(_abi.lib().cch_dyn_quant_i8_rows(_ptr(x), src_p, _ptr(q), _ptr(scale), rows_in, t, k, int(topk), int(mode), _stream()))
+    else:
+        check(_abi.lib().cch_dyn_quant_i8_rows_smooth(_ptr(x), src_p, _ptr(smooth),
+                                                      _ptr(smooth_rows) if smooth_rows is not None else None, smooth.shape[0],
+                                                      _ptr(q), _ptr(scale), rows_in, t, k, int(topk), int(mode), _stream()))
     return q, scale
 
 

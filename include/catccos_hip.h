@@ -210,8 +210,7 @@ int cch_moe_init_routing(const int32_t *expert_idx, int64_t rows, int num_expert
 
 /* ---- Per-token dynamic int8 quantisation with row gather (feeds config 4) ----
  * Replaces MoeV2GatherDynamicQuant (examples/aux_ops/moe_init_routing_quant_v2/
- * moe_v2_gather_dynamic_quant.h:117-150 Compute, :213-250 the gather loop), without its
- * smoothing vector.
+ * moe_v2_gather_dynamic_quant.h:117-150 Compute, :213-250 the gather loop).
  *   x         bf16 [rows_in, k] row-major
  *   src_rows  int32 [t] or NULL: output row i quantises input row src_rows[i] / topk
  *             (the reference's sorted expanded-row index divided by top-K); a negative
@@ -225,6 +224,15 @@ int cch_moe_init_routing(const int32_t *expert_idx, int64_t rows, int num_expert
 #define CCH_DQ_GOLDEN 1
 int cch_dyn_quant_i8_rows(const void *x, const int32_t *src_rows, void *q, float *scale, int64_t rows_in, int64_t t,
                           int64_t k, int topk, int mode, void *stream);
+/* The same with the reference's smoothing (quantSmooth, moe_v2_gather_dynamic_quant.h:127-130): every
+ * element is multiplied in fp32 by its column's entry of a smoothing vector before the maximum is taken.
+ *   smooth       fp32 [num_smooth, k]
+ *   smooth_rows  int32 [t] or NULL: output row i uses vector smooth_rows[i] (the row's expert, the
+ *                reference's smoothType 2, :241); an index outside [0, num_smooth) gives a zero row
+ *                with scale 0.  NULL: vector 0 for every row (smoothType 1, :170-174). */
+int cch_dyn_quant_i8_rows_smooth(const void *x, const int32_t *src_rows, const float *smooth, const int32_t *smooth_rows,
+                                 int64_t num_smooth, void *q, float *scale, int64_t rows_in, int64_t t, int64_t k, int topk,
+                                 int mode, void *stream);
 
 /* Library switches for tests and benchmarks: "force_generic_gemm" = 1 routes every GEMM entry
  * point through the shape-agnostic one-thread-per-element kernels instead of the tiled MFMA

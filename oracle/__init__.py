@@ -187,8 +187,9 @@ def mx_dequant_rows(payload, scales, k, fmt=E4M3):
 DQ_DEVICE, DQ_GOLDEN = 0, 1
 
 
-def dyn_quant_i8_rows(x_bf16, src=None, topk=1, mode=DQ_DEVICE):
-    """Per-token dynamic int8 quantisation: x uint16 [rows_in,K] -> (q int8 [T,K], scale float32 [T])."""
+def dyn_quant_i8_rows(x_bf16, src=None, topk=1, mode=DQ_DEVICE, smooth=None, smooth_rows=None):
+    """Per-token dynamic int8 quantisation: x uint16 [rows_in,K] -> (q int8 [T,K], scale float32 [T]).
+    smooth float32 [S,K] (or [K]) multiplies every row first; smooth_rows int32 [T] picks its vector."""
     x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
     rows_in, k = x.shape
     if src is not None:
@@ -196,10 +197,19 @@ def dyn_quant_i8_rows(x_bf16, src=None, topk=1, mode=DQ_DEVICE):
         t = src.shape[0]
     else:
         t = rows_in
+    ns = 0
+    if smooth is not None:
+        smooth = np.ascontiguousarray(smooth, dtype=np.float32).reshape(-1, k)
+        ns = smooth.shape[0]
+        if smooth_rows is not None:
+            smooth_rows = np.ascontiguousarray(smooth_rows, dtype=np.int32)
+            assert smooth_rows.shape == (t,)
     q = np.empty((t, k), dtype=np.int8)
     scale = np.empty(t, dtype=np.float32)
     lib().orc_dyn_quant_i8_rows(_p(x), _p(src) if src is not None else None, _i64(rows_in), _i64(t), _i64(k), int(topk),
-                                int(mode), _p(q), _p(scale))
+                                int(mode), _p(smooth) if smooth is not None else None,
+                                _p(smooth_rows) if smooth is not None and smooth_rows is not None else None, _i64(ns),
+                                _p(q), _p(scale))
     return q, scale
 
 

@@ -485,29 +485,42 @@ float orc_trunc_through_f16(float v)
  *   mode 1   the generator's golden (gen_data_dispatch_gmm_dequant_swiglu.py
  *            :275-280): q = rint(x * 127 / amax) in fp32 (ties to even),
  *            scale = amax / 127
+ *   smooth   fp32 [num_smooth, K] or NULL: every element is multiplied (in
+ *            fp32, one rounding) by the smoothing vector of its row before
+ *            anything else (:127-130).  smooth_rows int32 [T] picks the vector
+ *            of output row i (the row's expert, :241); NULL: vector 0 for every
+ *            row (:170-174).  An index outside [0, num_smooth) gives a zero row.
  *   An all-zero row gives q = 0 and scale 0 in both modes (the reference
  *   divides 0 by 0 there).
  * pinned by: mode 1 against torch (abs/max/round on the same data); mode 0
  *            against a numpy restatement built on the brute-force half
  *            truncation; |q| <= 127 with 127 reached in every non-zero row;
- *            |x - q*scale| <= scale (mode 0) and <= scale/2 (mode 1).
+ *            |x - q*scale| <= scale (mode 0) and <= scale/2 (mode 1);
+ *            smoothing: the same two restatements on the fp32 products, and
+ *            power-of-two vectors against the unsmoothed routine on the
+ *            pre-scaled input (the products are then exact bf16 values).
  */
 void orc_dyn_quant_i8_rows(const uint16_t *x, const int32_t *src, int64_t rows_in, int64_t T, int64_t K, int topk,
-                           int mode, int8_t *q, float *scale)
+                           int mode, const float *smooth, const int32_t *smooth_rows, int64_t num_smooth, int8_t *q,
+                           float *scale)
 {
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < T; i++) {
         int64_t r = src ? (src[i] < 0 ? -1 : (int64_t)src[i] / topk) : i;
         int8_t *qo = q + i * K;
-        if (r < 0 || r >= rows_in) {
+        const int64_t sv = smooth ? (smooth_rows ? (int64_t)smooth_rows[i] : 0) : 0;
+        if (r < 0 || r >= rows_in || (smooth && (sv < 0 || sv >= num_smooth))) {
             memset(qo, 0, (size_t)K);
             scale[i] = 0.0f;
             continue;
         }
         const uint16_t *xr = x + r * K;
+        const float *sm = smooth ? smooth + sv * K : NULL;
         float amax = 0.0f;
         for (int64_t k = 0; k < K; k++) {
-            float a = fabsf(orc_bf16_to_f32(xr[k]));
+            float v = orc_bf16_to_f32(xr[k]);
+            if (sm) v = v * sm[k];
+            const float a = fabsf(v);
             if (a > amax) amax = a;
         }
         if (!(amax > 0.0f)) {
@@ -518,7 +531,8 @@ void orc_dyn_quant_i8_rows(const uint16_t *x, const int32_t *src, int64_t rows_i
         const float sc = amax / 127.0f;
         scale[i] = sc;
         for (int64_t k = 0; k < K; k++) {
-            const float v = orc_bf16_to_f32(xr[k]);
+            float v = orc_bf16_to_f32(xr[k]);
+            if (sm) v = v * sm[k];
             float y;
             if (mode == 0) {
                 const float t = orc_trunc_through_f16(v / sc);

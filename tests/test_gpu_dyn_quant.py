@@ -79,3 +79,40 @@ def test_dyn_quant_feeds_grouped_gemm():
     want = orc.gmm_i8_dequant_swiglu(wq, w, gs, ws, pc)
     m = orc.compare(out.float().cpu().numpy(), want)
     assert m["max_rel_floor1"] <= 1e-2 and m["max_rel_floor_rms"] <= 1e-2, m
+
+
+@pytest.mark.parametrize("mode", [cc.DQ_DEVICE, cc.DQ_GOLDEN])
+@pytest.mark.parametrize("shape", [(64, 512), (200, 7168), (17, 1000), (5, 8200), (3, 12288), (2, 7), (3, 16384), (2, 20000)])
+@pytest.mark.parametrize("per_row", [False, True])
+def test_dyn_quant_smoothing_bit_exact(shape, mode, per_row):
+    """Smoothing vectors (one for all rows, or one per expert picked by row), with a gather, a dropped row
+    and vector indices out of range."""
+    rows, k = shape
+    experts, topk = 5, 2
+    rng = np.random.default_rng(rows * 7 + k + mode)
+    xb = rand_rows(rng, rows, k, 2.5)
+    xb[rows // 2] = 0
+    t = rows * topk
+    src = rng.permutation(t).astype(np.int32)
+    src[1] = -1
+    smooth = (rng.uniform(0.2, 5.0, (experts, k)) * np.where(rng.random((experts, k)) < 0.5, -1, 1)).astype(np.float32)
+    idx = None
+    if per_row:
+        idx = rng.integers(0, experts, t).astype(np.int32)
+        idx[0] = experts
+        idx[t - 1] = -3
+    q, s = cc.dynamic_quant_i8(dev_bf16(xb), torch.from_numpy(src).cuda(), topk, mode,
+                               smooth=torch.from_numpy(smooth).cuda(),
+                               smooth_rows=torch.from_numpy(idx).cuda() if per_row else None)
+    torch.cuda.synchronize()
+    wq, ws = orc.dyn_quant_i8_rows(xb, src=src, topk=topk, mode=mode, smooth=smooth, smooth_rows=idx)
+    assert np.array_equal(s.cpu().numpy(), ws)
+    assert np.array_equal(q.cpu().numpy(), wq)
+
+
+def test_dyn_quant_smoothing_arguments():
+    x = torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        cc.dynamic_quant_i8(x, smooth_rows=torch.zeros(4, dtype=torch.int32, device="cuda"))
+    with pytest.raises(ValueError):
+        cc.dynamic_quant_i8(x, smooth=torch.ones(2, 32, device="cuda"))

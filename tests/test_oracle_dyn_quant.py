@@ -81,3 +81,55 @@ def test_properties_and_gather():
             assert np.all(q[i] == 0) and s[i] == 0
         else:
             assert np.array_equal(q[i], q0[sidx // 2]) and s[i] == s0[sidx // 2]
+
+
+def test_smoothing_against_the_two_restatements():
+    """Smoothing multiplies in fp32 first (moe_v2_gather_dynamic_quant.h:127-130); everything after is
+    the unsmoothed arithmetic on the products."""
+    mags = all_halves()
+    rng = np.random.default_rng(4)
+    rows, k, experts = 12, 384, 3
+    xb = rand_rows(rng, rows, k, 2.0)
+    smooth = rng.uniform(0.25, 4.0, (experts, k)).astype(np.float32)
+    idx = rng.integers(0, experts, rows).astype(np.int32)
+    y = (orc.bf16_to_f32(xb) * smooth[idx]).astype(np.float32)
+    amax = np.abs(y).max(axis=1)
+    sc = (amax / np.float32(127.0)).astype(np.float32)
+    # golden mode against torch
+    q, s = orc.dyn_quant_i8_rows(xb, mode=orc.DQ_GOLDEN, smooth=smooth, smooth_rows=idx)
+    yt = torch.from_numpy(y)
+    want = torch.round(yt * 127.0 / torch.from_numpy(amax)[:, None]).to(torch.int8).numpy()
+    assert np.array_equal(q, want) and np.array_equal(s, sc)
+    # device mode against the brute-force half truncation
+    q, s = orc.dyn_quant_i8_rows(xb, mode=orc.DQ_DEVICE, smooth=smooth, smooth_rows=idx)
+    d = (y / sc[:, None]).astype(np.float32)
+    t = mags[np.searchsorted(mags, np.abs(d), side="right") - 1] * np.sign(d)
+    assert np.array_equal(q, (np.sign(t) * np.floor(np.abs(t) + 0.5)).astype(np.int8)) and np.array_equal(s, sc)
+    # one vector for all rows = vector 0
+    q1, s1 = orc.dyn_quant_i8_rows(xb, smooth=smooth[0])
+    q2, s2 = orc.dyn_quant_i8_rows(xb, smooth=smooth, smooth_rows=np.zeros(rows, np.int32))
+    assert np.array_equal(q1, q2) and np.array_equal(s1, s2)
+
+
+def test_power_of_two_smoothing_equals_prescaled_input():
+    """Products with powers of two are exact bf16 values, so the smoothed result is the unsmoothed
+    one of the pre-scaled rows; a vector index out of range gives a zero row."""
+    rng = np.random.default_rng(5)
+    rows, k = 10, 200
+    xb = rand_rows(rng, rows, k)
+    smooth = np.exp2(rng.integers(-3, 4, (4, k))).astype(np.float32)
+    idx = rng.integers(0, 4, rows).astype(np.int32)
+    pre = orc.f32_to_bf16(orc.bf16_to_f32(xb) * smooth[idx])
+    src = rng.permutation(rows * 2).astype(np.int32)[:rows]       # top-2 expanded rows
+    idx[3] = 4
+    idx[7] = -1
+    for mode in (orc.DQ_DEVICE, orc.DQ_GOLDEN):
+        q, s = orc.dyn_quant_i8_rows(xb, src=src, topk=2, mode=mode, smooth=smooth, smooth_rows=idx)
+        for i in range(rows):
+            if idx[i] < 0 or idx[i] >= 4:
+                assert np.all(q[i] == 0) and s[i] == 0
+                continue
+            row = (orc.bf16_to_f32(xb[src[i] // 2]) * smooth[idx[i]]).astype(np.float32)
+            q0, s0 = orc.dyn_quant_i8_rows(orc.f32_to_bf16(row)[None, :], mode=mode)
+            assert np.array_equal(q[i], q0[0]) and s[i] == s0[0]
+    assert pre.shape == xb.shape
