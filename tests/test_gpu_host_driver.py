@@ -158,3 +158,32 @@ def test_dispatch_gmm_swiglu_from_bf16_tokens(tmp_path, words):
     q, s = orc.dyn_quant_i8_rows(xb, order, topk, orc.DQ_DEVICE)
     want = orc.gmm_i8_dequant_swiglu(q, w, gs, s, pc)
     assert_close(bf16_file(tmp_path / "output_0.bin", (m * topk, n // 2)), want)
+
+
+def test_shape_list_walk(tmp_path):
+    """One process walks a test_shapes.csv (header + M,K,N lines, the loop of the reference's run.sh):
+    per-shape data directories, outputs against the oracle."""
+    shapes = [(256, 256, 384), (130, 512, 256)]
+    csv = tmp_path / "test_shapes.csv"
+    csv.write_text("M,K,N\n" + "".join(f"{m},{k},{n}\n" for m, k, n in shapes) + "\n")
+    want = {}
+    for i, (m, k, n) in enumerate(shapes):
+        d = tmp_path / f"{m}_{k}_{n}"
+        d.mkdir()
+        rng = np.random.default_rng(40 + i)
+        pa, sa = orc.mx_quant_rows(rand_bf16(rng, (m, k)), orc.E4M3)
+        pb, sb = orc.mx_quant_b(rand_bf16(rng, (k, n)), orc.E4M3, orc.RNE, 1)
+        for name, arr in (("a", pa), ("b", pb), ("a_scale", sa), ("b_scale", sb)):
+            arr.tofile(d / f"rank_0_{name}.bin")
+        want[(m, k, n)] = orc.mx_gmm(pa, sa, pb, sb, n, k, orc.E4M3, 1)
+    r = subprocess.run([DRIVER, "a5mxfp8mmrs", "--shapes", str(csv), str(tmp_path), "--transB", "1", "--iters", "1", "--warmup", "0"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("Processing test case") == 2 and "2 shapes finished" in r.stdout, r.stdout
+    for (m, k, n), w in want.items():
+        assert_close(bf16_file(tmp_path / f"{m}_{k}_{n}" / "output.bin", (m, n)), w)
+    # perf mode over the same list, and a list that cannot be read
+    r = subprocess.run([DRIVER, "a5mxfp8mmrs", "--shapes", str(csv), "-", "--iters", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.count("[PERF] Avg latency") == 2, r.stdout + r.stderr
+    r = subprocess.run([DRIVER, "a5mxfp8mmrs", "--shapes", str(tmp_path / "missing.csv"), "-"], capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0
