@@ -174,8 +174,9 @@ int cch_mx_gmm_mapped(const void *a, const void *sa, const void *b, const void *
     GemmProblem p{};
     int kind = 0;
     CCH_REQUIRE(group_sizes != nullptr || t == 0, "cch_mx_gmm_mapped: null group_sizes");
-    CCH_REQUIRE(out_row_map != nullptr || t == 0, "cch_mx_gmm_mapped: null out_row_map");
     CCH_REQUIRE(out_rows >= 0 && out_rows < ((int64_t)1 << 31), "cch_mx_gmm_mapped: out_rows=%lld", (long long)out_rows);
+    CCH_REQUIRE(out_row_map != nullptr || out_rows == t, "cch_mx_gmm_mapped: without a row map out has t=%lld rows, not %lld",
+                (long long)t, (long long)out_rows);
     CCH_REQUIRE(out_dtype == CCH_OUT_BF16 || out_dtype == CCH_OUT_FP16, "cch_mx_gmm_mapped: out_dtype %d", out_dtype);
     int rc = mx_problem("cch_mx_gmm_mapped", p, a, sa, b, sb, group_sizes, out, num_experts, t, n, k, fmt, trans_b, &kind);
     if (rc) return rc;

@@ -49,6 +49,11 @@ void LaunchAscend950Fp4MxAllToAllVGroupedMatmulBF16(void *, uint32_t, uint64_t, 
 void LaunchAscend950Fp8MxAllToAllVGroupedMatmulBF16(void *, uint32_t, uint64_t, KernelParams &, uint8_t *, uint8_t *,
                                                     CocTilingParams &, uint32_t, uint32_t);
 
+void LaunchAscend950Fp4MxAllToAllVGroupedMatmulFP16(void *, uint32_t, uint64_t, KernelParams &, uint8_t *, uint8_t *,
+                                                    CocTilingParams &, uint32_t, uint32_t);
+void LaunchAscend950Fp8MxAllToAllVGroupedMatmulFP16(void *, uint32_t, uint64_t, KernelParams &, uint8_t *, uint8_t *,
+                                                    CocTilingParams &, uint32_t, uint32_t);
+
 void LaunchAscend950Fp8MxGroupedMatmulAllToAllVBF16(void *, uint32_t, uint64_t, KernelParams &, uint8_t *, uint8_t *,
                                                     CocTilingParams &, uint32_t, uint32_t);
 void LaunchAscend950Fp4MxGroupedMatmulAllToAllVBF16(void *, uint32_t, uint64_t, KernelParams &, uint8_t *, uint8_t *,

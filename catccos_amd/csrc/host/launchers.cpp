@@ -81,6 +81,27 @@ void LaunchAscend950Fp8MxAllToAllVGroupedMatmulBF16(void *stream, uint32_t, uint
            stream, "Ascend950Fp8MxAllToAllVGroupedMatmul");
 }
 
+// The reference registers the two operators above for fp16 output (launch_map.h:100-101): the same
+// matmul through the entry point that takes an output type, without a row map.
+static void MxAllToAllVGroupedMatmulFP16(void *stream, KernelParams &p, CocTilingParams &t, uint32_t transB, int fmt, const char *what)
+{
+    Finish(cch_mx_gmm_mapped(p.ptrA, p.customPtrs[0], p.ptrB, p.customPtrs[1], reinterpret_cast<const int32_t *>(p.customPtrs[3]),
+                             nullptr, p.ptrC, t.m, CCH_OUT_FP16, t.expertNum, t.m, t.n, t.k, fmt, (int)transB, stream),
+           stream, what);
+}
+
+void LaunchAscend950Fp4MxAllToAllVGroupedMatmulFP16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
+                                                    CocTilingParams &t, uint32_t, uint32_t transB)
+{
+    MxAllToAllVGroupedMatmulFP16(stream, p, t, transB, CCH_FMT_E2M1, "Ascend950Fp4MxAllToAllVGroupedMatmul");
+}
+
+void LaunchAscend950Fp8MxAllToAllVGroupedMatmulFP16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
+                                                    CocTilingParams &t, uint32_t, uint32_t transB)
+{
+    MxAllToAllVGroupedMatmulFP16(stream, p, t, transB, CCH_FMT_E4M3, "Ascend950Fp8MxAllToAllVGroupedMatmul");
+}
+
 // Down projection.  The reference registers these two operators for fp16 output only
 // (tests/dynamic_tiling/impl/kernel_fp16_ascend950.cpp:446-485, launch_map.h:98-99); this build has
 // that launcher and a bf16 twin, which the driver uses by default like for every other operator.
@@ -128,3 +149,5 @@ static AutoRegister s_reg6(ASCEND950_FP8_MX_GROUPED_MATMUL_ALLTOALLV, BF16, &Lau
 static AutoRegister s_reg7(ASCEND950_FP4_MX_GROUPED_MATMUL_ALLTOALLV, BF16, &LaunchAscend950Fp4MxGroupedMatmulAllToAllVBF16);
 static AutoRegister s_reg8(ASCEND950_FP8_MX_GROUPED_MATMUL_ALLTOALLV, FP16, &LaunchAscend950Fp8MxGroupedMatmulAllToAllVFP16);
 static AutoRegister s_reg9(ASCEND950_FP4_MX_GROUPED_MATMUL_ALLTOALLV, FP16, &LaunchAscend950Fp4MxGroupedMatmulAllToAllVFP16);
+static AutoRegister s_reg10(ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL, FP16, &LaunchAscend950Fp4MxAllToAllVGroupedMatmulFP16);
+static AutoRegister s_reg11(ASCEND950_FP8_MX_ALLTOALLV_GROUPED_MATMUL, FP16, &LaunchAscend950Fp8MxAllToAllVGroupedMatmulFP16);

@@ -308,9 +308,9 @@ def mx_matmul(a, sa, b, sb, fmt="e4m3", trans_b=0):
     return out
 
 
-def mx_grouped_matmul(a, sa, b, sb, group_sizes, fmt="e4m3", trans_b=0):
+def mx_grouped_matmul(a, sa, b, sb, group_sizes, fmt="e4m3", trans_b=0, out_dtype=torch.bfloat16):
     """MX grouped GEMM: rows of a grouped by expert (group_sizes int32 [E] on the device),
-    b [E,...] / sb [E,...] one operand per expert; bf16 [T,N]."""
+    b [E,...] / sb [E,...] one operand per expert; bf16 (or, with out_dtype=torch.float16, half) [T,N]."""
     _require_gpu(a, sa, b, sb, group_sizes)
     if group_sizes.dtype != torch.int32 or group_sizes.dim() != 1:
         raise ValueError("group_sizes must be a 1-D int32 tensor")
@@ -318,9 +318,15 @@ def mx_grouped_matmul(a, sa, b, sb, group_sizes, fmt="e4m3", trans_b=0):
     fmt, t, n, k, e = _mx_shapes(a, sa, b, sb, fmt, trans_b, True)
     if group_sizes.numel() != e:
         raise ValueError("group_sizes must have one entry per expert")
-    out = torch.empty((t, n), dtype=torch.bfloat16, device=a.device)
-    check(_abi.lib().cch_mx_gmm(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(group_sizes), _ptr(out), e, t, n, k, fmt,
-                                int(trans_b), _stream()))
+    if out_dtype not in (torch.bfloat16, torch.float16):
+        raise ValueError("out_dtype must be torch.bfloat16 or torch.float16")
+    out = torch.empty((t, n), dtype=out_dtype, device=a.device)
+    if out_dtype == torch.float16:
+        check(_abi.lib().cch_mx_gmm_mapped(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(group_sizes), None, _ptr(out), t, 1, e,
+                                           t, n, k, fmt, int(trans_b), _stream()))
+    else:
+        check(_abi.lib().cch_mx_gmm(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(group_sizes), _ptr(out), e, t, n, k, fmt,
+                                    int(trans_b), _stream()))
     return out
 
 

@@ -150,6 +150,9 @@ int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, con
  *   out_row_map  int32 [t]: row of `out` that receives the result of row i of a; negative or
  *                >= out_rows = dropped.
  *                Entries of rows past sum(group_sizes) are ignored (those rows produce nothing).
+ *                NULL: no mapping, out_rows == t, and the call is cch_mx_gmm with a choice of output
+ *                type (rows past sum(group_sizes) zero-filled) - the fp16 launchers of the
+ *                AllToAllVGroupedMatmul operators (tests/dynamic_tiling/include/launch_map.h:100-101).
  *   out          [out_rows, n] of out_dtype; rows that the map does not name are not written
  *   out_dtype    CCH_OUT_BF16, or CCH_OUT_FP16 (IEEE half, the type the reference registers these
  *                operators for); fp32 accumulators are rounded to nearest even either way

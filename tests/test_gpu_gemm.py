@@ -443,3 +443,32 @@ def test_gmm_i8_dequant_without_activation(trans_b, tiled):
         cc.set_option("force_generic_gemm", 0)
     assert (got[r0:] == 0).all()
     assert_close(got, want, ("gmm i8 dequant", trans_b, tiled))
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e2m1"])
+@pytest.mark.parametrize("tiled", [True, False])
+def test_mx_gmm_half_output_without_a_row_map(fmt, tiled):
+    """out_dtype float16 on the plain grouped matmul: same accumulators, rounded to half; rows of no
+    group are zero-filled as in the bf16 call."""
+    ofmt = orc.E4M3 if fmt == "e4m3" else orc.E2M1
+    e, t, k, n = 3, 700, 512, 384
+    rng = np.random.default_rng(9)
+    gs = np.array([300, 0, 370], np.int32)             # 30 rows belong to no group
+    pa, sa = orc.mx_quant_rows(rand_bf16(rng, (t, k), 1.0), ofmt)
+    pbs, sbs = zip(*[orc.mx_quant_b(rand_bf16(rng, (k, n), 1.0), ofmt, orc.RNE, 0) for _ in range(e)])
+    pb, sb = np.stack(pbs), np.stack(sbs)
+    gold = orc.mx_gmm(pa, sa, pb, sb, n, k, ofmt, 0, group_sizes=gs)
+    cc.set_option("require_tiled_gemm", 1 if tiled else 0)
+    cc.set_option("force_generic_gemm", 0 if tiled else 1)
+    try:
+        h = cc.mx_grouped_matmul(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), fmt, 0, out_dtype=torch.float16)
+        b = cc.mx_grouped_matmul(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), fmt, 0)
+        torch.cuda.synchronize()
+    finally:
+        cc.set_option("require_tiled_gemm", 0)
+        cc.set_option("force_generic_gemm", 0)
+    assert h.dtype == torch.float16 and b.dtype == torch.bfloat16
+    hf, bf = h.float().cpu().numpy(), b.float().cpu().numpy()
+    assert (hf[670:] == 0).all() and (bf[670:] == 0).all()
+    assert_close(hf, gold, ("fp16 out", fmt, tiled))
+    assert np.abs(hf - gold).mean() < 0.2 * np.abs(bf - gold).mean()

@@ -88,8 +88,9 @@ def test_dispatch_gmm_swiglu_files(tmp_path):
     assert_close(bf16_file(tmp_path / "output_0.bin", (t, n // 2)), orc.gmm_i8_dequant_swiglu(x, w, gs, pt, pc))
 
 
+@pytest.mark.parametrize("fp16", [0, 1])
 @pytest.mark.parametrize("kernel,fmt", [("a5fp4mxatavgmm", orc.E2M1), ("a5fp8mxatavgmm", orc.E4M3)])
-def test_mx_grouped_files(tmp_path, kernel, fmt):
+def test_mx_grouped_files(tmp_path, kernel, fmt, fp16):
     """The reference's own shape for this operator: 1024 x 256 x 256, 4 experts (test_shapes.csv)."""
     e, t, k, n = 4, 1024, 256, 256
     rng = np.random.default_rng(4)
@@ -100,8 +101,12 @@ def test_mx_grouped_files(tmp_path, kernel, fmt):
     pa.tofile(tmp_path / "input_a_0.bin"); pb.tofile(tmp_path / "input_b_0.bin")
     sa.tofile(tmp_path / "input_a_scale_0.bin"); sb.tofile(tmp_path / "input_b_scale_0.bin")
     gs.tofile(tmp_path / "global_tokens_per_local_expert_0.bin")
-    drive(tmp_path, kernel, t, k, n, tmp_path, "--experts", e, "--iters", 1, "--warmup", 0)
-    assert_close(bf16_file(tmp_path / "output_0.bin", (t, n)), orc.mx_gmm(pa, sa, pb, sb, n, k, fmt, 0, group_sizes=gs))
+    drive(tmp_path, kernel, t, k, n, tmp_path, "--experts", e, "--fp16", fp16, "--iters", 1, "--warmup", 0)
+    if fp16:
+        got = np.fromfile(tmp_path / "output_0.bin", dtype=np.float16).astype(np.float32).reshape(t, n)
+    else:
+        got = bf16_file(tmp_path / "output_0.bin", (t, n))
+    assert_close(got, orc.mx_gmm(pa, sa, pb, sb, n, k, fmt, 0, group_sizes=gs))
 
 
 @pytest.mark.parametrize("fp16", [0, 1])

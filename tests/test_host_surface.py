@@ -43,10 +43,11 @@ def test_registry_and_dispatch_keys_match_reference():
             seen.setdefault(f[1], []).append((kv["name"], int(kv["type"]), int(kv["dtype"]), int(kv["key"])))
     for short, (name, ctype, dtype) in EXPECT.items():
         assert (name, ctype, dtype, (ctype << 8) | dtype) in seen[short]
-    # the two down-projection operators also have the half-precision launchers the reference registers (dtype FP16 = 1)
-    for short, ctype in (("a5fp8gmmata", 25), ("a5fp4gmmata", 26)):
+    # the four MX grouped operators also have the half-precision launchers the reference registers
+    # (dtype FP16 = 1, launch_map.h:98-101)
+    for short, ctype in (("a5fp8gmmata", 25), ("a5fp4gmmata", 26), ("a5fp8mxatavgmm", 27), ("a5fp4mxatavgmm", 28)):
         assert any(e[1:] == (ctype, 1, (ctype << 8) | 1) for e in seen[short])
-    assert sum(len(v) for v in seen.values()) == 10
+    assert sum(len(v) for v in seen.values()) == 12
 
 
 def test_unknown_kernel_and_bad_shape_fail_like_the_reference_main():
