@@ -29,6 +29,7 @@
 // tile loop of BlockMmadSchedulerAllToAllVAllGather
 // (include/catccos/dgemm/block/block_scheduler_alltoallv_allgather.hpp:122-168) and the epilogues
 // include/catccos/epilogue/block/block_epilogue_per_token_dequant[_swiglu].hpp.
+#include <atomic>
 #include <type_traits>
 #include <utility>
 
@@ -701,14 +702,16 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 template <int KIND, int EPI, int FMT, int TB>
 static int launch_tile_t(const GemmProblem &p, hipStream_t stream)
 {
-    static bool attr_set = false;
+    // the LDS size attribute is set once per device and kernel; setting it twice from two threads is harmless
+    static std::atomic<uint64_t> attr_set{0};
     auto kern = gemm_tile_kernel<KIND, EPI, FMT, TB>;
-    if (!attr_set) {
-        CCH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
-        attr_set = true;
-    }
     int dev = 0, cus = 0;
     CCH_HIP(hipGetDevice(&dev));
+    const uint64_t dev_bit = (uint64_t)1 << (dev & 63);
+    if (dev >= 64 || !(attr_set.load(std::memory_order_acquire) & dev_bit)) {
+        CCH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
+        attr_set.fetch_or(dev_bit, std::memory_order_release);
+    }
     CCH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     constexpr int bn_out = EPI == EPI_DEQUANT_SWIGLU ? BN / 2 : BN;
     const int64_t row_tiles = (p.T + BM - 1) / BM + (p.group_sizes ? p.num_groups : 0);  // upper bound
