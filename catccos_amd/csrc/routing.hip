@@ -7,7 +7,7 @@
 // MoeV2SrcToDstOp inverts the permutation, MoeV2ExpertTokenOut counts) and its CPU stand-in
 // (examples/utils/gen_data_moe.py:48-57: torch.argsort(stable=True) + bincount).  Keys are small
 // integers, so the sort is a counting sort in three launches: per-chunk histograms, one scan over
-// (expert, chunk), and a placement pass in which one wave walks its chunk in order.
+// (expert, chunk), and a placement pass in which four waves walk their quarters of a chunk in order.
 #include <algorithm>
 
 #include "common.h"
@@ -40,72 +40,115 @@ __global__ __launch_bounds__(256) void route_histogram_kernel(const int32_t *__r
 }
 
 // In-place exclusive scan of hist in (expert, chunk) order: hist[e * nchunks + c] becomes the first
-// sorted position of expert e's rows of chunk c.  One workgroup; also writes the per-expert token
-// counts (or their running sum).
+// sorted position of expert e's rows of chunk c.  One workgroup of 16 waves: a wave sums the
+// (contiguous) row of an expert, the per-expert totals are scanned across the workgroup, and the
+// wave then scans its rows 64 chunks at a time from the expert's start.  Also writes the
+// per-expert token counts (or their running sum).
 __global__ __launch_bounds__(1024) void route_scan_kernel(int32_t *__restrict__ hist, int experts, int nchunks,
                                                           int32_t *__restrict__ expert_tokens, int cumsum)
 {
-    __shared__ int32_t part[1024];
-    __shared__ int32_t carry;
-    const int n = experts * nchunks;
-    if (threadIdx.x == 0) carry = 0;
+    __shared__ int32_t part[1024];   // per-expert totals, then their inclusive scan (experts <= 1024)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    part[threadIdx.x] = 0;
     __syncthreads();
-    for (int base = 0; base < n; base += 1024) {
-        const int i = base + threadIdx.x;
-        const int v = i < n ? hist[i] : 0;
-        part[threadIdx.x] = v;
+    for (int e = wave; e < experts; e += 16) {
+        int sum = 0;
+        for (int c = lane; c < nchunks; c += 64) sum += hist[(size_t)e * nchunks + c];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
+        if (lane == 0) part[e] = sum;
+    }
+    __syncthreads();
+    const int own = part[threadIdx.x];
+    // Hillis-Steele inclusive scan over the 1024 totals
+    for (int off = 1; off < 1024; off <<= 1) {
+        const int add = threadIdx.x >= off ? part[threadIdx.x - off] : 0;
         __syncthreads();
-        // Hillis-Steele inclusive scan over the 1024 entries
-        for (int off = 1; off < 1024; off <<= 1) {
-            const int add = threadIdx.x >= off ? part[threadIdx.x - off] : 0;
-            __syncthreads();
-            part[threadIdx.x] += add;
-            __syncthreads();
-        }
-        const int incl = part[threadIdx.x], c0 = carry;
-        if (i < n) hist[i] = c0 + incl - v;
-        __syncthreads();
-        if (threadIdx.x == 1023) carry = c0 + incl;
+        part[threadIdx.x] += add;
         __syncthreads();
     }
-    // tokens per expert from the scanned starts
-    const int total = carry;
-    for (int e = threadIdx.x; e < experts; e += 1024) {
-        const int start = hist[(size_t)e * nchunks];
-        const int end = e + 1 < experts ? hist[(size_t)(e + 1) * nchunks] : total;
-        expert_tokens[e] = cumsum ? end : end - start;
+    if ((int)threadIdx.x < experts) expert_tokens[threadIdx.x] = cumsum ? part[threadIdx.x] : own;
+    for (int e = wave; e < experts; e += 16) {
+        int run = e > 0 ? part[e - 1] : 0;   // first position of expert e
+        for (int c0 = 0; c0 < nchunks; c0 += 64) {
+            const int c = c0 + lane;
+            const int v = c < nchunks ? hist[(size_t)e * nchunks + c] : 0;
+            int incl = v;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int up = __shfl_up(incl, off, 64);
+                if (lane >= off) incl += up;
+            }
+            if (c < nchunks) hist[(size_t)e * nchunks + c] = run + incl - v;
+            run += __shfl(incl, 63, 64);
+        }
     }
 }
 
-// One wave per chunk walks its rows in order, 64 at a time.  Inside a group of 64 the rank of a
-// row among the rows of the same expert comes from a ballot per distinct expert value; the
-// running position of every expert lives in LDS.
-__global__ __launch_bounds__(64) void route_place_kernel(const int32_t *__restrict__ expert_idx, int rows, int experts, int nchunks,
-                                                         const int32_t *__restrict__ starts, int32_t *__restrict__ dst_to_src,
-                                                         int32_t *__restrict__ src_to_dst)
+// Lanes of the wave that hold the same key as this lane (keys below 2^bits; lanes with
+// routed == false match nobody): one ballot per key bit.
+__device__ __forceinline__ uint64_t same_key_lanes(int key, bool routed, int bits)
 {
-    __shared__ int32_t next[ROUTE_MAX_EXPERTS];
-    const int lane = threadIdx.x;
-    for (int e = lane; e < experts; e += 64) next[e] = starts[(size_t)e * nchunks + blockIdx.x];
+    uint64_t m = __ballot(routed);
+    for (int b = 0; b < bits; b++) {
+        const uint64_t set = __ballot(routed && ((key >> b) & 1));
+        m &= ((key >> b) & 1) ? set : ~set;
+    }
+    return routed ? m : 0;
+}
+
+// Four waves per chunk, 256 consecutive rows each, 64 at a time.  Inside a group of 64 the rank
+// of a row among the rows of the same expert is a population count over the lanes that hold the
+// same key; a wave first counts its rows per expert, the counts of the waves before it (and the
+// chunk's scanned start) give its first position per expert, and a second walk over the same
+// rows hands the positions out in order.  A wave's LDS accesses execute in program order, so
+// "all lanes read the counter, then the first lane of each key moves it on" needs no barrier.
+constexpr int ROUTE_WAVES = 4;
+constexpr int ROUTE_GROUPS = ROUTE_CHUNK / 64 / ROUTE_WAVES;   // groups of 64 rows per wave
+__global__ __launch_bounds__(64 * ROUTE_WAVES) void route_place_kernel(const int32_t *__restrict__ expert_idx, int rows, int experts,
+                                                                      int nchunks, int bits, const int32_t *__restrict__ starts,
+                                                                      int32_t *__restrict__ dst_to_src,
+                                                                      int32_t *__restrict__ src_to_dst)
+{
+    __shared__ int32_t cnt[ROUTE_WAVES][ROUTE_MAX_EXPERTS];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    for (int e = threadIdx.x; e < experts; e += 64 * ROUTE_WAVES) {
+#pragma unroll
+        for (int v = 0; v < ROUTE_WAVES; v++) cnt[v][e] = 0;
+    }
     __syncthreads();
-    const int base = blockIdx.x * ROUTE_CHUNK;
-    for (int i = 0; i < ROUTE_CHUNK; i += 64) {
-        const int r = base + i + lane;
+    const int base = blockIdx.x * ROUTE_CHUNK + w * (ROUTE_GROUPS * 64);
+    const uint64_t below = (1ull << lane) - 1ull;
+    int key[ROUTE_GROUPS];
+    uint64_t same[ROUTE_GROUPS];
+#pragma unroll
+    for (int g = 0; g < ROUTE_GROUPS; g++) {
+        const int r = base + g * 64 + lane;
         const int e = r < rows ? expert_idx[r] : -1;
         const bool routed = e >= 0 && e < experts;
-        int pos = -1;
-        uint64_t remaining = __ballot(routed);
-        while (remaining) {   // wave-uniform: one round per distinct expert among the 64 rows
-            const int leader = __ffsll((long long)remaining) - 1;
-            const int v = __builtin_amdgcn_readlane(e, leader);
-            const uint64_t same = __ballot(routed && e == v);
-            const int first = next[v];
-            if (routed && e == v) pos = first + __popcll(same & ((1ull << lane) - 1ull));
-            __syncthreads();   // every lane has read next[v] before the leader moves it on
-            if (lane == leader) next[v] = first + __popcll(same);
-            __syncthreads();
-            remaining &= ~same;
+        key[g] = routed ? e : -1;
+        same[g] = same_key_lanes(e, routed, bits);
+        if (routed && (same[g] & below) == 0) cnt[w][e] += __popcll(same[g]);   // first lane of its key
+    }
+    __syncthreads();
+    // counts -> first positions: the chunk's start per expert, then the waves in order
+    for (int e = threadIdx.x; e < experts; e += 64 * ROUTE_WAVES) {
+        int run = starts[(size_t)e * nchunks + blockIdx.x];
+#pragma unroll
+        for (int v = 0; v < ROUTE_WAVES; v++) {
+            const int c = cnt[v][e];
+            cnt[v][e] = run;
+            run += c;
         }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < ROUTE_GROUPS; g++) {
+        const int r = base + g * 64 + lane;
+        const bool routed = key[g] >= 0;
+        int pos = -1;
+        if (routed) pos = cnt[w][key[g]] + __popcll(same[g] & below);
+        if (routed && (same[g] & below) == 0) cnt[w][key[g]] += __popcll(same[g]);
         if (r < rows) {
             src_to_dst[r] = pos;
             if (pos >= 0) dst_to_src[pos] = r;
@@ -142,8 +185,10 @@ extern "C" int cch_moe_init_routing(const int32_t *expert_idx, int64_t rows, int
     hipLaunchKernelGGL(route_histogram_kernel, dim3((unsigned)nchunks), dim3(256), 0, s, expert_idx, (int)rows, num_experts,
                        (int)nchunks, hist, dst_to_src);
     hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, hist, num_experts, (int)nchunks, expert_tokens, cumsum);
+    int bits = 0;
+    while ((1 << bits) < num_experts) bits++;
     if (rows > 0)
-        hipLaunchKernelGGL(route_place_kernel, dim3((unsigned)nchunks), dim3(64), 0, s, expert_idx, (int)rows, num_experts,
-                           (int)nchunks, hist, dst_to_src, src_to_dst);
+        hipLaunchKernelGGL(route_place_kernel, dim3((unsigned)nchunks), dim3(64 * ROUTE_WAVES), 0, s, expert_idx, (int)rows,
+                           num_experts, (int)nchunks, bits, hist, dst_to_src, src_to_dst);
     return launch_status("route kernels");
 }
