@@ -358,6 +358,30 @@ def main():
         extra["moe_token_unpermute_top2"] = {"gb_per_s": round(un_bytes / un_us / 1e3, 1), "frac_of_hbm_peak": round(un_bytes / un_us / 1e3 / HBM_PEAK_GBS, 4),
                                              "us": round(un_us, 2), "bytes": un_bytes}
         del ys, out_u
+        # routing sort of config 4's routes (8192 tokens, top-2, 16 experts): three short launches through the C ABI
+        rt_rows, rt_e = 8192 * 2, 16
+        rt_idx = torch.randint(0, rt_e, (rt_rows,), dtype=torch.int32, device=dev)
+        rt_d2s = torch.empty(rt_rows, dtype=torch.int32, device=dev)
+        rt_s2d = torch.empty_like(rt_d2s)
+        rt_cnt = torch.empty(rt_e, dtype=torch.int32, device=dev)
+        rt_wsb = int(_abi.lib().cch_moe_init_routing_workspace_bytes(rt_rows, rt_e))
+        rt_ws = torch.empty(max(rt_wsb, 4), dtype=torch.uint8, device=dev)
+
+        def rt_launch():
+            _abi.check(_abi.lib().cch_moe_init_routing(rt_idx.data_ptr(), rt_rows, rt_e, rt_d2s.data_ptr(), rt_s2d.data_ptr(),
+                                                       rt_cnt.data_ptr(), 0, rt_ws.data_ptr(), rt_wsb, st4))
+
+        for _ in range(200):
+            rt_launch()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(100):
+            rt_launch()
+        e1.record()
+        torch.cuda.synchronize()
+        extra["moe_init_routing_cfg4_routes"] = {"us": round(e0.elapsed_time(e1) * 1e3 / 100, 2), "routes": rt_rows, "experts": rt_e,
+                                                 "launches_per_call": 3}
         # config 5: MXFP4 grouped (same groups as the headline)
         a5, sa5 = cc.mx_quant((torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16), "e2m1")
         b5 = torch.empty((E, K, N // 2), dtype=torch.uint8, device=dev)
