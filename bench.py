@@ -391,6 +391,22 @@ def main():
         t5 = [queue_time_ms(lambda: cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", TRANS_B), 30, 60.0)]
         extra["mxfp4_grouped_cfg5"] = {"tflops": round(flop / (np.mean(t5) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t5)) * 1e3, 1)}
         extra["mxfp4_grouped_cfg5"]["frac_of_fp4_peak"] = round(extra["mxfp4_grouped_cfg5"]["tflops"] / FP4_PEAK_TFLOPS, 4)
+        del a5, sa5, b5, sb5
+        # Yardstick, not part of this build: the vendor library's dense FP8 GEMM (per-tensor scales, E4M3,
+        # bf16 out) on the headline's shape as one group, and this kernel on the same bytes with unit scales.
+        try:
+            ya = (torch.randn(T, K, device=dev) * 0.5).to(torch.float8_e4m3fn)
+            yb = (torch.randn(N, K, device=dev) * 0.5).to(torch.float8_e4m3fn)
+            one = torch.tensor(1.0, device=dev)
+            t_lib = queue_time_ms(lambda: torch._scaled_mm(ya, yb.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16), 100, 150.0)
+            ysa = torch.full((T, K // 32), 127, dtype=torch.uint8, device=dev)
+            ysb = torch.full((N, K // 32), 127, dtype=torch.uint8, device=dev)
+            t_own = queue_time_ms(lambda: cc.mx_matmul(ya.view(torch.uint8), ysa, yb.view(torch.uint8), ysb, "e4m3", 1), 100, 150.0)
+            extra["yardstick_dense_fp8_16384x4096x7168"] = {
+                "library_scaled_mm_tflops": round(flop / (t_lib * 1e-3) / 1e12, 1), "this_kernel_same_data_tflops": round(flop / (t_own * 1e-3) / 1e12, 1),
+                "note": "library = torch._scaled_mm (per-tensor scales); both with B as [N,K]"}
+        except Exception as exc:   # the library call is optional: a box without it still reports everything else
+            extra["yardstick_dense_fp8_16384x4096x7168"] = {"error": repr(exc)[:200]}
         result["extra"] = extra
 
     print(json.dumps(result), flush=True)
