@@ -12,10 +12,14 @@ bool gemm_tile_supports(const GemmProblem &p, int kind, int epi);
 
 static std::atomic<int> g_force_generic{0};
 static std::atomic<int> g_require_tiled{0};
+static std::atomic<int> g_tile_order{-1};   // -1: chosen per problem
 
-static int run(const GemmProblem &p, int kind, int epi, hipStream_t stream)
+static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
 {
-    if (p.T == 0 || p.n_out == 0) return CCH_OK;
+    if (prob.T == 0 || prob.n_out == 0) return CCH_OK;
+    GemmProblem p = prob;
+    const int order = g_tile_order.load();
+    p.tile_order = order >= 0 ? order : (p.group_sizes != nullptr && p.num_groups > 1);
     if (!g_force_generic.load() && gemm_tile_supports(p, kind, epi)) return launch_gemm_tile(p, kind, epi, stream);
     if (g_require_tiled.load())
         return fail(CCH_ENOSUP, "the tiled MFMA kernels do not take this problem (T=%d N=%d K=%d trans_b=%d) and "
@@ -44,6 +48,10 @@ int cch_set_option(const char *name, int value)
     }
     if (strcmp(name, "require_tiled_gemm") == 0) {
         g_require_tiled.store(value);
+        return CCH_OK;
+    }
+    if (strcmp(name, "gemm_tile_order") == 0) {
+        g_tile_order.store(value);
         return CCH_OK;
     }
     return fail(CCH_EINVAL, "cch_set_option: unknown option %s", name);

@@ -271,6 +271,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         c.valid = t < total_tiles;
         c.lim = c.valid ? 0x7FFFFFFFu : 0u;
         t = max(min(t, total_tiles - 1), 0);
+        if (p.tile_order == 1 && (gridDim.x & 7) == 0 && t < total_tiles - total_tiles % (int)gridDim.x) {
+            // Workgroup w of a round runs on XCD w % 8: give each XCD a run of gridDim.x / 8
+            // consecutive tiles of the round (whole row tiles next to each other), so that its L2
+            // fetches one or two A panels and the B panels of one or two experts per round.
+            const int G = gridDim.x, j = t / G, w = t - j * G;
+            t = j * G + (w & 7) * (G >> 3) + (w >> 3);
+        }
         const int tr = t / n_tiles, nt = t - tr * n_tiles;
         c.e = uniform(find_group(tab, p.num_groups, tr));
         c.m0 = uniform(tab.row_start[c.e] + (tr - tab.tile_start[c.e]) * BM);

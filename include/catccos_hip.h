@@ -240,7 +240,11 @@ int cch_dyn_quant_i8_rows_smooth(const void *x, const int32_t *src_rows, const f
 /* Library switches for tests and benchmarks: "force_generic_gemm" = 1 routes every GEMM entry
  * point through the shape-agnostic one-thread-per-element kernels instead of the tiled MFMA
  * kernels; "require_tiled_gemm" = 1 makes a GEMM entry point return CCH_ENOSUP instead of
- * falling back to them when the tiled kernels do not take the problem. */
+ * falling back to them when the tiled kernels do not take the problem; "gemm_tile_order" picks the
+ * order in which the persistent workgroups of the tiled kernels walk the output tiles: 0 = row-major
+ * over (row tile, column tile), 1 = each XCD takes a run of consecutive tiles of every round (whole
+ * row tiles next to each other: fewer token and weight panels per L2), -1 (default) = 1 for grouped
+ * problems, 0 for dense ones.  Results do not depend on it. */
 int cch_set_option(const char *name, int value);
 
 #ifdef __cplusplus

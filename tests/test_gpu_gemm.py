@@ -472,3 +472,35 @@ def test_mx_gmm_half_output_without_a_row_map(fmt, tiled):
     assert (hf[670:] == 0).all() and (bf[670:] == 0).all()
     assert_close(hf, gold, ("fp16 out", fmt, tiled))
     assert np.abs(hf - gold).mean() < 0.2 * np.abs(bf - gold).mean()
+
+
+# ---------------------------------------------------------------- tile order
+
+def test_grouped_tile_order_covers_every_tile_once():
+    """More tiles than workgroups (several rounds and a partial last one), so the per-XCD tile order of
+    the grouped kernels is in force: every tile must still be computed exactly once.  The output equals
+    the row-major order's bit for bit (each tile accumulates in the same order), and the oracle's."""
+    e, t, k, n = 7, 4700, 256, 4096
+    rng = np.random.default_rng(11)
+    gs = np.array([900, 0, 1300, 37, 256, 1700, 507], np.int32)
+    assert gs.sum() == t
+    pa, sa = orc.mx_quant_rows(rand_bf16(rng, (t, k), 1.0), orc.E4M3)
+    pbs, sbs = zip(*[orc.mx_quant_b(rand_bf16(rng, (k, n), 1.0), orc.E4M3, orc.RNE, 0) for _ in range(e)])
+    pb, sb = np.stack(pbs), np.stack(sbs)
+    gold = orc.mx_gmm(pa, sa, pb, sb, n, k, orc.E4M3, 0, group_sizes=gs)
+    ident = np.arange(t, dtype=np.int32)
+    outs = {}
+    cc.set_option("require_tiled_gemm", 1)
+    try:
+        for order in (0, 1, -1):
+            cc.set_option("gemm_tile_order", order)
+            # the output starts as NaN: a tile that no workgroup computes would keep it
+            out = torch.full((t, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+            cc.mx_grouped_matmul_mapped(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), dev(ident), out, "e4m3", 0)
+            outs[order] = out_f32(out)
+    finally:
+        cc.set_option("gemm_tile_order", -1)
+        cc.set_option("require_tiled_gemm", 0)
+    assert not np.isnan(outs[1]).any()
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[-1])
+    assert_close(outs[1], gold, "per-XCD tile order")
