@@ -1,0 +1,51 @@
+"""torch.ops.catccos.* on the GPU: the dispatcher reaches the HIP library (results equal the oracle's,
+bit-exact for the quantiser, within the GEMM gate otherwise) and refuses to run before init, as the
+reference's binding does (examples/torch_binding/src/torch_bindings.cpp:131-133)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+import catccos_amd.torch_library  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+OPS = torch.ops.catccos
+
+
+def dev(x):
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def close(got, want):
+    m = orc.compare(got.float().cpu().numpy(), want)
+    assert m["max_rel_floor1"] <= 1e-2 and m["max_rel_floor_rms"] <= 1e-2, m
+
+
+def test_ops_need_init_then_match_the_oracle():
+    rng = np.random.default_rng(3)
+    e, t, k, n = 3, 333, 512, 256
+    gs = np.array([200, 0, 133], np.int32)
+    x = orc.f32_to_bf16(rng.standard_normal((t, k)).astype(np.float32))
+    xd = torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16)
+    assert OPS.finalize() == 0
+    with pytest.raises(RuntimeError, match="not initialized"):
+        OPS.mx_quant(xd, "e4m3", 0)
+    assert OPS.init(0, 1, 1 << 20, "tcp://127.0.0.1:8666") == 0
+    try:
+        a, sa = OPS.mx_quant(xd, "e4m3", 0)
+        pa, psa = orc.mx_quant_rows(x, orc.E4M3)
+        assert np.array_equal(a.cpu().numpy(), pa) and np.array_equal(sa.cpu().numpy(), psa)
+        pbs, sbs = zip(*[orc.mx_quant_b(orc.f32_to_bf16(rng.standard_normal((k, n)).astype(np.float32)), orc.E4M3, orc.RNE, 0)
+                         for _ in range(e)])
+        pb, sb = np.stack(pbs), np.stack(sbs)
+        close(OPS.mx_grouped_matmul(a, sa, dev(pb), dev(sb), dev(gs), "e4m3", 0),
+              orc.mx_gmm(pa, psa, pb, sb, n, k, orc.E4M3, 0, group_sizes=gs))
+        close(OPS.mx_matmul(a, sa, dev(pb[0]), dev(sb[0]), "e4m3", 0), orc.mx_gmm(pa, psa, pb[:1], sb[:1], n, k, orc.E4M3, 0))
+        xi = rng.integers(-127, 128, (t, k)).astype(np.int8)
+        wi = rng.integers(-127, 128, (e, k, n)).astype(np.int8)
+        pt = rng.uniform(0.001, 0.02, t).astype(np.float32)
+        pc = rng.uniform(0.001, 0.02, (e, n)).astype(np.float32)
+        close(OPS.gmm_dequant_swiglu(dev(xi), dev(wi), dev(gs), dev(pt), dev(pc), 0), orc.gmm_i8_dequant_swiglu(xi, wi, gs, pt, pc))
+        close(OPS.w8a8_matmul_dequant(dev(xi), dev(wi[0]), dev(pt), dev(pc[0]), 0), orc.gemm_i8_dequant(xi, wi[0], pt, pc[0]))
+    finally:
+        assert OPS.finalize() == 0
