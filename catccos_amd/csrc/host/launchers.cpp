@@ -1,9 +1,16 @@
 // Launch<Op><DType> functions with the reference's KernelFuncPtr signature
 // (tests/dynamic_tiling/include/launch_map.h:15-16; bodies there: impl/kernel_int8.cpp:113-130,
 // impl/kernel_mxfp_ascend950.cpp:19, impl/kernel_fp16_ascend950.cpp:592-612).  Each one maps the
-// KernelParams pointer roles of its operator onto one C-ABI call and, like DeviceDGemm::Run
-// (include/catccos/dgemm/device/device_dgemm.hpp:89-120), synchronises the stream before returning.
+// KernelParams pointer roles of its operator onto the kernel's Arguments and runs it through the
+// device-operator facade like the reference's bodies do (Arguments -> Initialize -> Run, which
+// synchronises the stream, include/catccos/dgemm/device/device_dgemm.hpp:89-120); the launchers of
+// the dispatch / combine additions call the C ABI directly and synchronise the same way.
+#include "device_dgemm.h"
 #include "launch_map.h"
+
+using namespace Catccos;
+using Catccos::DGemm::Device::DeviceDGemm;
+namespace K = Catccos::DGemm::Kernel;
 
 namespace {
 void Finish(int rc, void *stream, const char *what)
@@ -11,30 +18,68 @@ void Finish(int rc, void *stream, const char *what)
     if (rc != CCH_OK) fprintf(stderr, "%s: cchError:%d %s\n", what, rc, cch_last_error());
     CCH_CHECK(cch_stream_sync(stream));
 }
+inline GM_ADDR Gm(void *p) { return static_cast<GM_ADDR>(p); }
+template <class Kernel> void RunOp(const typename Kernel::Arguments &args, void *stream, uint32_t blockNum, uint64_t fftsAddr,
+                                   uint8_t *workSpace)
+{
+    DeviceDGemm<Kernel> op;
+    op.Initialize(args, workSpace);
+    op.Run(stream, blockNum, fftsAddr);
+}
 struct AutoRegister {
     AutoRegister(CocCommType type, CocDataType dtype, KernelFuncPtr fn) { KernelDispatcher::RegisterKernelFunc(type, dtype, fn); }
 };
 }  // namespace
 
-void LaunchAscend950BF16QuantAllGatherFP8E4M3FN(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
-                                                CocTilingParams &t, uint32_t, uint32_t)
+void LaunchAscend950BF16QuantAllGatherFP8E4M3FN(void *stream, uint32_t blockNum, uint64_t fftsAddr, KernelParams &p,
+                                                uint8_t *workSpace, uint8_t *symmetricPtr, CocTilingParams &t, uint32_t, uint32_t)
 {
-    Finish(cch_mx_quant_rows(p.ptrA, p.ptrC, p.ptrB, t.m, t.n, CCH_FMT_E4M3, CCH_ROUND_RNE, stream), stream, "MxQuantAllGather");
+    K::MxQuantAllGather::Arguments args{};
+    args.problemShape = MatrixCoord{t.m, t.n};
+    args.rankIdx = 0;
+    args.rankSize = t.rankSize;
+    args.ptrInput = Gm(p.ptrA);
+    args.ptrOutput = Gm(p.ptrC);
+    args.ptrMxScale = Gm(p.ptrB);
+    args.ptrSymmetric = symmetricPtr;
+    RunOp<K::MxQuantAllGather>(args, stream, blockNum, fftsAddr, workSpace);
 }
 
-void LaunchAllGatherMatmulDequantINT8(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
-                                      CocTilingParams &t, uint32_t, uint32_t transB)
+void LaunchAllGatherMatmulDequantINT8(void *stream, uint32_t blockNum, uint64_t fftsAddr, KernelParams &p, uint8_t *workSpace,
+                                      uint8_t *symmetricPtr, CocTilingParams &t, uint32_t, uint32_t transB)
 {
-    Finish(cch_gemm_i8_dequant(p.ptrA, p.ptrB, reinterpret_cast<const float *>(p.customPtrs[1]),
-                               reinterpret_cast<const float *>(p.customPtrs[0]), p.ptrC, t.m, t.n, t.k, (int)transB, stream),
-           stream, "AllGatherMatmulDequant");
+    K::AllGatherMatmulDequant::Arguments args{};
+    args.problemShape = GemmCoord{t.m, t.n, t.k};
+    args.rankSize = t.rankSize;
+    args.commInterval = t.commInterval;
+    args.ptrA = Gm(p.ptrA);
+    args.ptrB = Gm(p.ptrB);
+    args.ptrD = Gm(p.ptrC);
+    args.ptrScale = Gm(p.customPtrs[0]);
+    args.ptrPerToken = Gm(p.customPtrs[1]);
+    args.ptrWB = workSpace;
+    args.ptrSymmetric = symmetricPtr;
+    args.transB = transB;
+    RunOp<K::AllGatherMatmulDequant>(args, stream, blockNum, fftsAddr, workSpace);
 }
 
-void LaunchAscend950MxFp8MatmulReduceScatterFP8E4M3FN(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
-                                                      CocTilingParams &t, uint32_t, uint32_t transB)
+void LaunchAscend950MxFp8MatmulReduceScatterFP8E4M3FN(void *stream, uint32_t blockNum, uint64_t fftsAddr, KernelParams &p,
+                                                      uint8_t *workSpace, uint8_t *symmetricPtr, CocTilingParams &t, uint32_t,
+                                                      uint32_t transB)
 {
-    Finish(cch_mx_gemm(p.ptrA, p.customPtrs[0], p.ptrB, p.customPtrs[1], p.ptrC, t.m, t.n, t.k, CCH_FMT_E4M3, (int)transB, stream),
-           stream, "Ascend950MxFp8MatmulReduceScatter");
+    K::MatmulReduceScatterMx::Arguments args{};
+    args.problemShape = GemmCoord{t.m, t.n, t.k};
+    args.rankSize = t.rankSize;
+    args.commInterval = t.commInterval;
+    args.ptrA = Gm(p.ptrA);
+    args.ptrB = Gm(p.ptrB);
+    args.ptrMxScaleA = Gm(p.customPtrs[0]);
+    args.ptrMxScaleB = Gm(p.customPtrs[1]);
+    args.ptrD = Gm(p.ptrC);
+    args.ptrSymmetric = symmetricPtr;
+    args.format = CCH_FMT_E4M3;
+    args.transB = transB;
+    RunOp<K::MatmulReduceScatterMx>(args, stream, blockNum, fftsAddr, workSpace);
 }
 
 void LaunchDispatchGmmDequantSwigluINT8(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
@@ -58,48 +103,73 @@ void LaunchDispatchGmmDequantSwigluINT8(void *stream, uint32_t, uint64_t, Kernel
         Finish(rc, stream, "DispatchGmmDequantSwiglu");
         return;
     }
-    Finish(cch_gmm_i8_dequant_swiglu(p.ptrA, p.ptrB, reinterpret_cast<const int32_t *>(p.customPtrs[1]),
-                                     reinterpret_cast<const float *>(p.customPtrs[2]),
-                                     reinterpret_cast<const float *>(p.customPtrs[0]), p.ptrC, t.expertNum, t.m, t.n, t.k,
-                                     (int)transB, stream),
-           stream, "DispatchGmmDequantSwiglu");
+    K::AlltoallvGmmDequantSwiglu::Arguments args{};
+    args.problemShape = GemmCoord{t.m, t.n, t.k};
+    args.EP = 1;
+    args.expertPerRank = (int32_t)t.expertNum;
+    args.rankSize = t.rankSize;
+    args.ptrA = Gm(p.ptrA);
+    args.ptrB = Gm(p.ptrB);
+    args.ptrC = Gm(p.ptrC);
+    args.ptrScale = Gm(p.customPtrs[0]);
+    args.ptrTokenPerExpert = Gm(p.customPtrs[1]);
+    args.ptrPerTokenScale = Gm(p.customPtrs[2]);
+    args.transB = transB;
+    RunOp<K::AlltoallvGmmDequantSwiglu>(args, stream, 0, 0, nullptr);
 }
 
-void LaunchAscend950Fp4MxAllToAllVGroupedMatmulBF16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
-                                                    CocTilingParams &t, uint32_t, uint32_t transB)
+// Up projection (Arguments as in tests/dynamic_tiling/impl/kernel_fp16_ascend950.cpp:592-612).  The
+// reference registers these operators for fp16 output (launch_map.h:100-101); this build has that
+// launcher and a bf16 twin.
+static void MxAllToAllVGroupedMatmul(void *stream, uint32_t blockNum, uint64_t fftsAddr, KernelParams &p, uint8_t *workSpace,
+                                     uint8_t *symmetricPtr, CocTilingParams &t, uint32_t transB, int fmt, bool fp16)
 {
-    Finish(cch_mx_gmm(p.ptrA, p.customPtrs[0], p.ptrB, p.customPtrs[1], reinterpret_cast<const int32_t *>(p.customPtrs[3]),
-                      p.ptrC, t.expertNum, t.m, t.n, t.k, CCH_FMT_E2M1, (int)transB, stream),
-           stream, "Ascend950Fp4MxAllToAllVGroupedMatmul");
+    K::MxAllToAllVGroupMatmul::Arguments args{};
+    args.gemmShape = GemmCoord{t.m, t.n, t.k};
+    args.rankSize = t.rankSize;
+    args.commInterval = t.commInterval;
+    args.epSize = 1;                 // the experts of this call are this rank's
+    args.expertNum = t.expertNum;
+    args.ptrA = Gm(p.ptrA);
+    args.ptrB = Gm(p.ptrB);
+    args.ptrC = Gm(p.ptrC);
+    args.ptrMxScaleA = Gm(p.customPtrs[0]);
+    args.ptrMxScaleB = Gm(p.customPtrs[1]);
+    args.ptrLocalTokensPerExpert = Gm(p.customPtrs[2]);
+    args.ptrGlobalTokensPerLocalExpert = Gm(p.customPtrs[3]);
+    args.ptrSymmetric = symmetricPtr;
+    args.format = fmt;
+    args.transB = transB;
+    args.outFp16 = fp16;
+    RunOp<K::MxAllToAllVGroupMatmul>(args, stream, blockNum, fftsAddr, workSpace);
 }
 
-void LaunchAscend950Fp8MxAllToAllVGroupedMatmulBF16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
-                                                    CocTilingParams &t, uint32_t, uint32_t transB)
+void LaunchAscend950Fp4MxAllToAllVGroupedMatmulBF16(void *stream, uint32_t blockNum, uint64_t fftsAddr, KernelParams &p,
+                                                    uint8_t *workSpace, uint8_t *symmetricPtr, CocTilingParams &t, uint32_t,
+                                                    uint32_t transB)
 {
-    Finish(cch_mx_gmm(p.ptrA, p.customPtrs[0], p.ptrB, p.customPtrs[1], reinterpret_cast<const int32_t *>(p.customPtrs[3]),
-                      p.ptrC, t.expertNum, t.m, t.n, t.k, CCH_FMT_E4M3, (int)transB, stream),
-           stream, "Ascend950Fp8MxAllToAllVGroupedMatmul");
+    MxAllToAllVGroupedMatmul(stream, blockNum, fftsAddr, p, workSpace, symmetricPtr, t, transB, CCH_FMT_E2M1, false);
 }
 
-// The reference registers the two operators above for fp16 output (launch_map.h:100-101): the same
-// matmul through the entry point that takes an output type, without a row map.
-static void MxAllToAllVGroupedMatmulFP16(void *stream, KernelParams &p, CocTilingParams &t, uint32_t transB, int fmt, const char *what)
+void LaunchAscend950Fp8MxAllToAllVGroupedMatmulBF16(void *stream, uint32_t blockNum, uint64_t fftsAddr, KernelParams &p,
+                                                    uint8_t *workSpace, uint8_t *symmetricPtr, CocTilingParams &t, uint32_t,
+                                                    uint32_t transB)
 {
-    Finish(cch_mx_gmm_mapped(p.ptrA, p.customPtrs[0], p.ptrB, p.customPtrs[1], reinterpret_cast<const int32_t *>(p.customPtrs[3]),
-                             nullptr, p.ptrC, t.m, CCH_OUT_FP16, t.expertNum, t.m, t.n, t.k, fmt, (int)transB, stream),
-           stream, what);
+    MxAllToAllVGroupedMatmul(stream, blockNum, fftsAddr, p, workSpace, symmetricPtr, t, transB, CCH_FMT_E4M3, false);
 }
 
-void LaunchAscend950Fp4MxAllToAllVGroupedMatmulFP16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
-                                                    CocTilingParams &t, uint32_t, uint32_t transB)
+void LaunchAscend950Fp4MxAllToAllVGroupedMatmulFP16(void *stream, uint32_t blockNum, uint64_t fftsAddr, KernelParams &p,
+                                                    uint8_t *workSpace, uint8_t *symmetricPtr, CocTilingParams &t, uint32_t,
+                                                    uint32_t transB)
 {
-    MxAllToAllVGroupedMatmulFP16(stream, p, t, transB, CCH_FMT_E2M1, "Ascend950Fp4MxAllToAllVGroupedMatmul");
+    MxAllToAllVGroupedMatmul(stream, blockNum, fftsAddr, p, workSpace, symmetricPtr, t, transB, CCH_FMT_E2M1, true);
 }
 
-void LaunchAscend950Fp8MxAllToAllVGroupedMatmulFP16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *,
-                                                    CocTilingParams &t, uint32_t, uint32_t transB)
+void LaunchAscend950Fp8MxAllToAllVGroupedMatmulFP16(void *stream, uint32_t blockNum, uint64_t fftsAddr, KernelParams &p,
+                                                    uint8_t *workSpace, uint8_t *symmetricPtr, CocTilingParams &t, uint32_t,
+                                                    uint32_t transB)
 {
-    MxAllToAllVGroupedMatmulFP16(stream, p, t, transB, CCH_FMT_E4M3, "Ascend950Fp8MxAllToAllVGroupedMatmul");
+    MxAllToAllVGroupedMatmul(stream, blockNum, fftsAddr, p, workSpace, symmetricPtr, t, transB, CCH_FMT_E4M3, true);
 }
 
 // Down projection.  The reference registers these two operators for fp16 output only

@@ -65,3 +65,47 @@ def test_no_device_is_an_error_not_a_fallback():
         pytest.skip("GPU present")
     r = run("agmmdq", "128", "128", "128", "-")
     assert r.returncode != 0 and "cch_init failed" in r.stdout
+
+
+FACADE_PROGRAM = r"""
+#include <cstdio>
+#include "device_dgemm.h"
+using namespace Catccos;
+using Op = DGemm::Device::DeviceDGemm<DGemm::Kernel::AllGatherMatmulDequant>;
+using Mx = DGemm::Device::DeviceDGemm<DGemm::Kernel::MxAllToAllVGroupMatmul>;
+int main()
+{
+    Op op;
+    if (op.Run(nullptr, 20, 0) != Status::kErrorInvalidProblem) return 1;          // not initialised
+    Op::Arguments args{};
+    args.problemShape = GemmCoord{128, 256, 512};
+    args.rankSize = 1;
+    args.transB = 7;                                                               // not a layout
+    if (Op::GetWorkspaceSize(args) != 0) return 2;
+    if (op.Initialize(args) != Status::kSuccess) return 3;
+    if (op.params().problemShape.m() != 128 || op.params().problemShape.n() != 256 || op.params().problemShape.k() != 512) return 4;
+    if (op(nullptr, 20, 0) != Status::kErrorInvalidProblem) return 5;              // refused by the C ABI's argument checks
+    Mx::Arguments g{};
+    g.gemmShape = GemmCoord{64, 128, 256};
+    g.expertNum = 32;
+    g.epSize = 4;
+    Mx mx;
+    mx.Initialize(g);
+    if (mx.params().localExperts != 8) return 6;
+    puts("facade ok");
+    return 0;
+}
+"""
+
+
+def test_device_operator_facade(tmp_path):
+    """DeviceDGemm<Kernel>: GetWorkspaceSize / Initialize / Run as the reference's launcher bodies call
+    them (include/catccos/dgemm/device/device_dgemm.hpp:50-126), without a GPU: state and error paths."""
+    src = tmp_path / "facade.cpp"
+    src.write_text(FACADE_PROGRAM)
+    exe = tmp_path / "facade"
+    pkg = os.path.join(ROOT, "catccos_amd")
+    subprocess.run(["g++", "-std=c++17", "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(pkg, "csrc", "host"),
+                    str(src), "-o", str(exe), "-L" + pkg, "-Wl,-rpath," + pkg, "-lcatccos_hip"], check=True, timeout=120)
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0 and "facade ok" in r.stdout, (r.returncode, r.stdout, r.stderr)
