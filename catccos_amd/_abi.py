@@ -40,6 +40,10 @@ PROTOTYPES = {
     "cch_dyn_quant_i8_rows": [_P, _P, _P, _P, _I64, _I64, _I64, _I, _I, _P],
     "cch_dyn_quant_i8_rows_smooth": [_P, _P, _P, _P, _I64, _P, _P, _I64, _I64, _I64, _I, _I, _P],
     "cch_gemm_i8_dequant": [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I, _P],
+    "cch_gemm_i8_dequant_out": [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I, _I, _P],
+    "cch_gmm_i8_dequant_out": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _I, _P],
+    "cch_gmm_i8_dequant_swiglu_out": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _I, _P],
+    "cch_mx_gemm_out": [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I, _I, _I, _P],
     "cch_gmm_i8_dequant": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _P],
     "cch_gmm_i8_dequant_swiglu": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _P],
     "cch_mx_gemm": [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I, _I, _P],

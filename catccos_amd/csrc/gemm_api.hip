@@ -60,8 +60,15 @@ int cch_set_option(const char *name, int value)
 int cch_gemm_i8_dequant(const void *a, const void *b, const float *per_tok, const float *per_ch, void *out, int64_t m,
                         int64_t n, int64_t k, int trans_b, void *stream)
 {
+    return cch_gemm_i8_dequant_out(a, b, per_tok, per_ch, out, m, n, k, trans_b, CCH_OUT_BF16, stream);
+}
+
+int cch_gemm_i8_dequant_out(const void *a, const void *b, const float *per_tok, const float *per_ch, void *out, int64_t m,
+                            int64_t n, int64_t k, int trans_b, int out_dtype, void *stream)
+{
     int rc = check_shape("cch_gemm_i8_dequant", m, n, k);
     if (rc) return rc;
+    CCH_REQUIRE(out_dtype == CCH_OUT_BF16 || out_dtype == CCH_OUT_FP16, "cch_gemm_i8_dequant: out_dtype %d", out_dtype);
     CCH_REQUIRE(trans_b == 0 || trans_b == 1, "cch_gemm_i8_dequant: trans_b %d", trans_b);
     if (m == 0 || n == 0) return CCH_OK;
     CCH_REQUIRE(out && per_tok && per_ch && (k == 0 || (a && b)), "cch_gemm_i8_dequant: null pointer");
@@ -74,6 +81,7 @@ int cch_gemm_i8_dequant(const void *a, const void *b, const float *per_tok, cons
     p.num_groups = 1;
     p.T = (int)m; p.N = (int)n; p.K = (int)k; p.n_out = (int)n;
     p.trans_b = trans_b;
+    p.out_fp16 = out_dtype == CCH_OUT_FP16;
     return run(p, KIND_I8, EPI_DEQUANT, static_cast<hipStream_t>(stream));
 }
 
@@ -81,8 +89,16 @@ int cch_gmm_i8_dequant_swiglu(const void *x, const void *w, const int32_t *group
                               const float *per_ch, void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k,
                               int trans_b, void *stream)
 {
+    return cch_gmm_i8_dequant_swiglu_out(x, w, group_sizes, per_tok, per_ch, out, num_experts, t, n, k, trans_b, CCH_OUT_BF16, stream);
+}
+
+int cch_gmm_i8_dequant_swiglu_out(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok,
+                                  const float *per_ch, void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k,
+                                  int trans_b, int out_dtype, void *stream)
+{
     int rc = check_shape("cch_gmm_i8_dequant_swiglu", t, n, k);
     if (rc) return rc;
+    CCH_REQUIRE(out_dtype == CCH_OUT_BF16 || out_dtype == CCH_OUT_FP16, "cch_gmm_i8_dequant_swiglu: out_dtype %d", out_dtype);
     CCH_REQUIRE(trans_b == 0 || trans_b == 1, "cch_gmm_i8_dequant_swiglu: trans_b %d", trans_b);
     CCH_REQUIRE(n % 2 == 0, "cch_gmm_i8_dequant_swiglu: n=%lld must be even (gate | up halves)", (long long)n);
     CCH_REQUIRE(num_experts >= 1 && num_experts <= 65535, "cch_gmm_i8_dequant_swiglu: num_experts=%lld", (long long)num_experts);
@@ -99,14 +115,23 @@ int cch_gmm_i8_dequant_swiglu(const void *x, const void *w, const int32_t *group
     p.T = (int)t; p.N = (int)n; p.K = (int)k; p.n_out = (int)(n / 2);
     p.trans_b = trans_b;
     p.b_stride = n * k;
+    p.out_fp16 = out_dtype == CCH_OUT_FP16;
     return run(p, KIND_I8, EPI_DEQUANT_SWIGLU, static_cast<hipStream_t>(stream));
 }
 
 int cch_gmm_i8_dequant(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok, const float *per_ch,
                        void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k, int trans_b, void *stream)
 {
+    return cch_gmm_i8_dequant_out(x, w, group_sizes, per_tok, per_ch, out, num_experts, t, n, k, trans_b, CCH_OUT_BF16, stream);
+}
+
+int cch_gmm_i8_dequant_out(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok, const float *per_ch,
+                           void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k, int trans_b, int out_dtype,
+                           void *stream)
+{
     int rc = check_shape("cch_gmm_i8_dequant", t, n, k);
     if (rc) return rc;
+    CCH_REQUIRE(out_dtype == CCH_OUT_BF16 || out_dtype == CCH_OUT_FP16, "cch_gmm_i8_dequant: out_dtype %d", out_dtype);
     CCH_REQUIRE(trans_b == 0 || trans_b == 1, "cch_gmm_i8_dequant: trans_b %d", trans_b);
     CCH_REQUIRE(num_experts >= 1 && num_experts <= 65535, "cch_gmm_i8_dequant: num_experts=%lld", (long long)num_experts);
     if (t == 0 || n == 0) return CCH_OK;
@@ -122,6 +147,7 @@ int cch_gmm_i8_dequant(const void *x, const void *w, const int32_t *group_sizes,
     p.T = (int)t; p.N = (int)n; p.K = (int)k; p.n_out = (int)n;
     p.trans_b = trans_b;
     p.b_stride = n * k;
+    p.out_fp16 = out_dtype == CCH_OUT_FP16;
     return run(p, KIND_I8, EPI_DEQUANT, static_cast<hipStream_t>(stream));
 }
 
@@ -157,10 +183,18 @@ static int mx_problem(const char *who, GemmProblem &p, const void *a, const void
 int cch_mx_gemm(const void *a, const void *sa, const void *b, const void *sb, void *out, int64_t m, int64_t n, int64_t k,
                 int fmt, int trans_b, void *stream)
 {
+    return cch_mx_gemm_out(a, sa, b, sb, out, m, n, k, fmt, trans_b, CCH_OUT_BF16, stream);
+}
+
+int cch_mx_gemm_out(const void *a, const void *sa, const void *b, const void *sb, void *out, int64_t m, int64_t n, int64_t k,
+                    int fmt, int trans_b, int out_dtype, void *stream)
+{
     GemmProblem p{};
     int kind = 0;
+    CCH_REQUIRE(out_dtype == CCH_OUT_BF16 || out_dtype == CCH_OUT_FP16, "cch_mx_gemm: out_dtype %d", out_dtype);
     int rc = mx_problem("cch_mx_gemm", p, a, sa, b, sb, nullptr, out, 1, m, n, k, fmt, trans_b, &kind);
     if (rc) return rc;
+    p.out_fp16 = out_dtype == CCH_OUT_FP16;
     return run(p, kind, EPI_PLAIN, static_cast<hipStream_t>(stream));
 }
 

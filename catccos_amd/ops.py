@@ -213,13 +213,20 @@ def set_option(name, value):
     check(_abi.lib().cch_set_option(name.encode(), int(value)))
 
 
+def _out_code(out_dtype):
+    if out_dtype not in (torch.bfloat16, torch.float16):
+        raise ValueError("out_dtype must be torch.bfloat16 or torch.float16")
+    return 1 if out_dtype == torch.float16 else 0
+
+
 def _check_2d(name, t, dtype):
     if t.dim() != 2 or t.dtype != dtype:
         raise ValueError("%s must be a 2-D %s tensor" % (name, dtype))
 
 
-def w8a8_matmul_dequant(a, b, per_tok, per_ch, trans_b=0):
-    """int8 [M,K] x int8 [K,N] (or [N,K] with trans_b=1) -> bf16 [M,N], scaled per token and per channel."""
+def w8a8_matmul_dequant(a, b, per_tok, per_ch, trans_b=0, out_dtype=torch.bfloat16):
+    """int8 [M,K] x int8 [K,N] (or [N,K] with trans_b=1) -> bf16 (or half) [M,N], scaled per token and per channel."""
+    code = _out_code(out_dtype)
     _require_gpu(a, b, per_tok, per_ch)
     _check_2d("a", a, torch.int8)
     _check_2d("b", b, torch.int8)
@@ -232,24 +239,25 @@ def w8a8_matmul_dequant(a, b, per_tok, per_ch, trans_b=0):
     per_ch = per_ch.contiguous().float()
     if per_tok.numel() != m or per_ch.numel() != n:
         raise ValueError("per_tok must have M entries and per_ch N entries")
-    out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
-    check(_abi.lib().cch_gemm_i8_dequant(_ptr(a), _ptr(b), _ptr(per_tok), _ptr(per_ch), _ptr(out), m, n, k,
-                                         int(trans_b), _stream()))
+    out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    check(_abi.lib().cch_gemm_i8_dequant_out(_ptr(a), _ptr(b), _ptr(per_tok), _ptr(per_ch), _ptr(out), m, n, k,
+                                             int(trans_b), code, _stream()))
     return out
 
 
-def gmm_dequant(x, w, group_sizes, per_tok, per_ch, trans_b=0):
-    """Grouped int8 matmul + per-token x per-channel dequant (no activation); returns bf16 [T, N]."""
-    return _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, False)
+def gmm_dequant(x, w, group_sizes, per_tok, per_ch, trans_b=0, out_dtype=torch.bfloat16):
+    """Grouped int8 matmul + per-token x per-channel dequant (no activation); returns bf16 (or half) [T, N]."""
+    return _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, False, out_dtype)
 
 
-def gmm_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, trans_b=0):
+def gmm_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, trans_b=0, out_dtype=torch.bfloat16):
     """Grouped int8 matmul + dequant + SwiGLU: x int8 [T,K] grouped by expert, w int8 [E,K,N]
-    (or [E,N,K]), group_sizes int32 [E] on the device; returns bf16 [T, N/2]."""
-    return _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, True)
+    (or [E,N,K]), group_sizes int32 [E] on the device; returns bf16 (or half) [T, N/2]."""
+    return _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, True, out_dtype)
 
 
-def _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, swiglu):
+def _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, swiglu, out_dtype=torch.bfloat16):
+    code = _out_code(out_dtype)
     _require_gpu(x, w, group_sizes, per_tok, per_ch)
     _check_2d("x", x, torch.int8)
     if w.dim() != 3 or w.dtype != torch.int8:
@@ -266,9 +274,10 @@ def _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, swiglu):
     per_ch = per_ch.contiguous().float()
     if per_tok.numel() != t or tuple(per_ch.shape) != (e, n):
         raise ValueError("per_tok must be [T] and per_ch [E,N]")
-    out = torch.empty((t, n // 2 if swiglu else n), dtype=torch.bfloat16, device=x.device)
-    fn = _abi.lib().cch_gmm_i8_dequant_swiglu if swiglu else _abi.lib().cch_gmm_i8_dequant
-    check(fn(_ptr(x), _ptr(w), _ptr(group_sizes), _ptr(per_tok), _ptr(per_ch), _ptr(out), e, t, n, k, int(trans_b), _stream()))
+    out = torch.empty((t, n // 2 if swiglu else n), dtype=out_dtype, device=x.device)
+    fn = _abi.lib().cch_gmm_i8_dequant_swiglu_out if swiglu else _abi.lib().cch_gmm_i8_dequant_out
+    check(fn(_ptr(x), _ptr(w), _ptr(group_sizes), _ptr(per_tok), _ptr(per_ch), _ptr(out), e, t, n, k, int(trans_b), code,
+             _stream()))
     return out
 
 
@@ -298,13 +307,14 @@ def _mx_shapes(a, sa, b, sb, fmt, trans_b, grouped):
     return fmt, t, n, k, e
 
 
-def mx_matmul(a, sa, b, sb, fmt="e4m3", trans_b=0):
-    """MX dense GEMM: payload/scales as produced by mx_quant (a) and mx_quant_b (b); bf16 [M,N]."""
+def mx_matmul(a, sa, b, sb, fmt="e4m3", trans_b=0, out_dtype=torch.bfloat16):
+    """MX dense GEMM: payload/scales as produced by mx_quant (a) and mx_quant_b (b); bf16 (or half) [M,N]."""
+    code = _out_code(out_dtype)
     _require_gpu(a, sa, b, sb)
     a, sa, b, sb = a.contiguous(), sa.contiguous(), b.contiguous(), sb.contiguous()
     fmt, m, n, k, _ = _mx_shapes(a, sa, b, sb, fmt, trans_b, False)
-    out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
-    check(_abi.lib().cch_mx_gemm(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(out), m, n, k, fmt, int(trans_b), _stream()))
+    out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    check(_abi.lib().cch_mx_gemm_out(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(out), m, n, k, fmt, int(trans_b), code, _stream()))
     return out
 
 

@@ -41,6 +41,10 @@ extern "C" {
 #define CCH_ROUND_RNE 0
 #define CCH_ROUND_LUT 1
 
+/* Output element types of the GEMM entry points that take an out_dtype. */
+#define CCH_OUT_BF16 0
+#define CCH_OUT_FP16 1
+
 /* ---- runtime shims: what the host operator layer needs in place of acl.h ----
  * Replace aclInit/aclrtSetDevice, aclrtMalloc/aclrtFree, aclrtMallocHost/
  * aclrtFreeHost, aclrtMemcpy, aclrtMemset, aclrtCreateStream/
@@ -96,6 +100,11 @@ int cch_mx_quant_b(const void *b, void *payload, void *scales, int64_t k, int64_
  *   per_ch fp32 [n]; out bf16 [m,n]. */
 int cch_gemm_i8_dequant(const void *a, const void *b, const float *per_tok, const float *per_ch, void *out, int64_t m,
                         int64_t n, int64_t k, int trans_b, void *stream);
+/* The same with a choice of output type: out_dtype CCH_OUT_BF16 or CCH_OUT_FP16 (IEEE half, the
+ * type the reference's int8 launchers write: `using ElementC = half`,
+ * tests/dynamic_tiling/impl/kernel_int8.cpp:16); both are the fp32 result rounded to nearest even. */
+int cch_gemm_i8_dequant_out(const void *a, const void *b, const float *per_tok, const float *per_ch, void *out, int64_t m,
+                            int64_t n, int64_t k, int trans_b, int out_dtype, void *stream);
 
 /* ---- MoE grouped W8A8 matmul + dequant, without the activation ----------------
  * The grouped GEMM and per-token dequantisation of AlltoallvGmmDequantKernel
@@ -106,6 +115,10 @@ int cch_gemm_i8_dequant(const void *a, const void *b, const float *per_tok, cons
  * operands and grouping as below.  Rows past sum(group_sizes) are written as zeros. */
 int cch_gmm_i8_dequant(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok, const float *per_ch,
                        void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k, int trans_b, void *stream);
+/* The same with a choice of output type (CCH_OUT_BF16 / CCH_OUT_FP16). */
+int cch_gmm_i8_dequant_out(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok, const float *per_ch,
+                           void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k, int trans_b, int out_dtype,
+                           void *stream);
 
 /* ---- MoE grouped W8A8 matmul + dequant + SwiGLU (config 4) -------------------
  * Replaces the grouped GEMM of AlltoallvGmmDequantKernel::operator()<AIC>
@@ -118,6 +131,10 @@ int cch_gmm_i8_dequant(const void *x, const void *w, const int32_t *group_sizes,
 int cch_gmm_i8_dequant_swiglu(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok,
                               const float *per_ch, void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k,
                               int trans_b, void *stream);
+/* The same with a choice of output type (CCH_OUT_BF16 / CCH_OUT_FP16). */
+int cch_gmm_i8_dequant_swiglu_out(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok,
+                                  const float *per_ch, void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k,
+                                  int trans_b, int out_dtype, void *stream);
 
 /* ---- MX (FP8 / FP4 payload, E8M0 scales) dense GEMM (config 3) ---------------
  * Replaces the compute half of MatmulReduceScatterMxTla::operator()<AIC>
@@ -129,6 +146,11 @@ int cch_gmm_i8_dequant_swiglu(const void *x, const void *w, const int32_t *group
  *   trans_b=1: b [n,k] (FP4 [n,k/2]), sb [n, 2*ceil(k/64)] */
 int cch_mx_gemm(const void *a, const void *sa, const void *b, const void *sb, void *out, int64_t m, int64_t n, int64_t k,
                 int fmt, int trans_b, void *stream);
+/* The same with a choice of output type (CCH_OUT_BF16 / CCH_OUT_FP16; the reference's Ascend950 MX
+ * matmul launchers are registered for fp16, e.g. LaunchAscend950Fp4MxMatmulReduceScatterFP16,
+ * tests/dynamic_tiling/impl/kernel_fp16_ascend950.cpp:211). */
+int cch_mx_gemm_out(const void *a, const void *sa, const void *b, const void *sb, void *out, int64_t m, int64_t n, int64_t k,
+                    int fmt, int trans_b, int out_dtype, void *stream);
 
 /* ---- MX grouped matmul over variable-size expert groups (config 5) -----------
  * Replaces the compute half of MxAllToAllVGroupedMatmulTla::operator()<AIC>
@@ -157,8 +179,6 @@ int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, con
  *   out_dtype    CCH_OUT_BF16, or CCH_OUT_FP16 (IEEE half, the type the reference registers these
  *                operators for); fp32 accumulators are rounded to nearest even either way
  * Destination rows must be distinct. */
-#define CCH_OUT_BF16 0
-#define CCH_OUT_FP16 1
 int cch_mx_gmm_mapped(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes,
                       const int32_t *out_row_map, void *out, int64_t out_rows, int out_dtype, int64_t num_experts, int64_t t,
                       int64_t n, int64_t k, int fmt, int trans_b, void *stream);

@@ -51,6 +51,10 @@ def test_gemm_arguments():
     rejected(L.cch_mx_gmm(P, P, P, P, None, P, 2, 8, 8, 64, 0, 0, None))   # group sizes missing
     rejected(L.cch_mx_gmm_mapped(P, P, P, P, P, None, P, 9, 0, 2, 8, 8, 64, 0, 0, None), "row map")
     rejected(L.cch_mx_gmm_mapped(P, P, P, P, P, P, P, 8, 3, 2, 8, 8, 64, 0, 0, None), "out_dtype")
+    rejected(L.cch_gemm_i8_dequant_out(P, P, P, P, P, 8, 8, 8, 0, 2, None), "out_dtype")
+    rejected(L.cch_gmm_i8_dequant_out(P, P, P, P, P, P, 2, 8, 8, 8, 0, -1, None), "out_dtype")
+    rejected(L.cch_gmm_i8_dequant_swiglu_out(P, P, P, P, P, P, 2, 8, 8, 8, 0, 5, None), "out_dtype")
+    rejected(L.cch_mx_gemm_out(P, P, P, P, P, 8, 8, 64, 0, 0, 2, None), "out_dtype")
 
 
 def test_routing_and_unpermute_arguments():

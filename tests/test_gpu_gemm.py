@@ -504,3 +504,54 @@ def test_grouped_tile_order_covers_every_tile_once():
     assert not np.isnan(outs[1]).any()
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[-1])
     assert_close(outs[1], gold, "per-XCD tile order")
+
+
+# ---------------------------------------------------------------- half-precision output
+
+@pytest.mark.parametrize("tiled", [True, False], ids=["tiled", "generic"])
+def test_fp16_output_of_the_int8_and_dense_mx_operators(tiled):
+    """IEEE half output (what the reference's int8 launchers write, tests/dynamic_tiling/impl/kernel_int8.cpp:16)
+    is the same fp32 result rounded to half: within the gate against the oracle and closer to it than bf16's
+    8 bits allow (the oracle's fp32 value against a correctly rounded half: at most 2^-11 apart, relative)."""
+    rng = np.random.default_rng(21)
+    e, t, k, n = 3, 300, 256, 256
+    gs = np.array([130, 0, 170], np.int32)
+    xi = rng.integers(-127, 128, (t, k)).astype(np.int8)
+    wi = rng.integers(-127, 128, (e, k, n)).astype(np.int8)
+    pt = rng.uniform(0.001, 0.02, t).astype(np.float32)
+    pc = rng.uniform(0.001, 0.02, (e, n)).astype(np.float32)
+    pa, sa = orc.mx_quant_rows(rand_bf16(rng, (t, k), 1.0), orc.E4M3)
+    pb, sb = orc.mx_quant_b(rand_bf16(rng, (k, n), 1.0), orc.E4M3, orc.RNE, 0)
+    golds = {
+        "dense": orc.gemm_i8_dequant(xi, wi[0], pt, pc[0]),
+        "gmm": np.concatenate([orc.gemm_i8_dequant(xi[:130], wi[0], pt[:130], pc[0]), orc.gemm_i8_dequant(xi[130:], wi[2], pt[130:], pc[2])]),
+        "swiglu": orc.gmm_i8_dequant_swiglu(xi, wi, gs, pt, pc),
+        "mx": orc.mx_gmm(pa, sa, pb[None], sb[None], n, k, orc.E4M3, 0),
+    }
+    cc.set_option("require_tiled_gemm", 1 if tiled else 0)
+    cc.set_option("force_generic_gemm", 0 if tiled else 1)
+    try:
+        for dt in (torch.float16, torch.bfloat16):
+            outs = {
+                "dense": cc.w8a8_matmul_dequant(dev(xi), dev(wi[0]), dev(pt), dev(pc[0]), 0, out_dtype=dt),
+                "gmm": cc.gmm_dequant(dev(xi), dev(wi), dev(gs), dev(pt), dev(pc), 0, out_dtype=dt),
+                "swiglu": cc.gmm_dequant_swiglu(dev(xi), dev(wi), dev(gs), dev(pt), dev(pc), 0, out_dtype=dt),
+                "mx": cc.mx_matmul(dev(pa), dev(sa), dev(pb), dev(sb), "e4m3", 0, out_dtype=dt),
+            }
+            for name, out in outs.items():
+                assert out.dtype == dt
+                got = out_f32(out)
+                assert_close(got, golds[name], (name, dt, tiled))
+                if dt == torch.float16:
+                    # 11 significant bits: relative error of a correctly rounded half is at most 2^-11
+                    big = np.abs(golds[name]) > 1.0   # away from cancellation, where fp32 summation order shows
+                    rel = np.abs(got - golds[name])[big] / np.abs(golds[name])[big]
+                    if name == "mx":
+                        # the matrix unit's fp32 summation differs from the oracle's by up to ~1e-3 on single
+                        # values; on average the half output must still beat what bf16 could give (2^-10)
+                        assert rel.mean() <= 2.0 ** -11 and rel.max() <= 2.0 ** -9, (name, rel.mean(), rel.max())
+                    else:
+                        assert rel.max() <= 2.0 ** -10, (name, rel.max())
+    finally:
+        cc.set_option("require_tiled_gemm", 0)
+        cc.set_option("force_generic_gemm", 0)
