@@ -106,7 +106,7 @@ def quant_inputs(dev, m, k, nsets):
     return out
 
 
-def quant_batch_time_us(sets, launches, warmup):
+def quant_batch_time_us(sets, launches, warmup, entry="cch_mx_quant_rows"):
     """Average duration of the config-1 MX quantiser over a queue of back-to-back launches.
 
     One launch lasts about 16 us, the same order as the cost of a pair of events or of two tensor
@@ -122,7 +122,7 @@ def quant_batch_time_us(sets, launches, warmup):
     stream = torch.cuda.current_stream().cuda_stream
 
     def launch(i):
-        _abi.check(lib.cch_mx_quant_rows(sets[i % len(sets)].data_ptr(), payload.data_ptr(), scales.data_ptr(), m, k, 0, 0, stream))
+        _abi.check(getattr(lib, entry)(sets[i % len(sets)].data_ptr(), payload.data_ptr(), scales.data_ptr(), m, k, 0, 0, stream))
 
     for i in range(warmup):
         launch(i)
@@ -256,6 +256,13 @@ def main():
         q_gbs = qbytes / (q_us * 1e-6) / 1e9
         extra["mx_quant_cfg1"] = {"gb_per_s": round(q_gbs, 1), "frac_of_hbm_peak": round(q_gbs / HBM_PEAK_GBS, 4),
                                   "us": round(q_us, 2), "bytes": qbytes, "buffers": "6 rotating input sets (352 MB), 120 queued launches"}
+        # the half-input twin of the quantiser on the same values
+        sets16 = [x.to(torch.float16) for x in sets]
+        h_us = quant_batch_time_us(sets16, 120, 1500, "cch_mx_quant_rows_f16")
+        extra["mx_quant_f16_input_cfg1_shape"] = {"gb_per_s": round(qbytes / (h_us * 1e-6) / 1e9, 1),
+                                                  "frac_of_hbm_peak": round(qbytes / (h_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                                                  "us": round(h_us, 2), "bytes": qbytes}
+        del sets16
         # the same rows quantised once and scattered as packed [payload | scales] rows to their top-2 destinations
         idx1 = torch.randperm(M1 * 2, device=dev).to(torch.int32)
         packed1 = torch.empty((M1 * 2, cc.packed_row_bytes(K1)), dtype=torch.uint8, device=dev)

@@ -32,6 +32,7 @@ PROTOTYPES = {
     "cch_stream_sync": [_P],
     "cch_stream_destroy": [_P],
     "cch_mx_quant_rows": [_P, _P, _P, _I64, _I64, _I, _I, _P],
+    "cch_mx_quant_rows_f16": [_P, _P, _P, _I64, _I64, _I, _I, _P],
     "cch_mx_quant_b": [_P, _P, _P, _I64, _I64, _I, _I, _I, _P],
     "cch_mx_quant_scatter_packed": [_P, _P, _P, _I64, _I64, _I, _I, _I, _P],
     "cch_moe_token_unpermute": [_P, _P, _P, _P, _I64, _I64, _I64, _I, _P],

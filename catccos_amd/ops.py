@@ -45,20 +45,21 @@ def scale_cols(k):
 
 
 def mx_quant(x, fmt="e4m3", rounding=ROUND_RNE):
-    """MX block quantisation along the last axis of a 2-D bf16 tensor.
+    """MX block quantisation along the last axis of a 2-D bf16 (or IEEE half) tensor.
 
     Returns (payload uint8 [M, K] or [M, ceil(K/2)] for FP4, scales uint8 [M, scale_cols(K)]).
     """
     fmt = _fmt(fmt)
     _require_gpu(x)
-    if x.dim() != 2 or x.dtype != torch.bfloat16:
-        raise ValueError("mx_quant expects a 2-D bfloat16 tensor")
+    if x.dim() != 2 or x.dtype not in (torch.bfloat16, torch.float16):
+        raise ValueError("mx_quant expects a 2-D bfloat16 (or float16) tensor")
     x = x.contiguous()
     m, k = x.shape
     pld = (k + 1) // 2 if fmt in _FP4 else k
     payload = torch.empty((m, pld), dtype=torch.uint8, device=x.device)
     scales = torch.empty((m, scale_cols(k)), dtype=torch.uint8, device=x.device)
-    check(_abi.lib().cch_mx_quant_rows(_ptr(x), _ptr(payload), _ptr(scales), m, k, fmt, rounding, _stream()))
+    fn = _abi.lib().cch_mx_quant_rows_f16 if x.dtype == torch.float16 else _abi.lib().cch_mx_quant_rows
+    check(fn(_ptr(x), _ptr(payload), _ptr(scales), m, k, fmt, rounding, _stream()))
     return payload, scales
 
 

@@ -81,6 +81,13 @@ int cch_stream_destroy(void *stream);
 int cch_mx_quant_rows(const void *x, void *payload, void *scales, int64_t m, int64_t k, int fmt, int rounding,
                       void *stream);
 
+/* The same quantiser for IEEE half input, the `half` instantiation of the reference's quantiser
+ * (MxQuantTraits<half>, include/catccos/epilogue/block/block_epilogue_dynamic_mx_quant.hpp:57-71:
+ * the input is widened to fp32 and the shared exponent is taken from the fp32 exponent field of the
+ * block maximum).  x: half [m,k]; outputs, formats and rounding rules as cch_mx_quant_rows. */
+int cch_mx_quant_rows_f16(const void *x, void *payload, void *scales, int64_t m, int64_t k, int fmt, int rounding,
+                          void *stream);
+
 /* Same quantiser for a right-hand GEMM operand b [k,n] (row-major bf16) with
  * blocks running down the k axis, i.e. what the reference's generators do for B
  * (examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/gen_data_mxfp8_mmrs.py:202-217).

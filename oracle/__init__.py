@@ -139,6 +139,20 @@ def mx_quant_rows(x_bf16, fmt=E4M3, rounding=RNE):
     return payload, scales
 
 
+def mx_quant_rows_f16(x_f16, fmt=E4M3, rounding=RNE):
+    """IEEE half bits (uint16 [M,K], or a float16 array) -> (payload, scales) as mx_quant_rows."""
+    x = np.asarray(x_f16)
+    if x.dtype == np.float16:
+        x = x.view(np.uint16)
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    m, k = x.shape
+    pld = (k + 1) // 2 if fmt in FP4_FORMATS else k
+    payload = np.empty((m, pld), dtype=np.uint8)
+    scales = np.empty((m, scale_cols(k)), dtype=np.uint8)
+    lib().orc_mx_quant_rows_f16(_p(x), _i64(m), _i64(k), fmt, rounding, _p(payload), _p(scales))
+    return payload, scales
+
+
 def packed_row_bytes(k, fmt=E4M3):
     """Bytes of one packed row: payload followed by the padded E8M0 scales."""
     return ((k + 1) // 2 if fmt in FP4_FORMATS else k) + scale_cols(k)

@@ -210,6 +210,24 @@ float orc_decode(uint8_t c, int fmt)
 
 /* --------------------------------------------------------- E8M0 exponent */
 
+/* IEEE half bits -> fp32 (exact; subnormals normalised, Inf/NaN kept). */
+float orc_f16_to_f32(uint16_t h)
+{
+    uint32_t sign = (uint32_t)(h >> 15) << 31, ex = (h >> 10) & 0x1Fu, man = h & 0x3FFu, u;
+    float f;
+    if (ex == 0) {
+        f = ldexpf((float)man, -24);
+        memcpy(&u, &f, 4);
+        u |= sign;
+    } else if (ex == 31) {
+        u = sign | 0x7F800000u | (man << 13);
+    } else {
+        u = sign | ((ex + 112u) << 23) | (man << 13);
+    }
+    memcpy(&f, &u, 4);
+    return f;
+}
+
 /*
  * Shared exponent of one block from its absolute maximum
  * (gen_mx_quant_allgather_data.py:168-189):
@@ -246,8 +264,8 @@ static int fmt_emax(int fmt) { build_tables(); return g_tab[fmt].emax; }
  *            idempotence on dequantised data (the check the reference's own
  *            run.sh performs), torch-cast cross-check on random data.
  */
-int orc_mx_quant_rows(const uint16_t *x, int64_t M, int64_t K, int fmt, int rounding,
-                      uint8_t *payload, uint8_t *scales)
+static int mx_quant_rows_impl(const uint16_t *x, int in_half, int64_t M, int64_t K, int fmt, int rounding,
+                              uint8_t *payload, uint8_t *scales)
 {
     build_tables();
     const int64_t nblk = (K + 31) / 32;
@@ -266,7 +284,7 @@ int orc_mx_quant_rows(const uint16_t *x, int64_t M, int64_t K, int fmt, int roun
             float amax = 0.0f;
             int bad = 0;
             for (int64_t k = k0; k < k1; k++) {
-                float v = fabsf(orc_bf16_to_f32(xr[k]));
+                float v = fabsf(in_half ? orc_f16_to_f32(xr[k]) : orc_bf16_to_f32(xr[k]));
                 if (v != v) bad = 1;
                 if (v > amax) amax = v;
             }
@@ -279,7 +297,7 @@ int orc_mx_quant_rows(const uint16_t *x, int64_t M, int64_t K, int fmt, int roun
             }
             if (e < -127) e = -127;
             for (int64_t k = k0; k < k1; k++) {
-                float v = orc_bf16_to_f32(xr[k]);
+                float v = in_half ? orc_f16_to_f32(xr[k]) : orc_bf16_to_f32(xr[k]);
                 /* division by 2^e is exact in fp32 unless the quotient is subnormal */
                 float y = is_nan ? NAN : ldexpf(v, -e);
                 uint8_t q = orc_encode(y, fmt, rounding);
@@ -289,6 +307,29 @@ int orc_mx_quant_rows(const uint16_t *x, int64_t M, int64_t K, int fmt, int roun
         }
     }
     return 0;
+}
+
+int orc_mx_quant_rows(const uint16_t *x, int64_t M, int64_t K, int fmt, int rounding,
+                      uint8_t *payload, uint8_t *scales)
+{
+    return mx_quant_rows_impl(x, 0, M, K, fmt, rounding, payload, scales);
+}
+
+/*
+ * The same quantiser on IEEE half input: the reference's `half` instantiation
+ * widens to fp32 and takes the shared exponent from the fp32 exponent field
+ * (MxQuantTraits<half>, include/catccos/epilogue/block/block_epilogue_dynamic_mx_quant.hpp:57-71:
+ * CalcType float, EXP_MASK 0x7F800000, SHR_NUM 23), then scales and casts as the
+ * bf16 path does.  The reference holds no golden for half input; the rule is the
+ * same OCP recipe applied to the widened values.
+ * pinned by: the independent numpy / torch recipe on half data incl. half
+ *            subnormals as block maxima, and equality with orc_mx_quant_rows on
+ *            values that both input types represent exactly.
+ */
+int orc_mx_quant_rows_f16(const uint16_t *x, int64_t M, int64_t K, int fmt, int rounding,
+                          uint8_t *payload, uint8_t *scales)
+{
+    return mx_quant_rows_impl(x, 1, M, K, fmt, rounding, payload, scales);
 }
 
 /*
