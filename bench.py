@@ -143,6 +143,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=100, help="untimed launches (about 55 ms: the clock's ramp from idle)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--set-option", action="append", default=[], metavar="NAME=VALUE",
+                    help="library switch for an A/B run, e.g. gemm_tile_order=0 (cch_set_option)")
     ap.add_argument("--only", choices=["copy", "quant"], help="profiling aid: run only a 512 MiB device copy (counter "
                     "calibration) or only the config-1 MX quantiser, print a short JSON line and exit")
     args = ap.parse_args()
@@ -176,6 +178,9 @@ def main():
     E, T, K, N = 32, 16384, 7168, 4096
     TRANS_B = 0   # W stored [E, K, N] as the configurations name it (B scales [E, K/64, N, 2])
     cc.set_option("require_tiled_gemm", 1)   # a fall-back to the generic kernels is an error here, not a slow number
+    for kv in args.set_option:
+        name, _, val = kv.partition("=")
+        cc.set_option(name, int(val))
     gs_host = zipf_groups(rng, T, E)
     gs = torch.from_numpy(gs_host).to(dev)
     x0 = (torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16)

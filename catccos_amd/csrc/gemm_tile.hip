@@ -261,6 +261,15 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             o16[i] = (v4u){0, 0, 0, 0};
     }
 
+    // Workgroups that take tiles: all of them, or (balance) just enough for the same number of
+    // rounds, in whole groups of eight so that every XCD keeps the same share.
+    int nwg = gridDim.x;
+    if (p.balance_rounds && total_tiles > 0) {
+        const int rounds = (total_tiles + (int)gridDim.x - 1) / (int)gridDim.x;
+        nwg = min((int)gridDim.x, (((total_tiles + rounds - 1) / rounds) + 7) & ~7);
+    }
+    nwg = uniform(nwg);
+
     int gi = 0;           // scale groups requested so far; group n lives in scale buffer n & 1
     int gbase = 0;        // value of gi when the current tile's group 0 was requested
 
@@ -271,11 +280,11 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         c.valid = t < total_tiles;
         c.lim = c.valid ? 0x7FFFFFFFu : 0u;
         t = max(min(t, total_tiles - 1), 0);
-        if (p.tile_order == 1 && (gridDim.x & 7) == 0 && t < total_tiles - total_tiles % (int)gridDim.x) {
+        if (p.tile_order == 1 && (nwg & 7) == 0 && t < total_tiles - total_tiles % nwg) {
             // Workgroup w of a round runs on XCD w % 8: give each XCD a run of gridDim.x / 8
             // consecutive tiles of the round (whole row tiles next to each other), so that its L2
             // fetches one or two A panels and the B panels of one or two experts per round.
-            const int G = gridDim.x, j = t / G, w = t - j * G;
+            const int G = nwg, j = t / G, w = t - j * G;
             t = j * G + (w & 7) * (G >> 3) + (w >> 3);
         }
         const int tr = t / n_tiles, nt = t - tr * n_tiles;
@@ -384,7 +393,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     };
 
     TileCtx cur, nxt;
-    int t = blockIdx.x, parity = 0;
+    int t = (int)blockIdx.x < nwg ? (int)blockIdx.x : total_tiles, parity = 0;
     int gstep = 0;        // K-steps executed by this workgroup so far; ring stage = gstep & 1
     bool first = true;
     decode(t, cur);
@@ -610,7 +619,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             int nk = ksteps;
             asm volatile("" : "+s"(nk));
             for (int kt = 0; kt + 2 < nk; kt++) step(IC<0>{}, mta_c, kt);
-            decode(t + gridDim.x, nxt);
+            decode(t + nwg, nxt);
             step(IC<1>{}, mta_c, nk - 2);
             step(IC<2>{}, mta_c, nk - 1);
         };
@@ -708,7 +717,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         }
         cur = nxt;
         gbase = nbase;
-        t += gridDim.x;
+        t += nwg;
         parity ^= 1;
     }
 }

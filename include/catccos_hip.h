@@ -271,7 +271,10 @@ int cch_dyn_quant_i8_rows_smooth(const void *x, const int32_t *src_rows, const f
  * order in which the persistent workgroups of the tiled kernels walk the output tiles: 0 = row-major
  * over (row tile, column tile), 1 = each XCD takes a run of consecutive tiles of every round (whole
  * row tiles next to each other: fewer token and weight panels per L2), -1 (default) = 1 for grouped
- * problems, 0 for dense ones.  Results do not depend on it. */
+ * problems, 0 for dense ones; "gemm_balance_rounds" = 1 lets only as many workgroups take tiles as
+ * the number of rounds needs (640 tiles on 256 CUs are three rounds: 216 workgroups do them in the
+ * same three, with fewer CUs competing for L2 and memory), 0 (default) uses every CU.  Results do not
+ * depend on either. */
 int cch_set_option(const char *name, int value);
 
 #ifdef __cplusplus

@@ -492,17 +492,20 @@ def test_grouped_tile_order_covers_every_tile_once():
     outs = {}
     cc.set_option("require_tiled_gemm", 1)
     try:
-        for order in (0, 1, -1):
-            cc.set_option("gemm_tile_order", order)
+        for order in (0, 1, -1, 2):
+            # 2: the default order again, with a balanced count of workgroups taking tiles instead of every CU
+            cc.set_option("gemm_balance_rounds", 1 if order == 2 else 0)
+            cc.set_option("gemm_tile_order", -1 if order == 2 else order)
             # the output starts as NaN: a tile that no workgroup computes would keep it
             out = torch.full((t, n), float("nan"), dtype=torch.bfloat16, device="cuda")
             cc.mx_grouped_matmul_mapped(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), dev(ident), out, "e4m3", 0)
             outs[order] = out_f32(out)
     finally:
         cc.set_option("gemm_tile_order", -1)
+        cc.set_option("gemm_balance_rounds", 0)
         cc.set_option("require_tiled_gemm", 0)
     assert not np.isnan(outs[1]).any()
-    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[-1])
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[-1]) and np.array_equal(outs[1], outs[2])
     assert_close(outs[1], gold, "per-XCD tile order")
 
 
