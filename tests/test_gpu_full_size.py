@@ -1,0 +1,120 @@
+"""The five configurations at their full sizes on the tiled kernels: a random sample of output rows
+against the oracle (the gate of the small-shape tests), plus a property that holds at any size and needs
+no oracle - an exact power-of-two scaling (bf16 rounding commutes with a factor of two) or the equality
+of the grouped result with per-expert dense calls (same accumulation order along K for every element).
+Inputs are drawn on the GPU and quantised by the library's own quantisers, which have bit-exact parity
+tests of their own."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+import catccos_amd as cc
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def zipf_groups(rng, t, e):
+    p = (np.arange(e) + 1.0) ** -1.1
+    p = p[rng.permutation(e)]
+    gs = rng.multinomial(t, p / p.sum()).astype(np.int32)
+    if gs.min() > 0:
+        i, j = int(gs.argmin()), int(gs.argmax())
+        gs[j] += gs[i]
+        gs[i] = 0
+    return gs
+
+
+def close(got, want, what):
+    m = orc.compare(got, want)
+    assert m["max_rel_floor1"] <= TOL and m["max_rel_floor_rms"] <= TOL, (what, m)
+
+
+@pytest.fixture(autouse=True)
+def tiled_only():
+    cc.set_option("require_tiled_gemm", 1)
+    yield
+    cc.set_option("require_tiled_gemm", 0)
+
+
+def test_cfg2_w8a8_dequant_8192x4096x8192():
+    torch.manual_seed(2)
+    rng = np.random.default_rng(2)
+    m, k, n = 8192, 4096, 8192
+    a = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda")
+    b = torch.randint(-127, 128, (k, n), dtype=torch.int8, device="cuda")
+    pt = torch.rand(m, device="cuda") * 0.019 + 0.001
+    pc = torch.rand(n, device="cuda") * 0.019 + 0.001
+    out = cc.w8a8_matmul_dequant(a, b, pt, pc, 0)
+    rows = np.sort(rng.choice(m, 48, replace=False)).astype(np.int64)
+    gold = orc.gemm_i8_dequant(a.cpu().numpy(), b.cpu().numpy(), pt.cpu().numpy(), pc.cpu().numpy(), 0, rows=rows)
+    close(out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), gold, "cfg2 sample")
+    out2 = cc.w8a8_matmul_dequant(a, b, pt * 2, pc, 0)
+    assert torch.equal(out2.float(), out.float() * 2)          # exact: per-token scale times two
+
+
+def test_cfg3_mxfp8_dense_4096x2048x7168():
+    torch.manual_seed(3)
+    rng = np.random.default_rng(3)
+    m, k, n = 4096, 2048, 7168
+    a, sa = cc.mx_quant(torch.randn(m, k, device="cuda").to(torch.bfloat16), "e4m3")
+    b, sb = cc.mx_quant_b(torch.randn(k, n, device="cuda").to(torch.bfloat16), "e4m3", trans_b=0)
+    out = cc.mx_matmul(a, sa, b, sb, "e4m3", 0)
+    rows = np.sort(rng.choice(m, 48, replace=False)).astype(np.int64)
+    gold = orc.mx_gmm(a.cpu().numpy(), sa.cpu().numpy(), b.cpu().numpy()[None], sb.cpu().numpy()[None], n, k, orc.E4M3, 0, rows=rows)
+    close(out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), gold, "cfg3 sample")
+    out2 = cc.mx_matmul(a, sa + 1, b, sb, "e4m3", 0)           # every A block scale doubled
+    assert torch.equal(out2.float(), out.float() * 2)
+
+
+def test_cfg4_moe_w8a8_swiglu_8192_tokens_16_experts():
+    torch.manual_seed(4)
+    rng = np.random.default_rng(4)
+    e, t, k, n = 16, 8192, 7168, 4096
+    gs_h = zipf_groups(rng, t, e)
+    gs = torch.from_numpy(gs_h).cuda()
+    x = torch.randint(-127, 128, (t, k), dtype=torch.int8, device="cuda")
+    w = torch.randint(-127, 128, (e, k, n), dtype=torch.int8, device="cuda")
+    pt = torch.rand(t, device="cuda") * 0.019 + 0.001
+    pc = torch.rand(e, n, device="cuda") * 0.019 + 0.001
+    out = cc.gmm_dequant_swiglu(x, w, gs, pt, pc, 0)
+    rows = np.sort(rng.choice(t, 32, replace=False)).astype(np.int64)
+    gold = orc.gmm_i8_dequant_swiglu(x.cpu().numpy(), w.cpu().numpy(), gs_h, pt.cpu().numpy(), pc.cpu().numpy(), rows=rows)
+    close(out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), gold, "cfg4 sample")
+    # every expert on its own, as a one-group call over its rows, gives the same bits
+    r0 = 0
+    for g in range(e):
+        sz = int(gs_h[g])
+        if sz:
+            one = cc.gmm_dequant_swiglu(x[r0:r0 + sz], w[g:g + 1], gs[g:g + 1], pt[r0:r0 + sz], pc[g:g + 1], 0)
+            assert torch.equal(one, out[r0:r0 + sz]), g
+        r0 += sz
+
+
+@pytest.mark.parametrize("fmt,ofmt", [("e2m1", orc.E2M1), ("e4m3", orc.E4M3)], ids=["cfg5-mxfp4", "headline-mxfp8"])
+def test_cfg5_mx_grouped_16384_tokens_32_experts(fmt, ofmt):
+    torch.manual_seed(5)
+    rng = np.random.default_rng(5)
+    e, t, k, n = 32, 16384, 7168, 4096
+    gs_h = zipf_groups(rng, t, e)
+    gs = torch.from_numpy(gs_h).cuda()
+    a, sa = cc.mx_quant((torch.randn(t, k, device="cuda") * 0.02).to(torch.bfloat16), fmt)
+    pw = n // 2 if fmt == "e2m1" else n
+    b = torch.empty((e, k, pw), dtype=torch.uint8, device="cuda")
+    sb = torch.empty((e, k // 64, n, 2), dtype=torch.uint8, device="cuda")
+    for g in range(e):
+        b[g], sb[g] = cc.mx_quant_b((torch.randn(k, n, device="cuda") * 0.02).to(torch.bfloat16), fmt, trans_b=0)
+    out = cc.mx_grouped_matmul(a, sa, b, sb, gs, fmt, 0)
+    rows = np.sort(rng.choice(t, 24, replace=False)).astype(np.int64)
+    gold = orc.mx_gmm(a.cpu().numpy(), sa.cpu().numpy(), b.cpu().numpy(), sb.cpu().numpy(), n, k, ofmt, 0, group_sizes=gs_h, rows=rows)
+    close(out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), gold, fmt + " sample")
+    # per-expert dense calls equal the grouped result bit for bit; empty groups contribute nothing
+    r0 = 0
+    for g in range(e):
+        sz = int(gs_h[g])
+        if sz:
+            one = cc.mx_matmul(a[r0:r0 + sz], sa[r0:r0 + sz], b[g], sb[g], fmt, 0)
+            assert torch.equal(one, out[r0:r0 + sz]), g
+        r0 += sz
+    assert r0 == t
