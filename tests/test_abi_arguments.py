@@ -20,6 +20,11 @@ def test_quantiser_arguments():
     rejected(L.cch_mx_quant_rows(P, P, P, 4, 64, 9, 0, None))          # format
     rejected(L.cch_mx_quant_rows(P, P, P, 4, 64, 0, 5, None))          # rounding
     rejected(L.cch_mx_quant_rows(None, P, P, 4, 64, 0, 0, None))
+    rejected(L.cch_mx_quant_rows_f16(P, P, P, -1, 64, 0, 0, None), "cch_mx_quant_rows_f16")
+    rejected(L.cch_mx_quant_rows_f16(P, P, P, 4, 64, 9, 0, None), "format")
+    rejected(L.cch_mx_quant_rows_f16(P, P, P, 4, 64, 0, 5, None), "rounding")
+    rejected(L.cch_mx_quant_rows_f16(None, P, P, 4, 64, 0, 0, None), "null")
+    assert L.cch_mx_quant_rows_f16(None, None, None, 0, 64, 0, 0, None) == _abi.OK
     rejected(L.cch_mx_quant_scatter_packed(P, P, P, 4, 64, -1, 0, 0, None), "top_k")
     assert L.cch_mx_quant_scatter_packed(P, P, P, 4, 64, 0, 0, 0, None) == _abi.OK   # no routes: nothing to do
     rejected(L.cch_mx_quant_scatter_packed(P, P, P, 4, 64, 9, 0, 0, None), "top_k")
