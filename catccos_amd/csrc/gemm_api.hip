@@ -14,6 +14,7 @@ static std::atomic<int> g_force_generic{0};
 static std::atomic<int> g_require_tiled{0};
 static std::atomic<int> g_tile_order{-1};   // -1: chosen per problem
 static std::atomic<int> g_balance{0};
+static std::atomic<int> g_nt_small{1};
 
 static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
 {
@@ -22,6 +23,7 @@ static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
     const int order = g_tile_order.load();
     p.tile_order = order >= 0 ? order : (p.group_sizes != nullptr && p.num_groups > 1);
     p.balance_rounds = g_balance.load();
+    p.nt_b_max_tiles = (p.group_sizes != nullptr && p.num_groups > 1) ? g_nt_small.load() : 0;
     if (!g_force_generic.load() && gemm_tile_supports(p, kind, epi)) return launch_gemm_tile(p, kind, epi, stream);
     if (g_require_tiled.load())
         return fail(CCH_ENOSUP, "the tiled MFMA kernels do not take this problem (T=%d N=%d K=%d trans_b=%d) and "
@@ -50,6 +52,10 @@ int cch_set_option(const char *name, int value)
     }
     if (strcmp(name, "require_tiled_gemm") == 0) {
         g_require_tiled.store(value);
+        return CCH_OK;
+    }
+    if (strcmp(name, "gemm_nt_small_experts") == 0) {
+        g_nt_small.store(value);
         return CCH_OK;
     }
     if (strcmp(name, "gemm_balance_rounds") == 0) {

@@ -138,6 +138,18 @@ __device__ __forceinline__ void load16_to_lds(Rsrc rs, uint32_t voff, uint32_t s
                  : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
                  : "memory", "m0");
 }
+// The same load with the non-temporal hint: the line is not kept in L2 after use (weight panels of
+// experts so small that no other workgroup reads them again).
+__device__ __forceinline__ void load16_to_lds_nt(Rsrc rs, uint32_t voff, uint32_t soff, uint32_t lds_addr)
+{
+    rs = scalar_rsrc(rs);
+    soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
+    lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
+                 : "memory", "m0");
+}
 // The same 16-byte load, performed only when `enable` (wave-uniform) is non-zero, without a
 // branch: the load is issued with an empty EXEC mask otherwise.  Keeps the K loop one basic
 // block, which the register allocator handles far better than a loop with a diamond in it.
@@ -346,14 +358,19 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     // Requests K-step kt of tile c into ring stage `stage`: NV instructions per wave, issued one
     // at a time (piece 0..NV-1) so that they interleave with MFMAs instead of reaching the
     // texture addresser as one burst from all eight waves.
-    auto issue_piece = [&](const TileCtx &c, int kt, int stage, auto piece_c) {
+    auto issue_piece = [&](const TileCtx &c, int kt, int stage, auto piece_c, auto ntb_c) {
         constexpr int piece = decltype(piece_c)::value;
+        constexpr bool NTB = decltype(ntb_c)::value != 0;
         const uint32_t lds = lds_base + (uint32_t)(RING_OFF + stage * STAGE_BYTES) + (uint32_t)(wave * NJ) * 1024u;
         if constexpr (piece < NJ) {
             load16_to_lds(c.rs_a, c.off_a[piece], (uint32_t)kt * BKB, lds + piece * 1024u);
         } else if constexpr (piece < 2 * NJ) {
-            load16_to_lds(c.rs_b, c.off_b[piece - NJ], TB ? (uint32_t)kt * BKB : (uint32_t)kt * (BKB * EPB) * (uint32_t)ldb,
-                          lds + PANEL_BYTES + (piece - NJ) * 1024u);
+            if constexpr (NTB)
+                load16_to_lds_nt(c.rs_b, c.off_b[piece - NJ], TB ? (uint32_t)kt * BKB : (uint32_t)kt * (BKB * EPB) * (uint32_t)ldb,
+                                 lds + PANEL_BYTES + (piece - NJ) * 1024u);
+            else
+                load16_to_lds(c.rs_b, c.off_b[piece - NJ], TB ? (uint32_t)kt * BKB : (uint32_t)kt * (BKB * EPB) * (uint32_t)ldb,
+                              lds + PANEL_BYTES + (piece - NJ) * 1024u);
         }
     };
     // Scale group `grp` of tile c (steps grp*SPG .. grp*SPG+SPG-1) into scale buffer `buf`: waves
@@ -365,7 +382,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                              lds_base + (uint32_t)(SCALE_OFF + buf * SCALE_BUF) + (uint32_t)(wave >= 4) * 4096u + (uint32_t)(wave & 3) * 1024u);
     };
     auto issue_step = [&](const TileCtx &c, int kt, int stage) {
-        static_for<NV>([&](auto piece_c) { issue_piece(c, kt, stage, piece_c); });
+        static_for<NV>([&](auto piece_c) { issue_piece(c, kt, stage, piece_c, IC<0>{}); });
     };
 
     // Tile set-up: epilogue parameters of the tile (per-token / per-channel scales) and its
@@ -509,7 +526,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // it, two steps ahead of its use.  Everything that follows the barrier is threaded
         // between the step's remaining MFMAs, one or two instructions at a time, so that the
         // matrix pipe keeps running while the wave issues them.
-        auto step = [&](auto mode_c, auto mta_c, int kt) {
+        auto step = [&](auto mode_c, auto mta_c, auto ntb_c, int kt) {
             constexpr int MODE = decltype(mode_c)::value;
             constexpr int MTA = decltype(mta_c)::value;   // row blocks of this wave that hold rows of the group
             const int stage = gstep & 1, nstage = stage ^ 1;
@@ -551,7 +568,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 if constexpr (MODE == 0) {
                     static_for<PER_SLOT>([&](auto q_c) {
                         constexpr int piece = first_piece + decltype(q_c)::value;
-                        if constexpr (piece < NV) issue_piece(cur, kt + 2, stage, IC<piece>{});
+                        if constexpr (piece < NV) issue_piece(cur, kt + 2, stage, IC<piece>{}, ntb_c);
                         else if constexpr (piece == NV && MX) {
                             issue_scales(newgrp, cur, (kt + 2) / SPG, gi & 1);
                         }
@@ -603,7 +620,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // each count, and a wave whose rows lie wholly past the end of a short group issues its
         // requests and barriers but no matrix instruction (its SIMD then belongs to the other
         // wave it hosts, which covers the other half of the tile's rows).
-        auto k_loop = [&](auto mta_c) {
+        auto k_loop = [&](auto mta_c, auto ntb_c) {
             constexpr int MTA = decltype(mta_c)::value;
             const int stage = gstep & 1;
             if constexpr (MTA > 0) {
@@ -618,17 +635,28 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             // held in registers through the K loop.
             int nk = ksteps;
             asm volatile("" : "+s"(nk));
-            for (int kt = 0; kt + 2 < nk; kt++) step(IC<0>{}, mta_c, kt);
+            for (int kt = 0; kt + 2 < nk; kt++) step(IC<0>{}, mta_c, ntb_c, kt);
             decode(t + nwg, nxt);
-            step(IC<1>{}, mta_c, nk - 2);
-            step(IC<2>{}, mta_c, nk - 1);
+            step(IC<1>{}, mta_c, ntb_c, nk - 2);
+            step(IC<2>{}, mta_c, ntb_c, nk - 1);
         };
         const int mta = uniform(min(max((cur.m_end - cur.m0 - wm * WM + 31) >> 5, 0), MT));
-        if (mta == MT) k_loop(IC<MT>{});
-        else if (mta == 0) k_loop(IC<0>{});
-        else if (mta == 1) k_loop(IC<1>{});
-        else if (mta == 2) k_loop(IC<2>{});
-        else k_loop(IC<3>{});
+        // Weight panels of an expert with at most nt_b_max_tiles row tiles are read by that many
+        // workgroups and never again: their steady-state requests carry the non-temporal hint.
+        const bool ntb = uniform(p.nt_b_max_tiles > 0 && tab.tile_start[cur.e + 1] - tab.tile_start[cur.e] <= p.nt_b_max_tiles);
+        if (ntb) {
+            if (mta == MT) k_loop(IC<MT>{}, IC<1>{});
+            else if (mta == 0) k_loop(IC<0>{}, IC<1>{});
+            else if (mta == 1) k_loop(IC<1>{}, IC<1>{});
+            else if (mta == 2) k_loop(IC<2>{}, IC<1>{});
+            else k_loop(IC<3>{}, IC<1>{});
+        } else {
+            if (mta == MT) k_loop(IC<MT>{}, IC<0>{});
+            else if (mta == 0) k_loop(IC<0>{}, IC<0>{});
+            else if (mta == 1) k_loop(IC<1>{}, IC<0>{});
+            else if (mta == 2) k_loop(IC<2>{}, IC<0>{});
+            else k_loop(IC<3>{}, IC<0>{});
+        }
         first = false;
 
         // Epilogue.  Lane (r, g) holds, for sub-tile (i, j), column r and rows

@@ -273,8 +273,11 @@ int cch_dyn_quant_i8_rows_smooth(const void *x, const int32_t *src_rows, const f
  * row tiles next to each other: fewer token and weight panels per L2), -1 (default) = 1 for grouped
  * problems, 0 for dense ones; "gemm_balance_rounds" = 1 lets only as many workgroups take tiles as
  * the number of rounds needs (640 tiles on 256 CUs are three rounds: 216 workgroups do them in the
- * same three, with fewer CUs competing for L2 and memory), 0 (default) uses every CU.  Results do not
- * depend on either. */
+ * same three, with fewer CUs competing for L2 and memory), 0 (default) uses every CU;
+ * "gemm_nt_small_experts" = n: in grouped problems the weight requests of an expert with at most n row
+ * tiles of 256 rows carry the non-temporal hint (its panels are read by that many workgroups and never
+ * again, so they need not stay in L2); default 1, 0 switches it off.  Results do not depend on any of
+ * them. */
 int cch_set_option(const char *name, int value);
 
 #ifdef __cplusplus

@@ -492,10 +492,13 @@ def test_grouped_tile_order_covers_every_tile_once():
     outs = {}
     cc.set_option("require_tiled_gemm", 1)
     try:
-        for order in (0, 1, -1, 2):
+        for order in (0, 1, -1, 2, 3):
             # 2: the default order again, with a balanced count of workgroups taking tiles instead of every CU
+            # 3: the default order without non-temporal weight requests (3 as threshold: with them for every
+            #    expert of up to three row tiles; the default is one)
             cc.set_option("gemm_balance_rounds", 1 if order == 2 else 0)
-            cc.set_option("gemm_tile_order", -1 if order == 2 else order)
+            cc.set_option("gemm_nt_small_experts", 3 if order == 3 else 0 if order == 0 else 1)
+            cc.set_option("gemm_tile_order", -1 if order >= 2 else order)
             # the output starts as NaN: a tile that no workgroup computes would keep it
             out = torch.full((t, n), float("nan"), dtype=torch.bfloat16, device="cuda")
             cc.mx_grouped_matmul_mapped(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), dev(ident), out, "e4m3", 0)
@@ -503,9 +506,10 @@ def test_grouped_tile_order_covers_every_tile_once():
     finally:
         cc.set_option("gemm_tile_order", -1)
         cc.set_option("gemm_balance_rounds", 0)
+        cc.set_option("gemm_nt_small_experts", 1)
         cc.set_option("require_tiled_gemm", 0)
     assert not np.isnan(outs[1]).any()
-    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[-1]) and np.array_equal(outs[1], outs[2])
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[-1]) and np.array_equal(outs[1], outs[2]) and np.array_equal(outs[1], outs[3])
     assert_close(outs[1], gold, "per-XCD tile order")
 
 
