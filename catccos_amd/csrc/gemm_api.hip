@@ -15,6 +15,7 @@ static std::atomic<int> g_require_tiled{0};
 static std::atomic<int> g_tile_order{-1};   // -1: chosen per problem
 static std::atomic<int> g_balance{0};
 static std::atomic<int> g_nt_small{1};
+static std::atomic<int> g_nt_out{-1};      // -1: chosen per problem
 
 static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
 {
@@ -23,6 +24,8 @@ static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
     const int order = g_tile_order.load();
     p.tile_order = order >= 0 ? order : (p.group_sizes != nullptr && p.num_groups > 1);
     p.balance_rounds = g_balance.load();
+    const int nto = g_nt_out.load();
+    p.nt_out = nto >= 0 ? nto : (kind == KIND_F4);
     p.nt_b_max_tiles = (p.group_sizes != nullptr && p.num_groups > 1) ? g_nt_small.load() : 0;
     if (!g_force_generic.load() && gemm_tile_supports(p, kind, epi)) return launch_gemm_tile(p, kind, epi, stream);
     if (g_require_tiled.load())
@@ -56,6 +59,10 @@ int cch_set_option(const char *name, int value)
     }
     if (strcmp(name, "gemm_nt_small_experts") == 0) {
         g_nt_small.store(value);
+        return CCH_OK;
+    }
+    if (strcmp(name, "gemm_nt_output") == 0) {
+        g_nt_out.store(value);
         return CCH_OK;
     }
     if (strcmp(name, "gemm_balance_rounds") == 0) {

@@ -35,6 +35,7 @@ struct GemmProblem {
     int64_t b_stride;        // bytes between experts in b
     int64_t sb_stride;       // bytes between experts in sb
     int nt_b_max_tiles;      // tiled kernels: non-temporal weight requests for experts with at most this many row tiles (0: never)
+    int nt_out;              // tiled kernels: output stores carry the non-temporal hint
     int balance_rounds;      // tiled kernels: use only as many workgroups as the round count needs
     int tile_order;          // tiled kernels: 0 = row-major over (row tile, column tile); 1 = runs of consecutive tiles per XCD
 };

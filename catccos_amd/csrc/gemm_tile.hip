@@ -738,8 +738,9 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                         out_row = has_map ? (uint32_t)mapped : out_row;
                     }
                     const uint32_t off = ok ? (out_row * (uint32_t)p.n_out + (uint32_t)col) * 2u : 0xFFFFFFF0u;
-                    __builtin_amdgcn_raw_buffer_store_b128((v4u){(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]},
-                                                           rs_out, (int)off, 0, 0);
+                    const v4u sv = (v4u){(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]};
+                    if (p.nt_out) __builtin_amdgcn_raw_buffer_store_b128(sv, rs_out, (int)off, 0, 2);   // non-temporal
+                    else __builtin_amdgcn_raw_buffer_store_b128(sv, rs_out, (int)off, 0, 0);
                 }
             }
         }

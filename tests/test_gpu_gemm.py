@@ -498,6 +498,7 @@ def test_grouped_tile_order_covers_every_tile_once():
             #    expert of up to three row tiles; the default is one)
             cc.set_option("gemm_balance_rounds", 1 if order == 2 else 0)
             cc.set_option("gemm_nt_small_experts", 3 if order == 3 else 0 if order == 0 else 1)
+            cc.set_option("gemm_nt_output", 1 if order == 3 else 0 if order == 0 else -1)
             cc.set_option("gemm_tile_order", -1 if order >= 2 else order)
             # the output starts as NaN: a tile that no workgroup computes would keep it
             out = torch.full((t, n), float("nan"), dtype=torch.bfloat16, device="cuda")
@@ -507,6 +508,7 @@ def test_grouped_tile_order_covers_every_tile_once():
         cc.set_option("gemm_tile_order", -1)
         cc.set_option("gemm_balance_rounds", 0)
         cc.set_option("gemm_nt_small_experts", 1)
+        cc.set_option("gemm_nt_output", -1)
         cc.set_option("require_tiled_gemm", 0)
     assert not np.isnan(outs[1]).any()
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[-1]) and np.array_equal(outs[1], outs[2]) and np.array_equal(outs[1], outs[3])
