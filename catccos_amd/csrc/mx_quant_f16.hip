@@ -39,6 +39,8 @@ __device__ __forceinline__ uint32_t shared_exp_byte_f32(float amax, bool is_nan,
 typedef short s16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // Round-to-nearest-even payloads of 8 packed halves (w[i] = elements 2i, 2i+1) with gfx950's fused
 // conversions, which divide by the power-of-two scale and round straight from packed half.  The
@@ -104,9 +106,10 @@ __global__ __launch_bounds__(F16Q_THREADS) void mx_quant_rows_f16_kernel(const u
         uint32_t h[8];
         if (VEC) {
             if (k0 < k) {
-                const uint4 v = *reinterpret_cast<const uint4 *>(xr + k0);
-                h[0] = v.x & 0xFFFFu; h[1] = v.x >> 16; h[2] = v.y & 0xFFFFu; h[3] = v.y >> 16;
-                h[4] = v.z & 0xFFFFu; h[5] = v.z >> 16; h[6] = v.w & 0xFFFFu; h[7] = v.w >> 16;
+                // streamed once: non-temporal, like the stores below
+                const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xr + k0));
+                h[0] = v[0] & 0xFFFFu; h[1] = v[0] >> 16; h[2] = v[1] & 0xFFFFu; h[3] = v[1] >> 16;
+                h[4] = v[2] & 0xFFFFu; h[5] = v[2] >> 16; h[6] = v[3] & 0xFFFFu; h[7] = v[3] >> 16;
             } else {
 #pragma unroll
                 for (int i = 0; i < 8; i++) h[i] = 0;
@@ -146,7 +149,7 @@ __global__ __launch_bounds__(F16Q_THREADS) void mx_quant_rows_f16_kernel(const u
                                code[6] << 24 | code[7] << 28;
             uint8_t *pr = payload + row * pld + (k0 >> 1);
             if (VEC) {
-                if (k0 < k) *reinterpret_cast<uint32_t *>(pr) = w;
+                if (k0 < k) __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(pr));
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; i++)
@@ -157,7 +160,7 @@ __global__ __launch_bounds__(F16Q_THREADS) void mx_quant_rows_f16_kernel(const u
             const uint32_t hi = code[4] | code[5] << 8 | code[6] << 16 | code[7] << 24;
             uint8_t *pr = payload + row * pld + k0;
             if (VEC) {
-                if (k0 < k) *reinterpret_cast<uint2 *>(pr) = make_uint2(lo, hi);
+                if (k0 < k) __builtin_nontemporal_store((u32x2){lo, hi}, reinterpret_cast<u32x2 *>(pr));
             } else {
 #pragma unroll
                 for (int i = 0; i < 8; i++)
