@@ -16,7 +16,7 @@
 
 namespace cch {
 
-constexpr int F16Q_THREADS = 256;
+constexpr int F16Q_THREADS = 512;
 
 __device__ __forceinline__ float half_bits_to_f32(uint32_t h)
 {
@@ -190,7 +190,7 @@ static int launch_f16(const void *x, void *payload, void *scales, int64_t m, int
     CCH_HIP(hipGetDevice(&dev));
     CCH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     const int64_t want = (total + F16Q_THREADS - 1) / F16Q_THREADS;
-    const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>(want, (int64_t)cus * 16));
+    const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>(want, (int64_t)cus * 8));
     // 16-byte loads, 8-byte (FP8) or 4-byte (FP4) stores: whole groups and aligned rows
     const bool vec = k % 8 == 0 && aligned(x, 16) && aligned(payload, 8);
     const uint16_t *xi = static_cast<const uint16_t *>(x);
