@@ -8,7 +8,8 @@
 namespace cch {
 int launch_gemm_naive(const GemmProblem &p, int kind, int epi, hipStream_t stream);
 int launch_gemm_tile(const GemmProblem &p, int kind, int epi, hipStream_t stream);
-bool gemm_tile_supports(const GemmProblem &p, int kind, int epi);
+const char *gemm_tile_unsupported(const GemmProblem &p, int kind, int epi);
+bool quant_set_option(const char *name, int value);   // mx_quant.hip
 
 static std::atomic<int> g_force_generic{0};
 static std::atomic<int> g_require_tiled{0};
@@ -27,10 +28,21 @@ static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
     const int nto = g_nt_out.load();
     p.nt_out = nto >= 0 ? nto : (kind == KIND_F4);
     p.nt_b_max_tiles = (p.group_sizes != nullptr && p.num_groups > 1) ? g_nt_small.load() : 0;
-    if (!g_force_generic.load() && gemm_tile_supports(p, kind, epi)) return launch_gemm_tile(p, kind, epi, stream);
+    const bool forced = g_force_generic.load() != 0;
+    const char *why = forced ? "force_generic_gemm is set" : gemm_tile_unsupported(p, kind, epi);
+    if (why == nullptr) return launch_gemm_tile(p, kind, epi, stream);
     if (g_require_tiled.load())
-        return fail(CCH_ENOSUP, "the tiled MFMA kernels do not take this problem (T=%d N=%d K=%d trans_b=%d) and "
-                                "require_tiled_gemm is set", p.T, p.N, p.K, p.trans_b);
+        return fail(CCH_ENOSUP, "the tiled MFMA kernels do not take this problem (T=%d N=%d K=%d trans_b=%d: %s) and "
+                                "require_tiled_gemm is set", p.T, p.N, p.K, p.trans_b, why);
+    // The generic kernels are orders of magnitude slower: leave a note for cch_last_error() on every
+    // such call (the call still succeeds) and say it once per process on stderr.
+    fail(CCH_OK, "note: T=%d N=%d K=%d trans_b=%d ran on the one-thread-per-element kernels: %s", p.T, p.N, p.K, p.trans_b, why);
+    if (!forced) {
+        static std::atomic<int> told{0};
+        if (told.exchange(1) == 0)
+            fprintf(stderr, "[WARN] catccos_hip: GEMM T=%d N=%d K=%d trans_b=%d falls back to the generic kernels (%s); "
+                            "further fall-backs are reported through cch_last_error() only\n", p.T, p.N, p.K, p.trans_b, why);
+    }
     return launch_gemm_naive(p, kind, epi, stream);
 }
 
@@ -73,6 +85,7 @@ int cch_set_option(const char *name, int value)
         g_tile_order.store(value);
         return CCH_OK;
     }
+    if (quant_set_option(name, value)) return CCH_OK;
     return fail(CCH_EINVAL, "cch_set_option: unknown option %s", name);
 }
 
@@ -120,7 +133,7 @@ int cch_gmm_i8_dequant_swiglu_out(const void *x, const void *w, const int32_t *g
     CCH_REQUIRE(out_dtype == CCH_OUT_BF16 || out_dtype == CCH_OUT_FP16, "cch_gmm_i8_dequant_swiglu: out_dtype %d", out_dtype);
     CCH_REQUIRE(trans_b == 0 || trans_b == 1, "cch_gmm_i8_dequant_swiglu: trans_b %d", trans_b);
     CCH_REQUIRE(n % 2 == 0, "cch_gmm_i8_dequant_swiglu: n=%lld must be even (gate | up halves)", (long long)n);
-    CCH_REQUIRE(num_experts >= 1 && num_experts <= 65535, "cch_gmm_i8_dequant_swiglu: num_experts=%lld", (long long)num_experts);
+    CCH_REQUIRE(num_experts >= 1 && num_experts <= MAX_GROUPS, "cch_gmm_i8_dequant_swiglu: num_experts=%lld outside 1..%d", (long long)num_experts, MAX_GROUPS);
     if (t == 0 || n == 0) return CCH_OK;
     CCH_REQUIRE(out && per_tok && per_ch && group_sizes && (k == 0 || (x && w)), "cch_gmm_i8_dequant_swiglu: null pointer");
     GemmProblem p{};
@@ -152,7 +165,7 @@ int cch_gmm_i8_dequant_out(const void *x, const void *w, const int32_t *group_si
     if (rc) return rc;
     CCH_REQUIRE(out_dtype == CCH_OUT_BF16 || out_dtype == CCH_OUT_FP16, "cch_gmm_i8_dequant: out_dtype %d", out_dtype);
     CCH_REQUIRE(trans_b == 0 || trans_b == 1, "cch_gmm_i8_dequant: trans_b %d", trans_b);
-    CCH_REQUIRE(num_experts >= 1 && num_experts <= 65535, "cch_gmm_i8_dequant: num_experts=%lld", (long long)num_experts);
+    CCH_REQUIRE(num_experts >= 1 && num_experts <= MAX_GROUPS, "cch_gmm_i8_dequant: num_experts=%lld outside 1..%d", (long long)num_experts, MAX_GROUPS);
     if (t == 0 || n == 0) return CCH_OK;
     CCH_REQUIRE(out && per_tok && per_ch && group_sizes && (k == 0 || (x && w)), "cch_gmm_i8_dequant: null pointer");
     GemmProblem p{};
@@ -178,7 +191,7 @@ static int mx_problem(const char *who, GemmProblem &p, const void *a, const void
     if (rc) return rc;
     CCH_REQUIRE(trans_b == 0 || trans_b == 1, "%s: trans_b %d", who, trans_b);
     CCH_REQUIRE(fmt == CCH_FMT_E4M3 || fmt == CCH_FMT_E5M2 || fmt == CCH_FMT_E2M1, "%s: unknown format %d", who, fmt);
-    CCH_REQUIRE(num_experts >= 1 && num_experts <= 65535, "%s: num_experts=%lld", who, (long long)num_experts);
+    CCH_REQUIRE(num_experts >= 1 && num_experts <= MAX_GROUPS, "%s: num_experts=%lld outside 1..%d", who, (long long)num_experts, MAX_GROUPS);
     CCH_REQUIRE(t == 0 || n == 0 || (a && sa && b && sb && out) || k == 0, "%s: null pointer", who);
     const bool fp4 = fmt == CCH_FMT_E2M1;
     CCH_REQUIRE(!fp4 || (k % 2 == 0 && n % 2 == 0), "%s: FP4 needs even k and n", who);

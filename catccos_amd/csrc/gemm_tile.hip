@@ -773,27 +773,30 @@ static int launch_tile_t(const GemmProblem &p, hipStream_t stream)
     return launch_status("gemm_tile_kernel");
 }
 
-// True when the tiled kernels take this problem; otherwise the caller uses the generic path.
-bool gemm_tile_supports(const GemmProblem &p, int kind, int epi)
+// nullptr when the tiled kernels take this problem; otherwise the precondition that failed (the
+// caller then uses the generic path or reports it).
+const char *gemm_tile_unsupported(const GemmProblem &p, int kind, int epi)
 {
     const int epb = kind == KIND_F4 ? 2 : 1;
-    // whole 128-byte K-steps, at least two of them; output rows must take 16-byte stores
-    if (p.K < 2 * BKB * epb || p.K % (BKB * epb) != 0) return false;
-    if (p.n_out % 8 != 0 || !aligned(p.out, 16)) return false;
-    if ((int64_t)BM * p.n_out * 2 >= ((int64_t)1 << 31)) return false;
+    if (p.K < 2 * BKB * epb || p.K % (BKB * epb) != 0) return "K must be a whole number of 128-byte steps, at least two";
+    if (p.n_out % 8 != 0 || !aligned(p.out, 16)) return "output rows must take 16-byte stores (n_out % 8 == 0, out 16-byte aligned)";
+    if ((int64_t)BM * p.n_out * 2 >= ((int64_t)1 << 31)) return "output row tile beyond 2 GiB";
     // mapped output rows are addressed from the start of `out` with 32-bit offsets
-    if (p.out_row_map && (epi != EPI_PLAIN || p.out_rows * p.n_out * 2 >= ((int64_t)1 << 31) || !aligned(p.out_row_map, 4))) return false;
-    if (p.num_groups > MAX_GROUPS) return false;
-    if ((int64_t)p.N * (p.K / epb) >= ((int64_t)1 << 31)) return false;  // 32-bit source offsets
-    if (!aligned(p.a, 16) || !aligned(p.b, 16) || p.b_stride % 16 != 0) return false;
-    if (kind != KIND_I8 && (!aligned(p.sa, 4) || !aligned(p.sb, 4) || p.sb_stride % 4 != 0 || p.sld % 4 != 0)) return false;
+    if (p.out_row_map && (epi != EPI_PLAIN || p.out_rows * p.n_out * 2 >= ((int64_t)1 << 31) || !aligned(p.out_row_map, 4)))
+        return "mapped output beyond 2 GiB or misaligned row map";
+    if (p.num_groups > MAX_GROUPS) return "more than 256 groups";
+    if ((int64_t)p.N * (p.K / epb) >= ((int64_t)1 << 31)) return "one right-hand operand beyond 2 GiB (32-bit source offsets)";
+    if (!aligned(p.a, 16) || !aligned(p.b, 16) || p.b_stride % 16 != 0) return "operands must be 16-byte aligned";
+    if (kind != KIND_I8 && (!aligned(p.sa, 4) || !aligned(p.sb, 4) || p.sb_stride % 4 != 0 || p.sld % 4 != 0))
+        return "scale arrays must be 4-byte aligned with a row length that is a multiple of 4";
     if (!p.trans_b) {
         // [K, N] operands: 16-byte pieces of a row of B must not straddle its end
         const int cpc = 16 * epb;  // columns per 16-byte piece
-        if ((epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) % cpc != 0 || (epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) < cpc) return false;
-        if (kind != KIND_I8 && p.K % 64 != 0) return false;
+        if ((epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) % cpc != 0 || (epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) < cpc)
+            return "[K,N] operands need N to be a multiple of 16 bytes";
+        if (kind != KIND_I8 && p.K % 64 != 0) return "[K,N] MX operands need K % 64 == 0";
     }
-    return true;
+    return nullptr;
 }
 
 int launch_gemm_tile(const GemmProblem &p, int kind, int epi, hipStream_t stream)

@@ -6,6 +6,9 @@
 // Follows CommBlockMxQuant::ComputeMxQuant (include/catccos/comm/block/comm_block_mx_quant.hpp:414-663)
 // in intent and the generator examples/utils/gen_mx_quant_allgather_data.py:255-313, :385-449
 // bit for bit.
+#include <atomic>
+#include <cstring>
+
 #include "common.h"
 #include "mx_formats.h"
 
@@ -15,14 +18,8 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int QUANT_THREADS = 512;        // large workgroups: the dispatcher places 512 blocks of 256 threads noticeably slower
-#ifndef QUANT_UNROLL_V
-#define QUANT_UNROLL_V 2
-#endif
-#ifndef QUANT_BPC_V
-#define QUANT_BPC_V 8
-#endif
-constexpr int QUANT_UNROLL = QUANT_UNROLL_V;          // wave-steps (64 lanes x 8 elements) per batch
-constexpr int QUANT_BLOCKS_PER_CU = QUANT_BPC_V;      // resident workgroups per CU the grid is sized for
+constexpr int QUANT_UNROLL = 2;           // wave-steps (64 lanes x 8 elements) per batch
+constexpr int QUANT_BLOCKS_PER_CU = 8;    // resident workgroups per CU the grid is sized for
 
 typedef short s16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
@@ -562,6 +559,17 @@ static int launch_scatter(const void *x, const int32_t *dst_idx, void *packed, i
     return CCH_OK;
 }
 
+// Library switch "quant_integer_encoder": the E4M3 round-to-nearest-even quantiser runs through the
+// integer encoder instead of the hardware conversion, so that the two can be compared bit for bit
+// on the device.
+static std::atomic<int> g_quant_integer_encoder{0};
+bool quant_set_option(const char *name, int value)
+{
+    if (strcmp(name, "quant_integer_encoder") != 0) return false;
+    g_quant_integer_encoder.store(value);
+    return true;
+}
+
 }  // namespace cch
 
 extern "C" int cch_mx_quant_scatter_packed(const void *x, const int32_t *expanded_row_idx, void *packed_out, int64_t tokens,
@@ -609,6 +617,8 @@ extern "C" int cch_mx_quant_rows(const void *x, void *payload, void *scales, int
     const bool lut = rounding == CCH_ROUND_LUT;
     switch (fmt) {
         case CCH_FMT_E4M3:
+            if (!lut && g_quant_integer_encoder.load())   // cross-check of the hardware conversion on the device
+                return launch_rows<CCH_FMT_E4M3, CCH_ROUND_RNE, false>(x, payload, scales, m, k, s);
             return lut ? launch_rows<CCH_FMT_E4M3, CCH_ROUND_LUT, false>(x, payload, scales, m, k, s)
                        : launch_rows<CCH_FMT_E4M3, CCH_ROUND_RNE, true>(x, payload, scales, m, k, s);
         case CCH_FMT_E5M2:
@@ -623,17 +633,6 @@ extern "C" int cch_mx_quant_rows(const void *x, void *payload, void *scales, int
         default:
             return fail(CCH_EINVAL, "cch_mx_quant_rows: unknown format %d", fmt);
     }
-}
-
-// Test hook: the same E4M3 round-to-nearest-even quantiser through the integer encoder instead
-// of the hardware cast, so the two can be compared bit for bit on the device.
-extern "C" int cch_mx_quant_rows_e4m3_int(const void *x, void *payload, void *scales, int64_t m, int64_t k,
-                                           void *stream)
-{
-    using namespace cch;
-    if (m <= 0 || k <= 0) return CCH_OK;
-    CCH_REQUIRE(x && payload && scales, "cch_mx_quant_rows_e4m3_int: null pointer");
-    return launch_rows<CCH_FMT_E4M3, CCH_ROUND_RNE, false>(x, payload, scales, m, k, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int cch_mx_quant_b(const void *b, void *payload, void *scales, int64_t k, int64_t n, int fmt, int rounding,

@@ -134,7 +134,9 @@ int cch_gmm_i8_dequant_out(const void *x, const void *w, const int32_t *group_si
  *   rows of x are grouped by expert in expert order, group_sizes[e] rows each (device int32);
  *   c = float(acc) * per_ch[e,n] * per_tok[r];  out[r,j] = silu(c[j]) * c[j+n/2], j < n/2
  *   x int8 [t,k]; w int8 [E,k,n] (trans_b=0) or [E,n,k] (trans_b=1); per_ch fp32 [E,n];
- *   out bf16 [t,n/2].  Rows past sum(group_sizes) are written as zeros. */
+ *   out bf16 [t,n/2].  Rows past sum(group_sizes) are written as zeros.
+ * Every grouped entry point of this library takes 1 <= num_experts <= 256 (the kernels keep the
+ * group table in LDS); more is CCH_EINVAL. */
 int cch_gmm_i8_dequant_swiglu(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok,
                               const float *per_ch, void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k,
                               int trans_b, void *stream);
@@ -264,7 +266,9 @@ int cch_dyn_quant_i8_rows_smooth(const void *x, const int32_t *src_rows, const f
                                  int64_t num_smooth, void *q, float *scale, int64_t rows_in, int64_t t, int64_t k, int topk,
                                  int mode, void *stream);
 
-/* Library switches for tests and benchmarks: "force_generic_gemm" = 1 routes every GEMM entry
+/* Library switches for tests and benchmarks.  They are process-wide (one atomic each, read at
+ * every call): two callers that want different settings at the same time race; set them once, or
+ * from one thread between calls.  "force_generic_gemm" = 1 routes every GEMM entry
  * point through the shape-agnostic one-thread-per-element kernels instead of the tiled MFMA
  * kernels; "require_tiled_gemm" = 1 makes a GEMM entry point return CCH_ENOSUP instead of
  * falling back to them when the tiled kernels do not take the problem; "gemm_tile_order" picks the
@@ -278,7 +282,12 @@ int cch_dyn_quant_i8_rows_smooth(const void *x, const int32_t *src_rows, const f
  * tiles of 256 rows carry the non-temporal hint (its panels are read by that many workgroups and never
  * again, so they need not stay in L2); default 1, 0 switches it off; "gemm_nt_output" = 1 / 0 gives or
  * denies the output stores the same hint, -1 (default) gives it to the MXFP4 kernels, where it measured
- * 3-4 % faster (no difference for the others).  Results do not depend on any of them. */
+ * 3-4 % faster (no difference for the others); "quant_integer_encoder" = 1 runs the E4M3
+ * round-to-nearest-even quantiser through the integer encoder instead of the hardware conversion (an
+ * on-device cross-check; same bytes).  Results do not depend on any of them.
+ * When a GEMM entry point falls back from the tiled MFMA kernels to the one-thread-per-element
+ * kernels (orders of magnitude slower), the call still returns CCH_OK, cch_last_error() names the
+ * precondition that failed, and the first such call of the process prints one line to stderr. */
 int cch_set_option(const char *name, int value);
 
 #ifdef __cplusplus

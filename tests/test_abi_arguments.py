@@ -51,6 +51,11 @@ def test_gemm_arguments():
     rejected(L.cch_gmm_i8_dequant_swiglu(P, P, P, P, P, P, 0, 8, 8, 8, 0, None), "num_experts")
     rejected(L.cch_gmm_i8_dequant_swiglu(P, P, None, P, P, P, 2, 8, 8, 8, 0, None), "null")
     rejected(L.cch_gmm_i8_dequant(P, P, P, P, P, P, 70000, 8, 8, 8, 0, None), "num_experts")
+    # the group table of the kernels holds 256 experts: 257 is an error, not an overrun
+    rejected(L.cch_gmm_i8_dequant(P, P, P, P, P, P, 257, 8, 8, 8, 0, None), "num_experts", "256")
+    rejected(L.cch_gmm_i8_dequant_swiglu(P, P, P, P, P, P, 257, 8, 8, 8, 0, None), "num_experts", "256")
+    rejected(L.cch_mx_gmm(P, P, P, P, P, P, 257, 8, 8, 64, 0, 0, None), "num_experts", "256")
+    rejected(L.cch_mx_gmm_mapped(P, P, P, P, P, P, P, 8, 0, 257, 8, 8, 64, 0, 0, None), "num_experts", "256")
     rejected(L.cch_mx_gemm(P, P, P, P, P, 8, 8, 64, 7, 0, None))           # format
     rejected(L.cch_mx_gemm(P, P, P, P, P, 8, 7, 64, 2, 0, None), "FP4")   # FP4 packs two columns per byte
     rejected(L.cch_mx_gmm(P, P, P, P, None, P, 2, 8, 8, 64, 0, 0, None))   # group sizes missing

@@ -102,12 +102,12 @@ def test_hardware_cast_equals_integer_encoder():
     x = cfg1_input(512, 7168, seed=11)
     xd = to_dev(x)
     p1, s1 = cc.mx_quant(xd, "e4m3")
-    p2 = torch.empty_like(p1)
-    s2 = torch.empty_like(s1)
     L = _abi.lib()
-    L.cch_mx_quant_rows_e4m3_int.argtypes = _abi.PROTOTYPES["cch_mx_quant_rows"][:5] + [_abi._P]
-    assert L.cch_mx_quant_rows_e4m3_int(xd.data_ptr(), p2.data_ptr(), s2.data_ptr(), 512, 7168,
-                                        torch.cuda.current_stream().cuda_stream) == 0
+    assert L.cch_set_option(b"quant_integer_encoder", 1) == 0
+    try:
+        p2, s2 = cc.mx_quant(xd, "e4m3")
+    finally:
+        assert L.cch_set_option(b"quant_integer_encoder", 0) == 0
     torch.cuda.synchronize()
     assert torch.equal(p1, p2) and torch.equal(s1, s2)
 
