@@ -38,6 +38,7 @@ PROTOTYPES = {
     "cch_moe_token_unpermute": [_P, _P, _P, _P, _I64, _I64, _I64, _I, _P],
     "cch_moe_init_routing_workspace_bytes": [_I64, _I],
     "cch_moe_init_routing": [_P, _I64, _I, _P, _P, _P, _I, _P, _I64, _P],
+    "cch_moe_init_routing_noalloc": [_P, _I64, _I, _P, _P, _P, _I, _P],
     "cch_dyn_quant_i8_rows": [_P, _P, _P, _P, _I64, _I64, _I64, _I, _I, _P],
     "cch_dyn_quant_i8_rows_smooth": [_P, _P, _P, _P, _I64, _P, _P, _I64, _I64, _I64, _I, _I, _P],
     "cch_gemm_i8_dequant": [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I, _P],

@@ -9,6 +9,7 @@
 // integers, so the sort is a counting sort in three launches: per-chunk histograms, one scan over
 // (expert, chunk), and a placement pass in which four waves walk their quarters of a chunk in order.
 #include <algorithm>
+#include <atomic>
 
 #include "common.h"
 
@@ -156,6 +157,62 @@ __global__ __launch_bounds__(64 * ROUTE_WAVES) void route_place_kernel(const int
     }
 }
 
+// Checks shared by the two entry points; fills nchunks.
+static int route_check(const char *who, const int32_t *expert_idx, int64_t rows, int num_experts, const int32_t *dst_to_src,
+                       const int32_t *src_to_dst, const int32_t *expert_tokens, int64_t *nchunks)
+{
+    CCH_REQUIRE(rows >= 0 && rows < ((int64_t)1 << 30), "%s: rows=%lld", who, (long long)rows);
+    CCH_REQUIRE(num_experts >= 1 && num_experts <= ROUTE_MAX_EXPERTS, "%s: num_experts=%d outside 1..%d", who, num_experts,
+                ROUTE_MAX_EXPERTS);
+    CCH_REQUIRE(expert_tokens != nullptr, "%s: null expert_tokens", who);
+    *nchunks = std::max<int64_t>((rows + ROUTE_CHUNK - 1) / ROUTE_CHUNK, 1);
+    CCH_REQUIRE(*nchunks * num_experts < ((int64_t)1 << 31), "%s: rows x experts too large", who);
+    CCH_REQUIRE(rows == 0 || (expert_idx && dst_to_src && src_to_dst), "%s: null pointer", who);
+    return CCH_OK;
+}
+
+// The three launches; hist holds nchunks * num_experts entries, every one of which the histogram
+// pass writes before the scan reads it (nothing has to start at zero).
+static int route_launch(const int32_t *expert_idx, int64_t rows, int num_experts, int64_t nchunks, int32_t *dst_to_src,
+                        int32_t *src_to_dst, int32_t *expert_tokens, int cumsum, int32_t *hist, hipStream_t s)
+{
+    hipLaunchKernelGGL(route_histogram_kernel, dim3((unsigned)nchunks), dim3(256), 0, s, expert_idx, (int)rows, num_experts,
+                       (int)nchunks, hist, dst_to_src);
+    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, hist, num_experts, (int)nchunks, expert_tokens, cumsum);
+    int bits = 0;
+    while ((1 << bits) < num_experts) bits++;
+    if (rows > 0)
+        hipLaunchKernelGGL(route_place_kernel, dim3((unsigned)nchunks), dim3(64 * ROUTE_WAVES), 0, s, expert_idx, (int)rows,
+                           num_experts, (int)nchunks, bits, hist, dst_to_src, src_to_dst);
+    return launch_status("route kernels");
+}
+
+// Histogram area of cch_moe_init_routing_noalloc: part of the library's device image, so every GPU
+// the library runs on holds its own copy (1 MiB) from load to process end.  The name is only a
+// host-side handle; the device address is looked up once per device and kept in g_scratch_ptr.
+constexpr int64_t ROUTE_STATIC_ENTRIES = CCH_ROUTING_NOALLOC_MAX_ENTRIES;
+static __device__ __align__(256) int32_t scratch[ROUTE_STATIC_ENTRIES];
+constexpr int ROUTE_MAX_DEVICES = 64;
+static std::atomic<int32_t *> g_scratch_ptr[ROUTE_MAX_DEVICES];
+
+// Device address of `scratch` on the current device (looked up on first use, or by cch_init).
+int routing_scratch_setup(int32_t **out)
+{
+    int dev = 0;
+    CCH_HIP(hipGetDevice(&dev));
+    CCH_REQUIRE(dev >= 0 && dev < ROUTE_MAX_DEVICES, "routing scratch: device %d outside 0..%d", dev, ROUTE_MAX_DEVICES - 1);
+    int32_t *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        void *sym = nullptr;
+        CCH_HIP(hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)));
+        if (sym == nullptr) return fail(CCH_EHIP, "routing scratch: hipGetSymbolAddress gave a null address on device %d", dev);
+        ptr = static_cast<int32_t *>(sym);
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // two threads racing here store the same address
+    }
+    if (out) *out = ptr;
+    return CCH_OK;
+}
+
 }  // namespace cch
 
 extern "C" int64_t cch_moe_init_routing_workspace_bytes(int64_t rows, int num_experts)
@@ -170,25 +227,31 @@ extern "C" int cch_moe_init_routing(const int32_t *expert_idx, int64_t rows, int
                                     int64_t workspace_bytes, void *stream)
 {
     using namespace cch;
-    CCH_REQUIRE(rows >= 0 && rows < ((int64_t)1 << 30), "cch_moe_init_routing: rows=%lld", (long long)rows);
-    CCH_REQUIRE(num_experts >= 1 && num_experts <= ROUTE_MAX_EXPERTS, "cch_moe_init_routing: num_experts=%d outside 1..%d",
-                num_experts, ROUTE_MAX_EXPERTS);
-    CCH_REQUIRE(expert_tokens != nullptr, "cch_moe_init_routing: null expert_tokens");
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const int64_t nchunks = std::max<int64_t>((rows + ROUTE_CHUNK - 1) / ROUTE_CHUNK, 1);
-    CCH_REQUIRE(nchunks * num_experts < ((int64_t)1 << 31), "cch_moe_init_routing: rows x experts too large");
+    int64_t nchunks = 0;
+    int rc = route_check("cch_moe_init_routing", expert_idx, rows, num_experts, dst_to_src, src_to_dst, expert_tokens, &nchunks);
+    if (rc) return rc;
     CCH_REQUIRE(workspace != nullptr && workspace_bytes >= cch_moe_init_routing_workspace_bytes(rows, num_experts),
                 "cch_moe_init_routing: workspace of %lld bytes, need %lld", (long long)workspace_bytes,
                 (long long)cch_moe_init_routing_workspace_bytes(rows, num_experts));
-    CCH_REQUIRE(rows == 0 || (expert_idx && dst_to_src && src_to_dst), "cch_moe_init_routing: null pointer");
-    int32_t *hist = static_cast<int32_t *>(workspace);
-    hipLaunchKernelGGL(route_histogram_kernel, dim3((unsigned)nchunks), dim3(256), 0, s, expert_idx, (int)rows, num_experts,
-                       (int)nchunks, hist, dst_to_src);
-    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, hist, num_experts, (int)nchunks, expert_tokens, cumsum);
-    int bits = 0;
-    while ((1 << bits) < num_experts) bits++;
-    if (rows > 0)
-        hipLaunchKernelGGL(route_place_kernel, dim3((unsigned)nchunks), dim3(64 * ROUTE_WAVES), 0, s, expert_idx, (int)rows,
-                           num_experts, (int)nchunks, bits, hist, dst_to_src, src_to_dst);
-    return launch_status("route kernels");
+    return route_launch(expert_idx, rows, num_experts, nchunks, dst_to_src, src_to_dst, expert_tokens, cumsum,
+                        static_cast<int32_t *>(workspace), static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cch_moe_init_routing_noalloc(const int32_t *expert_idx, int64_t rows, int num_experts, int32_t *dst_to_src,
+                                            int32_t *src_to_dst, int32_t *expert_tokens, int cumsum, void *stream)
+{
+    using namespace cch;
+    int64_t nchunks = 0;
+    int rc = route_check("cch_moe_init_routing_noalloc", expert_idx, rows, num_experts, dst_to_src, src_to_dst, expert_tokens,
+                         &nchunks);
+    if (rc) return rc;
+    CCH_REQUIRE(nchunks * num_experts <= ROUTE_STATIC_ENTRIES,
+                "cch_moe_init_routing_noalloc: ceil(rows/%d) * num_experts = %lld exceeds the built-in area of %lld entries; "
+                "use cch_moe_init_routing with a workspace", ROUTE_CHUNK, (long long)(nchunks * num_experts),
+                (long long)ROUTE_STATIC_ENTRIES);
+    int32_t *hist = nullptr;
+    rc = routing_scratch_setup(&hist);
+    if (rc) return rc;
+    return route_launch(expert_idx, rows, num_experts, nchunks, dst_to_src, src_to_dst, expert_tokens, cumsum, hist,
+                        static_cast<hipStream_t>(stream));
 }

@@ -4,6 +4,8 @@
 #include "common.h"
 
 namespace cch {
+int routing_scratch_setup(int32_t **out);   // routing.hip: device address of its built-in histogram area
+
 static thread_local char g_err[512] = "";
 
 int fail(int code, const char *fmt, ...)
@@ -32,7 +34,8 @@ int cch_init(int device)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(CCH_ENODEV, "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
     CCH_HIP(hipSetDevice(device));
-    return CCH_OK;
+    // set-up for cch_moe_init_routing_noalloc, so that its calls look nothing up
+    return cch::routing_scratch_setup(nullptr);
 }
 
 int cch_device_info(char *name, size_t name_len, int *compute_units, int *clock_mhz, uint64_t *hbm_bytes)

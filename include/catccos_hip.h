@@ -240,6 +240,21 @@ int64_t cch_moe_init_routing_workspace_bytes(int64_t rows, int num_experts);
 int cch_moe_init_routing(const int32_t *expert_idx, int64_t rows, int num_experts, int32_t *dst_to_src, int32_t *src_to_dst,
                          int32_t *expert_tokens, int cumsum, void *workspace, int64_t workspace_bytes, void *stream);
 
+/* cch_moe_init_routing for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and results minus the workspace: the histogram area is a 1 MiB array
+ * inside the library's device image (one copy per GPU, held until the process ends), whose
+ * address is looked up once per device by cch_init or by the first call on that device.  The call
+ * itself allocates and frees nothing.
+ *   limit   ceil(rows / 1024) * num_experts <= CCH_ROUTING_NOALLOC_MAX_ENTRIES (e.g. 262144 rows
+ *           over 1024 experts, or 8 Mi rows over 32); larger requests return CCH_EINVAL.
+ *   sharing every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
+ *           streams, two threads) race; calls in stream order do not.  Nothing in the array has to
+ *           be cleared between calls (each call writes every entry it later reads). */
+#define CCH_ROUTING_NOALLOC_MAX_ENTRIES 262144
+int cch_moe_init_routing_noalloc(const int32_t *expert_idx, int64_t rows, int num_experts, int32_t *dst_to_src,
+                                 int32_t *src_to_dst, int32_t *expert_tokens, int cumsum, void *stream);
+
 /* ---- Per-token dynamic int8 quantisation with row gather (feeds config 4) ----
  * Replaces MoeV2GatherDynamicQuant (examples/aux_ops/moe_init_routing_quant_v2/
  * moe_v2_gather_dynamic_quant.h:117-150 Compute, :213-250 the gather loop).
