@@ -1,27 +1,38 @@
-// Tiled MFMA GEMM family for gfx950 (B stored K-contiguous, i.e. trans_b = 1):
+// Tiled MFMA GEMM family for gfx950:
 //   int8 x int8 -> int32   v_mfma_i32_32x32x32_i8          + dequant / dequant+SwiGLU epilogue
 //   MXFP8 / MXFP4          v_mfma_scale_f32_32x32x64_f8f6f4 with per-lane E8M0 scale operands
 //
 // One persistent workgroup (8 waves) per CU walks a global list of 256x256 output tiles built
 // from the prefix sums of the group sizes (a dense problem is one group).
-//   * K advances in steps of 128 bytes per row, the size of an L2 line: direct-to-LDS loads
-//     that cover whole lines reach about 1.5x the L2 throughput of half-line requests.  The A
-//     and B panels of a step (256 rows x 128 B each) go global -> LDS without a VGPR round
-//     trip into a ring of two stages.  A stage is read for the last time about 5/8 through
-//     its step; the requests that refill it (two steps ahead of use) follow the step's one
-//     barrier and are threaded between the remaining MFMAs.
+//   * K advances in steps of 128 bytes per row, the size of an L2 line.  The A and B panels of a
+//     step (256 rows x 128 B each) go global -> LDS without a VGPR round trip (buffer_load ... lds)
+//     into a ring of two stages.
+//   * The eight waves form two groups of four, one wave of each group per SIMD: waves 0-3 own
+//     the upper 128 rows of the tile, waves 4-7 the lower 128, each wave 128 x 64 outputs.  A
+//     wave alternates between a memory slot (LDS fragment reads, global -> LDS requests) and a
+//     matrix slot (MFMAs only), the slots are separated by workgroup barriers, and the second
+//     group runs one slot behind the first: while one wave of a SIMD issues matrix instructions
+//     its neighbour fetches, and the next slot they swap.  A K-step is four slots per wave:
+//       L0  read all B fragments of the step and the A fragments of row blocks 0-1;
+//           request the A rows of row blocks 2-3 of step k+1
+//       C0  MFMAs of row blocks 0-1 (both 64-byte halves of the step)
+//       L1  read the A fragments of row blocks 2-3 (into the same registers);
+//           request B and the A rows of row blocks 0-1 of step k+2 - their place in the ring is the
+//           stage being computed, whose B panel and first A rows nobody reads any more
+//       C1  MFMAs of row blocks 2-3
+//     so a request has five slots (1.25 steps) to land before the barrier that publishes it.
 //   * MX scales travel 16 bytes per row at a time (4 MXFP8 steps, 2 MXFP4 steps) into a pair of
 //     scale buffers: a per-step 4-byte fetch touches one L2 line per lane and costs as many
 //     line requests as the whole data panel.
-//   * Each wave owns 128 x 64 outputs as 4 x 2 MFMA tiles of 32 x 32 and reads its fragments
-//     with 16-byte LDS reads from an XOR-swizzled panel layout (no bank conflicts).  Fragment
-//     registers are refilled as soon as the MFMAs that read them have been issued, so LDS
-//     latency hides behind the other MFMAs of the step.
-//   * The K loop is a single basic block without compiler-visible memory loads; the last two
-//     steps of a tile are peeled and request the next tile's first two steps, with empty
-//     buffer descriptors when there is no next tile, so they are branch-free as well.
-//   * Epilogues (dequant, SwiGLU, bf16 rounding) run on the accumulators; results pass through
-//     a wave-private 1 KiB LDS buffer so that every lane stores 16 contiguous bytes.
+//   * The K loop has no compiler-visible global loads (the requests are inline assembly tracked by
+//     explicit vmcnt waits with fixed counts; a request that is not due is issued against an empty
+//     buffer descriptor instead of being skipped); the last two steps of a tile are peeled and
+//     request the next tile's first two steps.  K needs no particular length: the last step is
+//     cut off per row (lanes past the row end fetch nothing), scale bytes past it are masked.
+//   * Epilogues (dequant, SwiGLU, bf16 rounding) run on the accumulators between a wave's last
+//     matrix slot of a tile and its first memory slot of the next; both groups do it in the same
+//     slot.  Results pass through a wave-private 1 KiB LDS buffer so that every lane stores 16
+//     contiguous bytes.
 //
 // Stands in for Catlass::Gemm::Block::BlockMmadTla<MmadMx<...>> as instantiated in
 // examples/ascend950_fp4_mx_alltoallv_grouped_matmul/ascend950_fp4_mx_alltoallv_grouped_matmul_device.h:59-71,
@@ -70,8 +81,9 @@ constexpr int EPI_OFF = SCALE_OFF + 2 * SCALE_BUF;           // per wave: 1 KiB 
 constexpr int EPI_WAVE = 1024;
 constexpr int PARAM_OFF = EPI_OFF + NWAVES * EPI_WAVE;       // per tile parity: 256 per_tok + 256 per_ch floats
 constexpr int PARAM_SET = 2048;
-constexpr int RING_OFF = PARAM_OFF + 2 * PARAM_SET;          // NSTAGE stages of an A panel and a B panel
-constexpr int LDS_BYTES = RING_OFF + NSTAGE * STAGE_BYTES;   // 156 KiB of the CU's 160 KiB
+constexpr int SINK_OFF = PARAM_OFF + 2 * PARAM_SET;          // 1 KiB where requests that are not due land (zeros)
+constexpr int RING_OFF = SINK_OFF + 1024;                    // NSTAGE stages of an A panel and a B panel
+constexpr int LDS_BYTES = RING_OFF + NSTAGE * STAGE_BYTES;   // 157 KiB of the CU's 160 KiB
 
 template <int KIND> struct KindTraits;
 template <> struct KindTraits<KIND_I8> { static constexpr int ELEMS_PER_BYTE = 1, SCALE_DW = 0; using Acc = v16i; };
@@ -95,19 +107,40 @@ template <int N, class F> __device__ __forceinline__ void static_for(F &&f)
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
-// s_waitcnt vmcnt(n) lgkmcnt(0) on gfx9: vmcnt in bits [3:0] and [15:14], expcnt [6:4], lgkmcnt [11:8].
+// s_waitcnt on gfx9: vmcnt in bits [3:0] and [15:14], expcnt [6:4], lgkmcnt [11:8].
 #define CCH_WAIT_VM_LGKM0(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4))
+// vmcnt only (lgkmcnt left at its maximum of 15)
+#define CCH_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 // s_waitcnt lgkmcnt(0) only (vmcnt left at its maximum of 63)
 #define CCH_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
+
+// Workgroup barrier that the compiler moves no memory access across (the intrinsic alone is not a
+// memory barrier to the optimiser) and that the instruction scheduler leaves where it is.
+#ifndef CCH_PRIO_C
+#define CCH_PRIO_C 1
+#define CCH_PRIO_L 0
+#endif
+#ifdef CCH_V_NOPRIO
+#define CCH_SETPRIO(n)
+#else
+#define CCH_SETPRIO(n) __builtin_amdgcn_s_setprio(n)
+#endif
+#define CCH_BARRIER()                                  \
+    do {                                               \
+        __builtin_amdgcn_sched_barrier(0);             \
+        asm volatile("s_barrier" ::: "memory");        \
+        __builtin_amdgcn_sched_barrier(0);             \
+    } while (0)
 
 // 16 / 4 bytes per lane, global -> LDS without passing through registers, as raw buffer loads:
 // the descriptor holds the wave-uniform base, `voff` is the per-lane byte offset, `soff` a
 // wave-uniform byte offset (the K position).  Lane l of the wave lands at LDS address
-// lds_addr + size*l.  Issued as inline assembly on purpose: the compiler's wait-count pass
+// lds_addr + size*l.  A lane whose offset lies at or past the descriptor's size fetches nothing
+// and receives zeros.  Issued as inline assembly on purpose: the compiler's wait-count pass
 // would otherwise drain every outstanding direct-to-LDS load before each LDS read;
 // completion is tracked by the explicit vmcnt waits instead.
 typedef int Rsrc __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ Rsrc make_rsrc(const void *base, uint32_t bytes = 0x7FFFFFFFu)
+__device__ __forceinline__ Rsrc make_rsrc(const void *base, uint32_t bytes)
 {
     const uint64_t b = reinterpret_cast<uint64_t>(base);
     Rsrc rs;
@@ -138,34 +171,6 @@ __device__ __forceinline__ void load16_to_lds(Rsrc rs, uint32_t voff, uint32_t s
                  : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
                  : "memory", "m0");
 }
-// The same load with the non-temporal hint: the line is not kept in L2 after use (weight panels of
-// experts so small that no other workgroup reads them again).
-__device__ __forceinline__ void load16_to_lds_nt(Rsrc rs, uint32_t voff, uint32_t soff, uint32_t lds_addr)
-{
-    rs = scalar_rsrc(rs);
-    soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
-    lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
-                 :
-                 : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
-                 : "memory", "m0");
-}
-// The same 16-byte load, performed only when `enable` (wave-uniform) is non-zero, without a
-// branch: the load is issued with an empty EXEC mask otherwise.  Keeps the K loop one basic
-// block, which the register allocator handles far better than a loop with a diamond in it.
-__device__ __forceinline__ void load16_to_lds_if(int enable, Rsrc rs, uint32_t voff, uint32_t soff, uint32_t lds_addr)
-{
-    rs = scalar_rsrc(rs);
-    soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
-    lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
-    enable = __builtin_amdgcn_readfirstlane(enable);
-    uint64_t saved;
-    asm volatile("s_mov_b64 %0, exec\n\ts_cmp_lg_u32 %1, 0\n\ts_cselect_b64 exec, %0, 0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\t"
-                 "buffer_load_dwordx4 %3, %4, %5 offen lds\n\ts_mov_b64 exec, %0"
-                 : "=&s"(saved)
-                 : "s"(enable), "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
-                 : "memory", "m0", "scc");
-}
 __device__ __forceinline__ void load4_to_lds(Rsrc rs, uint32_t voff, uint32_t soff, uint32_t lds_addr)
 {
     rs = scalar_rsrc(rs);
@@ -184,13 +189,24 @@ __device__ __forceinline__ uint32_t lds_read4(uint32_t off) { return *reinterpre
 // c ^ ((row >> 1) & 7), which spreads 16 consecutive rows over all 64 banks for 16-byte reads.
 __device__ __forceinline__ uint32_t swizzle_of_row(int row) { return (uint32_t)((row >> 1) & 7); }
 
+#ifdef CCH_PROF
+// Instrumented build: cycles per wave spent in the waits and barriers of the K loop.
+__device__ uint64_t cch_prof[256 * 8 * 8];
+#define PROF_BEGIN(t) const uint64_t t = __builtin_readcyclecounter()
+#define PROF_END(t, acc) acc += __builtin_readcyclecounter() - t
+#else
+#define PROF_BEGIN(t)
+#define PROF_END(t, acc)
+#endif
+
+constexpr uint32_t NO_FETCH = 0xFFFFFFF0u;   // a lane offset past every descriptor: the lane fetches nothing
+
 // What one tile needs, all wave-uniform except the per-lane source offsets.
 struct TileCtx {
     int valid, e, m0, m_end, j0;
-    uint32_t lim;                       // descriptor size: 0 for a tile past the end, whose requests then fetch nothing
-    Rsrc rs_a, rs_b, rs_sc;             // buffer descriptors: A rows from m0, B of the expert, scales
-    uint32_t off_a[NJ], off_b[NJ];      // per lane: source row * pitch + chunk * 16
-    uint32_t off_sc;                    // per lane: scale row * sld (A rows for waves 0-3, B columns for 4-7)
+    Rsrc rs_a, rs_b, rs_sc;             // buffer descriptors: A rows from m0, B of the expert from the tile's first column, scales
+    uint32_t off_sc;                    // per lane: byte offset of its scale row (A rows for waves 0-3, B columns for 4-7), rounded down to 4
+    uint32_t sel_a, sel_b;              // per lane: byte selectors that bring this lane's two scale bytes of a step to bytes 0 and 2
 };
 
 // TB = 1: B is stored [N, K] (K contiguous) and its panel is staged like A's.  TB = 0 (int8 and
@@ -200,7 +216,8 @@ struct TileCtx {
 // row segments of 8 bytes and returns to lane j byte (j & 7) of segments (j >> 3), (j >> 3) + 2,
 // ..., (j >> 3) + 14.  Lane i of a group therefore addresses K-row i/2 at columns 8*(i & 1) ..
 // +7, and lane j receives 8 consecutive K bytes of column j.
-template <int KIND, int EPI, int FMT, int TB>
+// UA = 1: MX scale rows (sld bytes each) do not all start on 4-byte boundaries (sld % 4 == 2).
+template <int KIND, int EPI, int FMT, int TB, int UA>
 __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 {
     using KT = KindTraits<KIND>;
@@ -210,7 +227,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;   // output columns per tile
     constexpr int WN_OUT = SWIGLU ? WN / 2 : WN;   // output columns per wave
     constexpr int SCALE_DW = KT::SCALE_DW;         // scale dwords per row per step
-    constexpr int NV = 2 * NJ;                     // direct-to-LDS instructions per wave per step
     // MX scales travel 16 bytes per row at a time: one request per wave covers SPG steps
     constexpr int SPG = SCALE_DW > 0 ? 4 / SCALE_DW : 1;
     constexpr int CBSZ = FMT == CCH_FMT_E2M1 ? 4 : (FMT == CCH_FMT_E5M2 ? 1 : 0);
@@ -218,6 +234,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     constexpr int CPR = ROWB / 16;                 // 16-byte chunks per staged row
     constexpr int PASS_ROWS = 64 / CPR;            // rows staged per pass: 1 KiB, one read-back instruction
     constexpr int NPASS = 32 / PASS_ROWS;          // passes per 32-row MFMA tile
+    constexpr int NSTORES = MT * NPASS;            // output stores per wave and tile (always issued; out-of-range lanes dropped)
+    constexpr int NPARAM = EPI != EPI_PLAIN ? 2 : 1;   // epilogue parameter requests per wave and tile
+    // requests per wave in the four slots of a step
+    constexpr int NL0 = 2;                          // A rows of row blocks 2-3 of the next step
+    constexpr int NC0 = 2;                          // A rows of row blocks 0-1 of the step after the next
+    constexpr int NL1 = NJ / 2 + (MX ? 1 : 0);      // half of the B panel share, scales (or a request that fetches nothing)
+    constexpr int NC1 = NJ / 2;                     // the other half of the B panel share
 
     __shared__ GroupTable tab;
     if (threadIdx.x == 0) build_group_table(tab, p.group_sizes, p.num_groups, p.T, BM);
@@ -231,7 +254,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     const int r = lane & 31, g = lane >> 5;
 
     const int lda = p.K / KT::ELEMS_PER_BYTE;  // bytes per row of A and of B (K-contiguous)
-    const int ksteps = lda / BKB;
+    const int ksteps = max((lda + BKB - 1) / BKB, 2);   // a one-step K runs a second, empty step: the pipeline has two stages
     const int n_tiles = (p.n_out + BN_OUT - 1) / BN_OUT;
     const int total_tiles = uniform(tab.tile_start[p.num_groups]) * n_tiles;  // rows past the groups are not ours
 
@@ -242,7 +265,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     // B scales: TB = 1 like A's, 16 bytes per column; TB = 0 eight 512-byte rows per group,
     // [K64 block][column][2]
     const uint32_t rd_sb = TB ? 4096u + (uint32_t)(wn * WN + r) * 16 : 4096u + (((uint32_t)(wn * WN + r) * 2) & ~3u);
-    const uint32_t sb_sel = (r & 1) ? 0x07060302u : 0x05040100u;   // TB = 0: which half of the dwords holds this column
     // TB = 0 fragment reads: lane (q = lane / 16, i = lane % 16) addresses K-row 16*(q/2) + i/2 of
     // the substep part and the 8-byte half (i & 1) of 16-byte chunk wn*4 + j*2 + (q & 1), whose
     // position in the row is swizzled by twice the row's low bits (i / 2): the 32 lanes of one pass
@@ -262,6 +284,10 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                                 : (uint32_t)PANEL_BYTES + (uint32_t)(16 * (tq >> 1) + (ti >> 1)) * 256u +
                                       ((uint32_t)((wn * 4 + (tq & 1)) ^ ((ti >> 1) << 1)) << 4) + (uint32_t)(ti & 1) * 8u;
     const int ldb = TB ? lda : p.N / EPB;   // bytes between consecutive rows of B as stored
+    const uint32_t b_bytes = (uint32_t)min((int64_t)p.N * lda, (int64_t)0x7FFFFFFF);   // one right-hand operand
+    // Byte position inside its 128-byte row piece that this lane fetches in the K-contiguous panels
+    // (even / odd request of a wave), for cutting the last step off at the row end.
+    const uint32_t cb0 = (uint32_t)((lane & 7) ^ (lane >> 4)) << 4, cb1 = cb0 ^ 64u;
     // Rows that belong to no group are written as zeros (the reference's golden pads them,
     // examples/utils/gen_data_fp4_mx_alltoallv_gmm.py:788-790): all workgroups share the range,
     // 16 bytes per thread and pass; usually it is empty.
@@ -282,6 +308,46 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     }
     nwg = uniform(nwg);
 
+    // Per-lane source offsets of the panel requests, relative to the descriptors' starts: the same
+    // for every tile, and the same for every second request of a wave up to a wave-uniform term.
+    //   A: request q = 2*h + jj fills rows wm*128 + h*64 + (wn*2 + jj)*8 .. +7 of the panel (this wave
+    //   fetches rows of the half of the tile that its own group computes); lane l lands at row l/8,
+    //   chunk position l%8 and must therefore fetch chunk (l%8) ^ swizzle(row).
+    //   B, TB = 1: request j fills rows (wave*NJ + j)*8 .. +7 in the same way; with SwiGLU tile row
+    //   wn*64 + h*32 + c is the gate (h = 0) or up (h = 1) column j0 + wn*32 + c.
+    //   B, TB = 0: request j fills K-rows (wave*NJ + j)*BRPI .. of the panel, BROW bytes each; lane l
+    //   lands at row l/BCPR, chunk position l%BCPR and fetches tile chunk (l%BCPR) ^ swizzle, 16 bytes
+    //   of columns; with SwiGLU chunk tc holds gate or up ((tc >> 1) & 1) columns j0 + (tc >> 2)*32 +
+    //   (tc & 1)*16 .. +15.
+    // The swizzle of a request's rows depends on the request's parity only, so requests q and q + 2
+    // differ by a fixed number of rows: offset(q) = par[q & 1] + (q >> 1) * pair_step.
+    uint32_t a_par[2], b_par[2];
+#pragma unroll
+    for (int x = 0; x < 2; x++) {
+        const int row = wm * WM + (wn * 2 + x) * 8 + (lane >> 3);
+        a_par[x] = (uint32_t)row * (uint32_t)lda + ((uint32_t)(lane & 7) ^ swizzle_of_row(row)) * 16u;
+        if (TB) {
+            const int brow = (wave * NJ + x) * 8 + (lane >> 3);
+            const uint32_t chunk = ((uint32_t)(lane & 7) ^ swizzle_of_row(brow)) * 16u;
+            const int col = SWIGLU ? ((brow >> 5) & 1) * p.n_out + (brow >> 6) * 32 + (brow & 31) : brow;   // relative to j0
+            b_par[x] = (uint32_t)col * (uint32_t)lda + chunk;
+        } else {
+            const int kr = (wave * NJ + x) * BRPI + lane / BCPR;
+            const int tc = (lane % BCPR) ^ (FP4K ? (kr >> 1) & 7 : (kr & 7) << 1);
+            const int col = SWIGLU ? ((tc >> 1) & 1) * p.n_out + (tc >> 2) * 32 + (tc & 1) * 16 : tc * 16 * EPB;   // relative to j0
+            b_par[x] = (uint32_t)kr * (uint32_t)ldb + (uint32_t)(col / EPB);
+        }
+    }
+    uint32_t off_a[NJ], off_b[NJ];
+    const uint32_t a_pair_step = 64u * (uint32_t)lda;                                   // rows between requests q and q + 2
+    const uint32_t b_pair_step = TB ? 16u * (uint32_t)lda : 2u * BRPI * (uint32_t)ldb;
+    for (int q = 0; q < NJ; q++) { off_a[q] = a_par[q & 1] + (uint32_t)(q >> 1) * a_pair_step; off_b[q] = b_par[q & 1] + (uint32_t)(q >> 1) * b_pair_step; }
+
+    const int nk_tile = ksteps;
+#ifdef CCH_PROF
+    uint64_t pf_wa = 0, pf_wb = 0, pf_b0 = 0, pf_b1 = 0, pf_b2 = 0, pf_b3 = 0, pf_l0 = 0;
+    const uint64_t pf_start = __builtin_readcyclecounter();
+#endif
     int gi = 0;           // scale groups requested so far; group n lives in scale buffer n & 1
     int gbase = 0;        // value of gi when the current tile's group 0 was requested
 
@@ -290,7 +356,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // can then be issued unconditionally (they read nothing and write zeros into LDS areas
         // that are never used), which keeps the peeled steps free of branches.
         c.valid = t < total_tiles;
-        c.lim = c.valid ? 0x7FFFFFFFu : 0u;
+        const uint32_t lim = c.valid ? 0x7FFFFFFFu : 0u;
         t = max(min(t, total_tiles - 1), 0);
         if (p.tile_order == 1 && (nwg & 7) == 0 && t < total_tiles - total_tiles % nwg) {
             // Workgroup w of a round runs on XCD w % 8: give each XCD a run of gridDim.x / 8
@@ -298,145 +364,173 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             // fetches one or two A panels and the B panels of one or two experts per round.
             const int G = nwg, j = t / G, w = t - j * G;
             t = j * G + (w & 7) * (G >> 3) + (w >> 3);
+        } else if (p.tile_order == 2 && nwg == 256 && n_tiles == 16 && t < total_tiles - total_tiles % nwg) {
+            // Each XCD takes a block of 4 row tiles x 8 column tiles of the round: a weight panel then
+            // has up to four users in one L2 and a token panel eight.
+            const int G = nwg, j = t / G, w = t - j * G, x = w & 7, i = w >> 3;
+            t = j * G + ((x >> 1) * 4 + (i >> 3)) * n_tiles + (x & 1) * 8 + (i & 7);
         }
         const int tr = t / n_tiles, nt = t - tr * n_tiles;
         c.e = uniform(find_group(tab, p.num_groups, tr));
         c.m0 = uniform(tab.row_start[c.e] + (tr - tab.tile_start[c.e]) * BM);
         c.m_end = uniform(tab.row_start[c.e + 1]);
         c.j0 = nt * BN_OUT;
-        // A's descriptor ends with the group: requests for tile rows past it are dropped by the
-        // bounds check (LDS receives zeros), and their products land in accumulators that are
-        // never stored.
-        c.rs_a = make_rsrc(p.a + (size_t)c.m0 * lda, min((uint32_t)min(c.m_end - c.m0, BM) * (uint32_t)lda, c.lim));
-        c.rs_b = make_rsrc(p.b + (size_t)c.e * p.b_stride, c.lim);
-        // Instruction j of this wave fills rows (wave*NJ + j)*8 .. +7 of a panel; lane l lands at
-        // row l/8, chunk position l%8 and must therefore fetch chunk (l%8) ^ swizzle(row).
-#pragma unroll
-        for (int j = 0; j < NJ; j++) {
-            const int row = (wave * NJ + j) * 8 + (lane >> 3);
-            const uint32_t chunk = ((uint32_t)(lane & 7) ^ swizzle_of_row(row)) * 16u;
-            c.off_a[j] = (uint32_t)row * (uint32_t)lda + chunk;
-            if (TB) {
-                int col;  // B row (= logical column) feeding tile row `row`
-                if (SWIGLU) {
-                    // tile row = wn*64 + h*32 + c: h = 0 gate, 1 up; output column j0 + wn*32 + c
-                    col = ((row >> 5) & 1) * p.n_out + min(c.j0 + (row >> 6) * 32 + (row & 31), p.n_out - 1);
-                } else {
-                    col = min(c.j0 + row, p.N - 1);
-                }
-                c.off_b[j] = (uint32_t)col * (uint32_t)lda + chunk;
-            } else {
-                // Instruction j fills K-rows (wave*NJ + j)*4 .. +3 of the panel, 256 bytes each;
-                // lane l lands at row l/16, chunk position l%16 and fetches tile chunk
-                // (l%16) ^ 2*(row & 7): 16 tile columns, clamped to stay inside the row of B.
-                const int kr = (wave * NJ + j) * BRPI + lane / BCPR;
-                const int tc = (lane % BCPR) ^ (FP4K ? (kr >> 1) & 7 : (kr & 7) << 1);
-                constexpr int CPC = 16 * EPB;  // columns per chunk
-                int col;
-                if (SWIGLU) col = ((tc >> 1) & 1) * p.n_out + min(c.j0 + (tc >> 2) * 32 + (tc & 1) * 16, p.n_out - 16);
-                else col = min(c.j0 + tc * CPC, p.N - CPC);
-                c.off_b[j] = (uint32_t)kr * (uint32_t)ldb + (uint32_t)(col / EPB);
-            }
-        }
+        // A's descriptor starts at the tile's first row and ends with the group: requests for tile
+        // rows past it are dropped by the bounds check (LDS receives zeros), and their products land
+        // in accumulators that are never stored.  B's descriptor starts at the tile's first column
+        // (TB = 1: row j0 of the expert's [N, K]; TB = 0: column j0 of its [K, N]) and ends with the
+        // expert's operand: what a request finds past the tile's last valid column - other columns'
+        // or the next expert's bytes, or nothing past the end - feeds columns that are never stored.
+        c.rs_a = make_rsrc(p.a + (size_t)c.m0 * lda, min((uint32_t)min(c.m_end - c.m0, BM) * (uint32_t)lda, lim));
+        const uint32_t b_first = TB ? (uint32_t)c.j0 * (uint32_t)lda : (uint32_t)(c.j0 / EPB);
+        c.rs_b = make_rsrc(p.b + (size_t)c.e * p.b_stride + b_first, min(b_bytes - min(b_first, b_bytes), lim));
         if (MX) {
+            // Scale rows are sld bytes long, an even number that need not be a multiple of 4, while the
+            // 16-byte fetches must start on 4-byte boundaries: a row that starts 2 bytes past one is
+            // fetched from 2 bytes earlier and the reader shifts (ph_a, ph_b).  The descriptors
+            // therefore start at the (aligned) beginning of the whole scale array.
             const int idx = (wave & 3) * 64 + lane;
             if (wave < 4) {
-                c.rs_sc = make_rsrc(p.sa + (size_t)c.m0 * p.sld, (uint32_t)min((int64_t)(p.T - c.m0) * p.sld, (int64_t)c.lim));
-                c.off_sc = (uint32_t)min(idx, c.m_end - 1 - c.m0) * (uint32_t)p.sld;
+                c.rs_sc = make_rsrc(p.sa, (uint32_t)min((int64_t)p.T * p.sld, (int64_t)lim));
+                c.off_sc = ((uint32_t)(c.m0 + min(idx, c.m_end - 1 - c.m0)) * (uint32_t)p.sld) & ~3u;
             } else if (TB) {
-                c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride, (uint32_t)min((int64_t)p.N * p.sld, (int64_t)c.lim));
-                c.off_sc = (uint32_t)min(c.j0 + idx, p.N - 1) * (uint32_t)p.sld;
+                c.rs_sc = make_rsrc(p.sb, (uint32_t)min((int64_t)p.num_groups * p.N * p.sld, (int64_t)lim));
+                c.off_sc = ((uint32_t)(c.e * p.N + min(c.j0 + idx, p.N - 1)) * (uint32_t)p.sld) & ~3u;
             } else {
                 // [K/64][N][2]: a scale group is 8 rows of K64 blocks (4 MXFP8 steps, 2 MXFP4 steps)
                 // x 256 columns x 2 bytes; wave 4+i fetches rows 2i, 2i+1, lane l 16 bytes of row l/32
-                c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride, (uint32_t)min((int64_t)p.N * p.sld, (int64_t)c.lim));
+                c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride, (uint32_t)min((int64_t)p.N * p.sld, (int64_t)lim));
                 c.off_sc = (uint32_t)((lane >> 5) + 2 * (wave - 4)) * (uint32_t)p.N * 2u + (uint32_t)c.j0 * 2u + (uint32_t)(lane & 31) * 16u;
             }
+            // Rows wm*128 + s*32 + r of A and columns j0 + wn*64 + s*32 + r of B: only r, m0, j0 and the
+            // expert decide by how many bytes (0 or 2) a scale row starts past a 4-byte boundary (the
+            // other terms are multiples of 4 rows).  The reader holds the 8 bytes from the fetched
+            // dword of a step on (lo, hi); lane group g wants the step's bytes g and 2 + g in bytes 0
+            // and 2 of one register (the matrix instruction picks either with its byte selector).
+            const uint32_t ph_a = ((uint32_t)(c.m0 + r) * (uint32_t)p.sld) & 3u;
+            const uint32_t ph_b = ((uint32_t)(c.e * p.N + c.j0 + r) * (uint32_t)p.sld) & 3u;
+            c.sel_a = 0x0c000c00u | (ph_a + g) | ((ph_a + g + 2) << 16);
+            // TB = 0: lo / hi are the dwords of K64 rows 2x and 2x+1, two columns of two bytes each
+            c.sel_b = TB ? 0x0c000c00u | (ph_b + g) | ((ph_b + g + 2) << 16)
+                         : 0x0c000c00u | (uint32_t)((r & 1) * 2 + g) | ((uint32_t)(4 + (r & 1) * 2 + g) << 16);
         }
     };
 
-    // Requests K-step kt of tile c into ring stage `stage`: NV instructions per wave, issued one
-    // at a time (piece 0..NV-1) so that they interleave with MFMAs instead of reaching the
-    // texture addresser as one burst from all eight waves.
-    auto issue_piece = [&](const TileCtx &c, int kt, int stage, auto piece_c, auto ntb_c) {
-        constexpr int piece = decltype(piece_c)::value;
-        constexpr bool NTB = decltype(ntb_c)::value != 0;
-        const uint32_t lds = lds_base + (uint32_t)(RING_OFF + stage * STAGE_BYTES) + (uint32_t)(wave * NJ) * 1024u;
-        if constexpr (piece < NJ) {
-            load16_to_lds(c.rs_a, c.off_a[piece], (uint32_t)kt * BKB, lds + piece * 1024u);
-        } else if constexpr (piece < 2 * NJ) {
-            if constexpr (NTB)
-                load16_to_lds_nt(c.rs_b, c.off_b[piece - NJ], TB ? (uint32_t)kt * BKB : (uint32_t)kt * (BKB * EPB) * (uint32_t)ldb,
-                                 lds + PANEL_BYTES + (piece - NJ) * 1024u);
-            else
-                load16_to_lds(c.rs_b, c.off_b[piece - NJ], TB ? (uint32_t)kt * BKB : (uint32_t)kt * (BKB * EPB) * (uint32_t)ldb,
-                              lds + PANEL_BYTES + (piece - NJ) * 1024u);
+    // ---- requests.  K-step kt of tile c into ring stage `stage`.
+    // Lanes whose 16 bytes start at or past the end of the row fetch nothing (LDS gets zeros).
+    auto issue_a = [&](const TileCtx &c, int kt, int stage, auto q_c) {
+        constexpr int q = decltype(q_c)::value;
+#ifdef CCH_V_NOLOAD
+        return;
+#endif
+        const uint32_t rem = (uint32_t)max(lda - kt * BKB, 0);
+        const uint32_t voff = ((q & 1) ? cb1 : cb0) < rem ? off_a[q] : NO_FETCH;
+        const uint32_t row0 = (uint32_t)(wm * WM + (q >> 1) * 64 + (wn * 2 + (q & 1)) * 8);
+        load16_to_lds(c.rs_a, voff, (uint32_t)kt * BKB, lds_base + (uint32_t)(RING_OFF + stage * STAGE_BYTES) + row0 * BKB);
+    };
+    auto issue_b = [&](const TileCtx &c, int kt, int stage, auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+#ifdef CCH_V_NOLOAD
+        return;
+#endif
+        const uint32_t lds = lds_base + (uint32_t)(RING_OFF + stage * STAGE_BYTES + PANEL_BYTES) + (uint32_t)(wave * NJ + j) * 1024u;
+        if constexpr (TB) {
+            const uint32_t rem = (uint32_t)max(lda - kt * BKB, 0);
+            const uint32_t voff = ((j & 1) ? cb1 : cb0) < rem ? off_b[j] : NO_FETCH;
+            load16_to_lds(c.rs_b, voff, (uint32_t)kt * BKB, lds);
+        } else {
+            // K-rows past the operand's last one lie past its descriptor
+            load16_to_lds(c.rs_b, off_b[j] + (uint32_t)kt * (BKB * EPB) * (uint32_t)ldb, 0u, lds);
         }
     };
     // Scale group `grp` of tile c (steps grp*SPG .. grp*SPG+SPG-1) into scale buffer `buf`: waves
     // 0-3 fetch 16 bytes of each A row, one row per lane; waves 4-7 the same for the B rows
-    // (TB = 1) or 1 KiB each of the group's eight [column][2] rows (TB = 0).
-    auto issue_scales = [&](int newgrp, const TileCtx &c, int grp, int buf) {
-        if constexpr (MX)
-            load16_to_lds_if(newgrp, c.rs_sc, c.off_sc, (TB || wave < 4) ? (uint32_t)grp * 16u : (uint32_t)grp * 16u * (uint32_t)p.N,
-                             lds_base + (uint32_t)(SCALE_OFF + buf * SCALE_BUF) + (uint32_t)(wave >= 4) * 4096u + (uint32_t)(wave & 3) * 1024u);
+    // (TB = 1) or 1 KiB each of the group's eight [column][2] rows (TB = 0).  When the group is
+    // not due the request is issued all the same, against an empty descriptor and into the sink,
+    // so that the number of requests in flight never depends on the step.
+    auto issue_scales = [&](int due, const TileCtx &c, int grp, int buf) {
+#ifdef CCH_V_NOLOAD
+        return;
+#endif
+        if constexpr (MX) {
+            due = uniform(due);
+            Rsrc rs = c.rs_sc;
+            rs[2] = due ? rs[2] : 0;
+            const uint32_t goff = (TB || wave < 4) ? (uint32_t)grp * 16u : (uint32_t)grp * 16u * (uint32_t)p.N;   // 8 rows of 2N bytes
+            const uint32_t dst = due ? (uint32_t)(SCALE_OFF + buf * SCALE_BUF) + (uint32_t)(wave >= 4) * 4096u + (uint32_t)(wave & 3) * 1024u
+                                     : (uint32_t)SINK_OFF;
+            load16_to_lds(rs, c.off_sc + goff, 0u, lds_base + dst);
+        }
     };
-    auto issue_step = [&](const TileCtx &c, int kt, int stage) {
-        static_for<NV>([&](auto piece_c) { issue_piece(c, kt, stage, piece_c, IC<0>{}); });
-    };
-
-    // Tile set-up: epilogue parameters of the tile (per-token / per-channel scales) and its
-    // first step.  Every wave issues the same number of instructions.
-    auto setup = [&](const TileCtx &c, int parity, int stage) {
+    // Epilogue parameters of a tile (per-token / per-channel scales, or the destination rows).
+    auto issue_params = [&](const TileCtx &c, int parity) {
+        const uint32_t lim = c.valid ? 0x7FFFFFFFu : 0u;
+        const int idx = (wave & 3) * 64 + lane;
+        // destination of lane 0 of this wave; lane l lands 4*l bytes further
+        const uint32_t dst = lds_base + (uint32_t)(PARAM_OFF + parity * PARAM_SET) + (uint32_t)(wave & 3) * 256u;
         if (EPI != EPI_PLAIN) {
-            const int idx = (wave & 3) * 64 + lane;
-            // destination of lane 0 of this wave; lane l lands 4*l bytes further
-            const uint32_t dst = lds_base + (uint32_t)(PARAM_OFF + parity * PARAM_SET) + (uint32_t)(wave & 3) * 256u;
-            load4_to_lds(make_rsrc(p.per_tok + c.m0, c.lim), (uint32_t)min(idx, c.m_end - 1 - c.m0) * 4u, 0u, dst);
+            load4_to_lds(make_rsrc(p.per_tok + c.m0, min((uint32_t)(p.T - c.m0) * 4u, lim)), (uint32_t)min(idx, c.m_end - 1 - c.m0) * 4u, 0u, dst);
             int col;
             if (SWIGLU) col = ((idx >> 5) & 1) * p.n_out + min(c.j0 + (idx >> 6) * 32 + (idx & 31), p.n_out - 1);
             else col = min(c.j0 + idx, p.N - 1);
-            load4_to_lds(make_rsrc(p.per_ch + (size_t)c.e * p.N, c.lim), (uint32_t)col * 4u, 0u, dst + 1024u);
+            load4_to_lds(make_rsrc(p.per_ch + (size_t)c.e * p.N, min((uint32_t)p.N * 4u, lim)), (uint32_t)col * 4u, 0u, dst + 1024u);
         } else {
             // destination rows of the tile's 256 rows, where the per-token scales of the other
             // epilogues go; without a map the descriptor is empty and nothing is fetched
-            const int idx = (wave & 3) * 64 + lane;
-            const uint32_t dst = lds_base + (uint32_t)(PARAM_OFF + parity * PARAM_SET) + (uint32_t)(wave & 3) * 256u;
-            load4_to_lds(make_rsrc(p.out_row_map + c.m0, has_map ? c.lim : 0u), (uint32_t)min(idx, c.m_end - 1 - c.m0) * 4u, 0u, dst);
+            load4_to_lds(make_rsrc(p.out_row_map + c.m0, has_map ? min((uint32_t)(p.T - c.m0) * 4u, lim) : 0u),
+                         (uint32_t)min(idx, c.m_end - 1 - c.m0) * 4u, 0u, dst);
         }
-        issue_scales(1, c, 0, gi & 1);
-        gi++;
-        issue_step(c, 0, stage);
+    };
+    // Requests by slot.  Step kt of tile c into `stage`:
+    //   L0  A rows of row blocks 2-3          C0  A rows of row blocks 0-1 (one request after each of the first MFMA blocks)
+    //   L1  B panel share, first half         C1  B panel share, second half (likewise)
+    auto issue_l0 = [&](const TileCtx &c, int kt, int stage) {
+        issue_a(c, kt, stage, IC<2>{});
+        issue_a(c, kt, stage, IC<3>{});
+    };
+    auto issue_l1 = [&](const TileCtx &c, int kt, int stage) {
+        issue_b(c, kt, stage, IC<0>{});
+        issue_b(c, kt, stage, IC<1>{});
     };
 
     TileCtx cur, nxt;
     int t = (int)blockIdx.x < nwg ? (int)blockIdx.x : total_tiles, parity = 0;
     int gstep = 0;        // K-steps executed by this workgroup so far; ring stage = gstep & 1
-    bool first = true;
     decode(t, cur);
+    nxt = cur;
     nxt.valid = 0;
-    if (cur.valid) {
-        setup(cur, 0, 0);
-        issue_step(cur, 1, 1);
+    const bool any = cur.valid;
+    if (any) {
+        // Everything the first tile's step 0 and step 1 need, except the last A rows of step 1 (slot
+        // L0 of step 0 requests them); all of it has landed before the first step starts.
+        static_for<NJ>([&](auto j_c) { issue_b(cur, 0, 0, j_c); });
+        static_for<NJ>([&](auto q_c) { issue_a(cur, 0, 0, q_c); });
+        issue_scales(1, cur, 0, gi & 1);
+        gi += MX ? 1 : 0;
+        issue_params(cur, 0);
+        static_for<NJ>([&](auto j_c) { issue_b(cur, 1, 1, j_c); });
+        issue_a(cur, 1, 1, IC<0>{});
+        issue_a(cur, 1, 1, IC<1>{});
+        issue_scales(SPG == 2 && nk_tile > 2, cur, 1, gi & 1);
+        gi += (MX && SPG == 2 && nk_tile > 2) ? 1 : 0;
+        CCH_WAIT_VM_LGKM0(0);
+        CCH_BARRIER();
+        // the second group starts one slot behind the first
+        if (wm == 1) CCH_BARRIER();
     }
     while (cur.valid) {
         Acc acc[MT][NT];
-#pragma unroll
-        for (int i = 0; i < MT; i++)
-#pragma unroll
-            for (int j = 0; j < NT; j++)
-#pragma unroll
-                for (int x = 0; x < 16; x++) acc[i][j][x] = 0;
-
         int nbase = 0;  // gi when the next tile's scale group 0 is requested
-        // Fragment registers.  fa[i] and fb0 hold the first 64-byte substep of the current
-        // step, fb1 the second; fa[i] is refilled with its next contents as soon as the MFMAs
-        // that read it have been issued, so that LDS latency hides behind the other MFMAs.
-        v8i fa[MT], fb0[NT], fb1[NT];
+        // Fragment registers of a slot pair: all B fragments of the step and the A fragments of two
+        // row blocks, both 64-byte halves each.
+        v8i fa[2][2], fb[NT][2];
         constexpr int NSC = SCALE_DW > 0 ? SCALE_DW : 1;
-        uint32_t sc[NSC][MT + NT];  // raw scale dwords of the current step
+        uint32_t sc[NSC][MT + NT];  // scale dwords of the current step, shifted so that byte 0 / 2 is this lane's
 
         auto read_frag = [&](uint32_t row_off, int ks) {
+#ifdef CCH_V_NOLDS
+            return (v8i){(int)row_off, ks, 0, 0, 0, 0, 0, 0};
+#endif
             // lane (r, g) feeds K bytes [16g, 16g+16) of each 32-byte half of the 64-byte substep
             const uint32_t c0 = (((uint32_t)(ks * 4 + g)) ^ swz) << 4, c1 = (((uint32_t)(ks * 4 + 2 + g)) ^ swz) << 4;
             const v4i lo = lds_read16(row_off + c0), hi = lds_read16(row_off + c1);
@@ -444,6 +538,9 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         };
         auto frag_a = [&](int stage, int ks, int i) { return read_frag((uint32_t)(RING_OFF + stage * STAGE_BYTES) + rd_a + i * 32 * BKB, ks); };
         auto frag_b = [&](int stage, int ks, int j) {
+#ifdef CCH_V_NOLDS
+            return (v8i){stage, ks, j, 0, 0, 0, 0, 0};
+#endif
             if constexpr (TB) {
                 return read_frag((uint32_t)(RING_OFF + stage * STAGE_BYTES) + rd_b + j * 32 * BKB, ks);
             } else {
@@ -467,138 +564,241 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 return (v8i){t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
             }
         };
-        // Scale dwords of K-step kt of the current tile
-        auto read_scales = [&](int kt, uint32_t (&dst)[NSC][MT + NT]) {
-            if (!MX) return;
-            const uint32_t ss = (uint32_t)(SCALE_OFF + ((gbase + kt / SPG) & 1) * SCALE_BUF) + (uint32_t)(kt % SPG) * (SCALE_DW * 4u);
+        // Scale dwords of K-step kt of the current tile, in two parts so that the LDS reads can be
+        // issued ahead of the fragment reads and the arithmetic done while those are under way.
+        // In the last two steps of a tile the bytes of the 32-element blocks that lie past K (fetched
+        // from the next row, or not at all) are cleared: their payload is zero, and a zero byte
+        // (2^-127) keeps the product zero where a stray 0xFF (NaN) would not.  Lane group g uses
+        // byte g and byte 2 + g of a dword: the shift lets the matrix instruction pick them with its
+        // byte selector (one byte permute per dword does both).
+        uint32_t raw_lo[NSC][MT + NT], raw_hi[NSC][MT + NT];
+        auto read_scales_raw = [&](int kt) {
+#ifdef CCH_V_NOSCALE
+            return;
+#endif
+            if constexpr (MX) {
+                const int grp = kt / SPG, w0 = (kt - grp * SPG) * SCALE_DW;   // dword of the step inside its group's 16 bytes
+                const uint32_t bufc = (uint32_t)(SCALE_OFF + ((gbase + grp) & 1) * SCALE_BUF);       // this group's buffer
+                const uint32_t bufn = (uint32_t)(SCALE_OFF + ((gbase + grp + 1) & 1) * SCALE_BUF);   // the next group's
 #pragma unroll
-            for (int d = 0; d < SCALE_DW; d++) {
+                for (int d = 0; d < SCALE_DW; d++) {
+                    // A row fetched from 2 bytes before its start holds the step's four bytes across two
+                    // dwords; the second one of a group's last dword is the first of the next group's.
+                    const int w = w0 + d;
+                    const uint32_t lo_off = bufc + (uint32_t)w * 4u, hi_off = w == 3 ? bufn : bufc + (uint32_t)w * 4u + 4u;
 #pragma unroll
-                for (int s = 0; s < MT; s++) dst[d][s] = lds_read4(ss + rd_sa + s * 512 + d * 4);
+                    for (int s = 0; s < MT; s++) {
+                        raw_lo[d][s] = lds_read4(lo_off + rd_sa + s * 512);
+                        if constexpr (UA) raw_hi[d][s] = lds_read4(hi_off + rd_sa + s * 512);
+                    }
 #pragma unroll
-                for (int s = 0; s < NT; s++) {
-                    if constexpr (TB) {
-                        dst[d][MT + s] = lds_read4(ss + rd_sb + s * 512 + d * 4);
-                    } else {
-                        // The two K32 scales of K64 row 2x and of row 2x+1, for this column: bytes
-                        // 2*ks + g of the step's dword as in the TB = 1 layout.  Each row holds two
-                        // columns per dword; the permute keeps this column's half of both.
-                        const uint32_t sb0 = (uint32_t)(SCALE_OFF + ((gbase + kt / SPG) & 1) * SCALE_BUF) + rd_sb + s * 64 +
-                                             (uint32_t)((kt % SPG) * (2 * SCALE_DW) + d * 2) * 512u;
-                        dst[d][MT + s] = __builtin_amdgcn_perm(lds_read4(sb0 + 512), lds_read4(sb0), sb_sel);
+                    for (int s = 0; s < NT; s++) {
+                        if constexpr (TB) {
+                            raw_lo[d][MT + s] = lds_read4(lo_off + rd_sb + s * 512);
+                            if constexpr (UA) raw_hi[d][MT + s] = lds_read4(hi_off + rd_sb + s * 512);
+                        } else {
+                            // the two K32 scales of K64 row 2x and of row 2x+1; each row holds two columns per dword
+                            const uint32_t sb0 = bufc + rd_sb + s * 64 + (uint32_t)((kt - grp * SPG) * (2 * SCALE_DW) + d * 2) * 512u;
+                            raw_lo[d][MT + s] = lds_read4(sb0);
+                            raw_hi[d][MT + s] = lds_read4(sb0 + 512);
+                        }
                     }
                 }
             }
         };
-        // One MFMA of row block i of a 64-byte substep; m = 0 .. MPR-1 walks the row: all
-        // column blocks on the low 32 bytes, then (int8 and FP4, which take two MFMAs per
-        // 64 bytes) all on the high 32 bytes, so that consecutive MFMAs never share an accumulator.
-        constexpr int MPR = KIND == KIND_F8 ? NT : 2 * NT;  // MFMAs per row block
-        auto mfma_one = [&](auto ks_c, auto i_c, auto m_c, const v8i &a, const v8i (&b)[NT]) {
-            constexpr int ks = decltype(ks_c)::value, i = decltype(i_c)::value, m = decltype(m_c)::value;
-            constexpr int j = m % NT, half = m / NT;
-            if constexpr (KIND == KIND_F8) {
-                // scale operands: lane group g presents byte 2*ks + g of the row's dword
-                const int sh = 8 * (2 * ks) + 8 * g;
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b[j], acc[i][j], CBSZ, CBSZ, 0, (int)(sc[0][i] >> sh), 0,
-                                                                            (int)(sc[0][MT + j] >> sh));
-            } else if constexpr (KIND == KIND_F4) {
-                // substep = 128 elements = scale dword ks; the low MFMA uses byte g, the high one byte 2+g
-                const int sA = (int)(sc[ks][i] >> (8 * g)), sB = (int)(sc[ks][MT + j] >> (8 * g));
-                const v8i ah = (v8i){a[4 * half], a[4 * half + 1], a[4 * half + 2], a[4 * half + 3], 0, 0, 0, 0};
-                const v8i bh = (v8i){b[j][4 * half], b[j][4 * half + 1], b[j][4 * half + 2], b[j][4 * half + 3], 0, 0, 0, 0};
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ah, bh, acc[i][j], 4, 4, 2 * half, sA, 2 * half, sB);
-            } else {
-                const v4i ah = (v4i){a[4 * half], a[4 * half + 1], a[4 * half + 2], a[4 * half + 3]};
-                const v4i bh = (v4i){b[j][4 * half], b[j][4 * half + 1], b[j][4 * half + 2], b[j][4 * half + 3]};
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah, bh, acc[i][j], 0, 0, 0);
+        auto finish_scales = [&](auto last_c, int kt) {
+#ifdef CCH_V_NOSCALE
+            for (int d = 0; d < NSC; d++) for (int s = 0; s < MT + NT; s++) sc[d][s] = 0x7f7f7f7fu;
+            return;
+#endif
+            if constexpr (MX) {
+                constexpr bool LAST = decltype(last_c)::value != 0;
+                const int nblk = (p.K + 31) >> 5;
+#pragma unroll
+                for (int d = 0; d < SCALE_DW; d++) {
+                    uint32_t keep = 0xFFFFFFFFu;
+                    if constexpr (LAST) {
+                        // blocks of this dword that lie inside K; this lane's two are g and 2 + g
+                        const int nb = nblk - (kt * SCALE_DW + d) * 4;
+                        keep = (g < nb ? 0xFFu : 0u) | (2 + g < nb ? 0xFF0000u : 0u);
+                    }
+#pragma unroll
+                    for (int s = 0; s < MT + NT; s++) {
+                        // rows that all start on 4-byte boundaries need the low dword only
+                        const bool two = UA || (!TB && s >= MT);
+                        const uint32_t v = __builtin_amdgcn_perm(two ? raw_hi[d][s] : raw_lo[d][s], raw_lo[d][s], s < MT ? cur.sel_a : cur.sel_b);
+                        sc[d][s] = LAST ? v & keep : v;
+                    }
+                }
             }
         };
-        auto mfma_row = [&](auto ks_c, auto i_c, const v8i &a, const v8i (&b)[NT]) {
-            static_for<MPR>([&](auto m_c) { mfma_one(ks_c, i_c, m_c, a, b); });
+        // The MFMAs of row block ai on the 64-byte substep ks: all column blocks on the low 32
+        // bytes, then (int8 and FP4, which take two MFMAs per 64 bytes) all on the high 32 bytes.
+        // With ZERO the accumulators start from zero instead of being read.
+        auto mfma_block = [&](auto zero_c, auto ks_c, auto ai_c, const v8i &a) {
+            constexpr int ks = decltype(ks_c)::value, ai = decltype(ai_c)::value;
+#ifdef CCH_V_NOMFMA
+            if (!decltype(zero_c)::value) { asm volatile("" :: "v"(a)); return; }
+#endif
+            constexpr bool ZERO = decltype(zero_c)::value != 0;
+            if constexpr (KIND == KIND_F8) {
+#pragma unroll
+                for (int j = 0; j < NT; j++) {
+                    Acc c;
+                    if (ZERO) c = (Acc)(0.0f);
+                    else c = acc[ai][j];
+                    acc[ai][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, fb[j][ks], c, CBSZ, CBSZ, 2 * ks, (int)sc[0][ai], 2 * ks,
+                                                                                 (int)sc[0][MT + j]);
+                }
+            } else {
+#pragma unroll
+                for (int half = 0; half < 2; half++)
+#pragma unroll
+                    for (int j = 0; j < NT; j++) {
+                        Acc c;
+                        if (ZERO && half == 0) c = (Acc)(0);
+                        else c = acc[ai][j];
+                        if constexpr (KIND == KIND_F4) {
+                            // substep = 128 elements = scale dword ks; the low MFMA uses byte g, the high one byte 2+g
+                            const v8i ah = (v8i){a[4 * half], a[4 * half + 1], a[4 * half + 2], a[4 * half + 3], 0, 0, 0, 0};
+                            const v8i bh = (v8i){fb[j][ks][4 * half], fb[j][ks][4 * half + 1], fb[j][ks][4 * half + 2], fb[j][ks][4 * half + 3], 0, 0, 0, 0};
+                            if (half == 0)
+                                acc[ai][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ah, bh, c, 4, 4, 0, (int)sc[ks][ai], 0, (int)sc[ks][MT + j]);
+                            else
+                                acc[ai][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ah, bh, c, 4, 4, 2, (int)sc[ks][ai], 2, (int)sc[ks][MT + j]);
+                        } else {
+                            const v4i ah = (v4i){a[4 * half], a[4 * half + 1], a[4 * half + 2], a[4 * half + 3]};
+                            const v4i bh = (v4i){fb[j][ks][4 * half], fb[j][ks][4 * half + 1], fb[j][ks][4 * half + 2], fb[j][ks][4 * half + 3]};
+                            acc[ai][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah, bh, c, 0, 0, 0);
+                        }
+                    }
+            }
         };
 
-        // One K-step.  On entry fa / fb0 / sc hold the step's first substep.  MODE 0: steady
-        // state, requests step kt+2 of this tile; 1: second to last step, requests the next
-        // tile's set-up and first step; 2: last step, requests the next tile's second step and
-        // prefetches no fragments.  The ring stage a step occupies is read for the last time
-        // just before the step's barrier, and the requests issued after that barrier refill
-        // it, two steps ahead of its use.  Everything that follows the barrier is threaded
-        // between the step's remaining MFMAs, one or two instructions at a time, so that the
-        // matrix pipe keeps running while the wave issues them.
-        auto step = [&](auto mode_c, auto mta_c, auto ntb_c, int kt) {
-            constexpr int MODE = decltype(mode_c)::value;
-            constexpr int MTA = decltype(mta_c)::value;   // row blocks of this wave that hold rows of the group
+        // One K-step of the current tile.  MODE 0: steady state; 1: second to last step (its L1
+        // requests the next tile's step 0, scales and epilogue parameters); 2: last step (requests
+        // the next tile's step 0 / step 1 shares, no barrier at its end: the caller places it
+        // around the epilogue).  FIRST: first step of a tile (accumulators start from zero; the
+        // previous tile's output stores are among the younger requests that the waits count).
+        // MTH: halves of this wave's 128 rows that hold rows of the group (0, 1, 2).
+        auto step = [&](auto mode_c, auto first_c, auto mth_c, int kt) {
+            constexpr int MODE = decltype(mode_c)::value, MTH = decltype(mth_c)::value;
+            constexpr int FIRST = decltype(first_c)::value;
             const int stage = gstep & 1, nstage = stage ^ 1;
-            static_for<MT>([&](auto i_c) {
-                constexpr int i = decltype(i_c)::value;
-                if constexpr (i < MTA) mfma_row(IC<0>{}, i_c, fa[i], fb0);
-                __builtin_amdgcn_sched_barrier(0);
-                if constexpr (i < MTA) fa[i] = frag_a(stage, 1, i);
-                if constexpr (i < NT && MTA > 0) fb1[i] = frag_b(stage, 1, i);
-                __builtin_amdgcn_sched_barrier(0);
-            });
-            if constexpr (MTA > 0) mfma_row(IC<1>{}, IC<0>{}, fa[0], fb1);
-            __builtin_amdgcn_sched_barrier(0);
-            // Every LDS read of this step has been issued; once they have returned and the
-            // requests of step kt+1 have landed, for all waves, the stage can be refilled.
-            CCH_WAIT_VM_LGKM0(0);
-            __syncthreads();
-            constexpr int SLOTS = MTA > 0 ? (MTA - 1) * MPR : 0;   // MFMAs left in this step
-            constexpr int NREQ = NV + (MX ? 1 : 0);                // requests of a steady step
-            constexpr int PER_SLOT = SLOTS >= 2 ? (NREQ + SLOTS - 2) / (SLOTS - 1) : NREQ;
-            const int newgrp = ((kt + 2) & (SPG - 1)) == 0;
-            // what follows the first MFMA after the barrier: the next step's first fragments, and
-            // in the peeled steps the next tile's requests
-            auto after_barrier = [&]() {
-                if constexpr (MODE != 2 && MTA > 0) {
+            // Requests that may still be in flight when a wait of this step is reached, oldest first:
+            //   [L0 C0 L1 C1 of the step before] [output stores] [this L0] [this C0] [this L1]
+            constexpr int PREV_L1 = MODE == 2 ? NL1 + NPARAM : NL1;   // what the step before this one issued in its L1
+            constexpr int STORES = FIRST ? NSTORES : 0;
+            constexpr int THIS_L1 = MODE == 1 ? NL1 + NPARAM : NL1;
+            // tile and step that the requests of C0, L1 and C1 are for (two steps ahead)
+            const TileCtx &rq = MODE == 0 ? cur : nxt;
+            const int rq_kt = MODE == 0 ? kt + 2 : MODE - 1;
+            // ------------------------------------------------------------------ L0
+            if constexpr (MTH > 0) {
+                read_scales_raw(kt);
 #pragma unroll
-                    for (int j = 0; j < NT; j++) fb0[j] = frag_b(nstage, 0, j);
-                    fa[0] = frag_a(nstage, 0, 0);
-                }
-                if constexpr (MODE == 1) {
-                    nbase = gi;
-                    setup(nxt, parity ^ 1, stage);
-                } else if constexpr (MODE == 2) {
-                    issue_step(nxt, 1, stage);
-                }
-            };
-            auto requests = [&](auto first_c) {
-                constexpr int first_piece = decltype(first_c)::value;
-                if constexpr (MODE == 0) {
-                    static_for<PER_SLOT>([&](auto q_c) {
-                        constexpr int piece = first_piece + decltype(q_c)::value;
-                        if constexpr (piece < NV) issue_piece(cur, kt + 2, stage, IC<piece>{}, ntb_c);
-                        else if constexpr (piece == NV && MX) {
-                            issue_scales(newgrp, cur, (kt + 2) / SPG, gi & 1);
-                        }
-                    });
-                }
-            };
-            if constexpr (SLOTS == 0) {
-                // a wave with at most one row block to compute: nothing to hide the requests behind
-                after_barrier();
-                requests(IC<0>{});
+                for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                    for (int j = 0; j < NT; j++) fb[j][ks] = frag_b(stage, ks, j);
+                __builtin_amdgcn_sched_barrier(0);
+                finish_scales(IC<MODE != 0>{}, kt);   // while the B fragments arrive; its inputs die before the A fragments need registers
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                    for (int i = 0; i < 2; i++) fa[i][ks] = frag_a(stage, ks, i);
             }
-            static_for<SLOTS>([&](auto slot_c) {
-                constexpr int slot = decltype(slot_c)::value;
-                constexpr int i = 1 + slot / MPR, m = slot % MPR;
-                mfma_one(IC<1>{}, IC<i>{}, IC<m>{}, fa[i], fb1);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (MODE == 2) issue_l0(nxt, 0, nstage);
+            else issue_l0(cur, kt + 1, nstage);
+            __builtin_amdgcn_sched_barrier(0);
+            { PROF_BEGIN(t_); CCH_WAIT_LGKM0(); PROF_END(t_, pf_l0); }
+            { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b0); }
+            // ------------------------------------------------------------------ C0
+            // (the first A rows of the step after the next are requested between the MFMA blocks: their
+            // place, the first rows of this stage's half, was read for the last time in L0)
+            if constexpr (MTH > 0) {
+                CCH_SETPRIO(CCH_PRIO_C);
+                mfma_block(IC<FIRST>{}, IC<0>{}, IC<0>{}, fa[0][0]);
                 __builtin_amdgcn_sched_barrier(0);
-                // The SwiGLU kernel measured 3 % faster with the requests ahead of the next step's
-                // first fragment reads, the others 1 % slower.
-                if constexpr (SWIGLU) {
-                    if constexpr (slot == SLOTS - 1) after_barrier();
-                    else requests(IC<slot * PER_SLOT>{});
-                } else {
-                    if constexpr (slot == 0) after_barrier();
-                    else requests(IC<(slot - 1) * PER_SLOT>{});
-                }
-                if constexpr (MODE != 2 && m == MPR - 1) fa[i] = frag_a(nstage, 0, i);
+                issue_a(rq, rq_kt, stage, IC<0>{});
                 __builtin_amdgcn_sched_barrier(0);
-            });
-            if constexpr (MODE == 0) gi += MX ? newgrp : 0;
-            if constexpr (MODE != 2) read_scales(kt + 1, sc);
+                mfma_block(IC<FIRST>{}, IC<0>{}, IC<1>{}, fa[1][0]);
+                __builtin_amdgcn_sched_barrier(0);
+                issue_a(rq, rq_kt, stage, IC<1>{});
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_block(IC<0>{}, IC<1>{}, IC<0>{}, fa[0][1]);
+                mfma_block(IC<0>{}, IC<1>{}, IC<1>{}, fa[1][1]);
+                CCH_SETPRIO(CCH_PRIO_L);
+            } else {
+                issue_a(rq, rq_kt, stage, IC<0>{});
+                issue_a(rq, rq_kt, stage, IC<1>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // the last A rows of this step (requested in the previous step's L0) must have landed:
+            // younger than them are the previous step's C0, L1 and C1, the stores, and this step's L0 and C0
+            { PROF_BEGIN(t_); CCH_WAIT_VM(NC0 + PREV_L1 + NC1 + STORES + NL0 + NC0); PROF_END(t_, pf_wa); }
+            { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b1); }
+            // ------------------------------------------------------------------ L1
+            if constexpr (MTH > 1) {
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                    for (int i = 0; i < 2; i++) fa[i][ks] = frag_a(stage, ks, 2 + i);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // Scale group n of a tile is requested three steps before its first step (a reader of the
+            // group before it needs its first bytes one step early, see read_scales_raw); group 0 comes
+            // with the tile's first step, and MXFP4's group 1 (steps 2-3) with its second.
+            issue_l1(rq, rq_kt, stage);
+            if constexpr (MODE == 0) {
+                const int due = ((kt + 3) & (SPG - 1)) == 0 && kt + 3 < nk_tile;
+                issue_scales(due, cur, (kt + 3) / SPG, gi & 1);
+                gi += MX ? due : 0;
+            } else if constexpr (MODE == 1) {
+                nbase = gi;
+                issue_scales(1, nxt, 0, gi & 1);
+                gi += MX ? 1 : 0;
+                issue_params(nxt, parity ^ 1);
+            } else {
+                const int due = SPG == 2 && nk_tile > 2;
+                issue_scales(due, nxt, 1, gi & 1);
+                gi += MX ? due : 0;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // B and the first A rows of the next step (requested in the previous step's C0, L1 and C1)
+            // must have landed: younger than them are the stores and this step's L0, C0 and L1
+            { PROF_BEGIN(t_); CCH_WAIT_VM_LGKM0(STORES + NL0 + NC0 + THIS_L1); PROF_END(t_, pf_wb); }
+            { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b2); }
+            // ------------------------------------------------------------------ C1
+            if constexpr (MTH > 1) {
+                CCH_SETPRIO(CCH_PRIO_C);
+                mfma_block(IC<FIRST>{}, IC<0>{}, IC<2>{}, fa[0][0]);
+                __builtin_amdgcn_sched_barrier(0);
+                issue_b(rq, rq_kt, stage, IC<2>{});
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_block(IC<FIRST>{}, IC<0>{}, IC<3>{}, fa[1][0]);
+                __builtin_amdgcn_sched_barrier(0);
+                issue_b(rq, rq_kt, stage, IC<3>{});
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_block(IC<0>{}, IC<1>{}, IC<2>{}, fa[0][1]);
+                mfma_block(IC<0>{}, IC<1>{}, IC<3>{}, fa[1][1]);
+                CCH_SETPRIO(CCH_PRIO_L);
+            } else {
+                issue_b(rq, rq_kt, stage, IC<2>{});
+                issue_b(rq, rq_kt, stage, IC<3>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (MODE != 2) { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b3); }
+            if constexpr (FIRST && MTH < 2) {
+                // row blocks that hold no row of the group are never stored; give them a value all the same
+#pragma unroll
+                for (int i = MTH == 0 ? 0 : 2; i < MT; i++)
+#pragma unroll
+                    for (int j = 0; j < NT; j++)
+#pragma unroll
+                        for (int x = 0; x < 16; x++) acc[i][j][x] = 0;
+            }
             if constexpr (MODE != 0) {
                 // Pin the accumulators here: otherwise the compiler sinks the MFMAs of the
                 // peeled steps into the epilogue and spills their fragments to get them there.
@@ -609,55 +809,35 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             }
             gstep++;
         };
-        // Tile prologue.  In flight, oldest first: this tile's set-up and first step, its
-        // second step (NV requests), then the previous tile's epilogue stores.
-        constexpr int NSTORES = MT * NPASS;
-        constexpr int NSTEP1 = NV;  // requests of the tile's second step
-        if (first) CCH_WAIT_VM_LGKM0(NSTEP1);
-        else CCH_WAIT_VM_LGKM0(NSTEP1 + NSTORES);
-        __syncthreads();
-        // Row blocks of this wave that hold rows of the group: the K loop is instantiated for
+        // Halves of this wave's rows that hold rows of the group: the K loop is instantiated for
         // each count, and a wave whose rows lie wholly past the end of a short group issues its
         // requests and barriers but no matrix instruction (its SIMD then belongs to the other
         // wave it hosts, which covers the other half of the tile's rows).
-        auto k_loop = [&](auto mta_c, auto ntb_c) {
-            constexpr int MTA = decltype(mta_c)::value;
-            const int stage = gstep & 1;
-            if constexpr (MTA > 0) {
-                read_scales(0, sc);
-#pragma unroll
-                for (int j = 0; j < NT; j++) fb0[j] = frag_b(stage, 0, j);
-#pragma unroll
-                for (int i = 0; i < MTA; i++) fa[i] = frag_a(stage, 0, i);
-            }
+        auto k_loop = [&](auto mth_c) {
             // The step count is made opaque per tile: addresses that depend on it (the scale
             // reads of the peeled steps) would otherwise be hoisted out of the tile loop and
             // held in registers through the K loop.
             int nk = ksteps;
             asm volatile("" : "+s"(nk));
-            for (int kt = 0; kt + 2 < nk; kt++) step(IC<0>{}, mta_c, ntb_c, kt);
-            decode(t + nwg, nxt);
-            step(IC<1>{}, mta_c, ntb_c, nk - 2);
-            step(IC<2>{}, mta_c, ntb_c, nk - 1);
+            if (nk > 2) {
+                step(IC<0>{}, IC<1>{}, mth_c, 0);
+                for (int kt = 1; kt + 2 < nk; kt++) step(IC<0>{}, IC<0>{}, mth_c, kt);
+                decode(t + nwg, nxt);
+                step(IC<1>{}, IC<0>{}, mth_c, nk - 2);
+            } else {
+                decode(t + nwg, nxt);
+                step(IC<1>{}, IC<1>{}, mth_c, 0);
+            }
+            step(IC<2>{}, IC<0>{}, mth_c, nk - 1);
         };
-        const int mta = uniform(min(max((cur.m_end - cur.m0 - wm * WM + 31) >> 5, 0), MT));
-        // Weight panels of an expert with at most nt_b_max_tiles row tiles are read by that many
-        // workgroups and never again: their steady-state requests carry the non-temporal hint.
-        const bool ntb = uniform(p.nt_b_max_tiles > 0 && tab.tile_start[cur.e + 1] - tab.tile_start[cur.e] <= p.nt_b_max_tiles);
-        if (ntb) {
-            if (mta == MT) k_loop(IC<MT>{}, IC<1>{});
-            else if (mta == 0) k_loop(IC<0>{}, IC<1>{});
-            else if (mta == 1) k_loop(IC<1>{}, IC<1>{});
-            else if (mta == 2) k_loop(IC<2>{}, IC<1>{});
-            else k_loop(IC<3>{}, IC<1>{});
-        } else {
-            if (mta == MT) k_loop(IC<MT>{}, IC<0>{});
-            else if (mta == 0) k_loop(IC<0>{}, IC<0>{});
-            else if (mta == 1) k_loop(IC<1>{}, IC<0>{});
-            else if (mta == 2) k_loop(IC<2>{}, IC<0>{});
-            else k_loop(IC<3>{}, IC<0>{});
-        }
-        first = false;
+        const int mth = uniform(min(max((cur.m_end - cur.m0 - wm * WM + 63) >> 6, 0), 2));
+        if (mth == 2) k_loop(IC<2>{});
+        else if (mth == 1) k_loop(IC<1>{});
+        else k_loop(IC<0>{});
+
+        // Both groups run the epilogue in the same slot: the first group after the barrier that
+        // ends its last matrix slot, the second (one slot behind) before it.
+        if (wm == 0) CCH_BARRIER();
 
         // Epilogue.  Lane (r, g) holds, for sub-tile (i, j), column r and rows
         // q*8 + g*4 + xr at accumulator index 4q + xr.  PASS_ROWS rows at a time go through the
@@ -737,26 +917,43 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                         ok = ok && (!has_map || (mapped >= 0 && mapped < (int)p.out_rows));   // dropped or out of range: not written
                         out_row = has_map ? (uint32_t)mapped : out_row;
                     }
-                    const uint32_t off = ok ? (out_row * (uint32_t)p.n_out + (uint32_t)col) * 2u : 0xFFFFFFF0u;
+                    const uint32_t off = ok ? (out_row * (uint32_t)p.n_out + (uint32_t)col) * 2u : NO_FETCH;
                     const v4u sv = (v4u){(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]};
                     if (p.nt_out) __builtin_amdgcn_raw_buffer_store_b128(sv, rs_out, (int)off, 0, 2);   // non-temporal
                     else __builtin_amdgcn_raw_buffer_store_b128(sv, rs_out, (int)off, 0, 0);
                 }
             }
         }
+        if (wm == 1) CCH_BARRIER();
         cur = nxt;
         gbase = nbase;
         t += nwg;
         parity ^= 1;
     }
+    if (any) {
+        // the first group executed one barrier fewer than the second (which started one slot behind);
+        // requests against empty descriptors may still be on their way to this workgroup's LDS
+        if (wm == 0) CCH_BARRIER();
+        CCH_WAIT_VM_LGKM0(0);
+    }
+#ifdef CCH_PROF
+    if (lane == 0 && blockIdx.x < 256) {
+        uint64_t *o = cch_prof + ((size_t)blockIdx.x * 8 + wave) * 8;
+        o[0] = __builtin_readcyclecounter() - pf_start; o[1] = pf_l0; o[2] = pf_b0; o[3] = pf_wa; o[4] = pf_b1; o[5] = pf_wb; o[6] = pf_b2; o[7] = pf_b3;
+    }
+#endif
 }
 
-template <int KIND, int EPI, int FMT, int TB>
-static int launch_tile_t(const GemmProblem &p, hipStream_t stream)
+#ifdef CCH_PROF
+extern "C" int cch_prof_read(uint64_t *host) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(cch_prof), sizeof(uint64_t) * 256 * 8 * 8); }
+#endif
+
+template <int KIND, int EPI, int FMT, int TB, int UA>
+static int launch_tile_ua(const GemmProblem &p, hipStream_t stream)
 {
     // the LDS size attribute is set once per device and kernel; setting it twice from two threads is harmless
     static std::atomic<uint64_t> attr_set{0};
-    auto kern = gemm_tile_kernel<KIND, EPI, FMT, TB>;
+    auto kern = gemm_tile_kernel<KIND, EPI, FMT, TB, UA>;
     int dev = 0, cus = 0;
     CCH_HIP(hipGetDevice(&dev));
     const uint64_t dev_bit = (uint64_t)1 << (dev & 63);
@@ -773,28 +970,41 @@ static int launch_tile_t(const GemmProblem &p, hipStream_t stream)
     return launch_status("gemm_tile_kernel");
 }
 
+template <int KIND, int EPI, int FMT, int TB>
+static int launch_tile_t(const GemmProblem &p, hipStream_t stream)
+{
+    if constexpr (KIND != KIND_I8) {
+        if ((p.sld & 3) != 0) return launch_tile_ua<KIND, EPI, FMT, TB, 1>(p, stream);
+    }
+    return launch_tile_ua<KIND, EPI, FMT, TB, 0>(p, stream);
+}
+
 // nullptr when the tiled kernels take this problem; otherwise the precondition that failed (the
 // caller then uses the generic path or reports it).
 const char *gemm_tile_unsupported(const GemmProblem &p, int kind, int epi)
 {
     const int epb = kind == KIND_F4 ? 2 : 1;
-    if (p.K < 2 * BKB * epb || p.K % (BKB * epb) != 0) return "K must be a whole number of 128-byte steps, at least two";
+    const int64_t lda = p.K / epb;
+    // rows are fetched in 16-byte pieces
+    if (p.K < 1 || p.K % (16 * epb) != 0) return "K must be a multiple of 16 bytes per row";
     if (p.n_out % 8 != 0 || !aligned(p.out, 16)) return "output rows must take 16-byte stores (n_out % 8 == 0, out 16-byte aligned)";
     if ((int64_t)BM * p.n_out * 2 >= ((int64_t)1 << 31)) return "output row tile beyond 2 GiB";
     // mapped output rows are addressed from the start of `out` with 32-bit offsets
     if (p.out_row_map && (epi != EPI_PLAIN || p.out_rows * p.n_out * 2 >= ((int64_t)1 << 31) || !aligned(p.out_row_map, 4)))
         return "mapped output beyond 2 GiB or misaligned row map";
     if (p.num_groups > MAX_GROUPS) return "more than 256 groups";
-    if ((int64_t)p.N * (p.K / epb) >= ((int64_t)1 << 31)) return "one right-hand operand beyond 2 GiB (32-bit source offsets)";
+    if ((int64_t)p.N * lda >= ((int64_t)1 << 31)) return "one right-hand operand beyond 2 GiB (32-bit source offsets)";
+    if ((int64_t)BM * lda >= ((int64_t)1 << 31)) return "a row tile of the left-hand operand beyond 2 GiB";
     if (!aligned(p.a, 16) || !aligned(p.b, 16) || p.b_stride % 16 != 0) return "operands must be 16-byte aligned";
-    if (kind != KIND_I8 && (!aligned(p.sa, 4) || !aligned(p.sb, 4) || p.sb_stride % 4 != 0 || p.sld % 4 != 0))
-        return "scale arrays must be 4-byte aligned with a row length that is a multiple of 4";
+    if (kind != KIND_I8 && (!aligned(p.sa, 4) || !aligned(p.sb, 4) || p.sb_stride % 2 != 0)) return "scale arrays must be 4-byte aligned";
+    if (kind != KIND_I8 && ((int64_t)p.num_groups * p.N * p.sld >= ((int64_t)1 << 31) || (int64_t)p.T * p.sld >= ((int64_t)1 << 31)))
+        return "scale arrays beyond 2 GiB";
+    if (kind != KIND_I8 && p.sb_stride != (int64_t)p.N * p.sld) return "scale arrays of the right-hand operands must be back to back";
+    if (epi != EPI_PLAIN && (!aligned(p.per_tok, 4) || !aligned(p.per_ch, 4))) return "dequantisation scales must be 4-byte aligned";
     if (!p.trans_b) {
-        // [K, N] operands: 16-byte pieces of a row of B must not straddle its end
-        const int cpc = 16 * epb;  // columns per 16-byte piece
-        if ((epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) % cpc != 0 || (epi == EPI_DEQUANT_SWIGLU ? p.n_out : p.N) < cpc)
-            return "[K,N] operands need N to be a multiple of 16 bytes";
-        if (kind != KIND_I8 && p.K % 64 != 0) return "[K,N] MX operands need K % 64 == 0";
+        // [K, N] operands: rows of B are fetched in 16-byte pieces that start on 4-byte boundaries
+        if ((p.N / epb) % 4 != 0) return "[K,N] operands need rows of a multiple of 4 bytes";
+        if (epi == EPI_DEQUANT_SWIGLU && p.n_out % 4 != 0) return "[K,N] SwiGLU operands need n/2 to be a multiple of 4";
     }
     return nullptr;
 }
