@@ -83,7 +83,8 @@ constexpr int PARAM_OFF = EPI_OFF + NWAVES * EPI_WAVE;       // per tile parity:
 constexpr int PARAM_SET = 2048;
 constexpr int SINK_OFF = PARAM_OFF + 2 * PARAM_SET;          // 1 KiB where requests that are not due land (zeros)
 constexpr int RING_OFF = SINK_OFF + 1024;                    // NSTAGE stages of an A panel and a B panel
-constexpr int LDS_BYTES = RING_OFF + NSTAGE * STAGE_BYTES;   // 157 KiB of the CU's 160 KiB
+constexpr int RING_B_OFF = RING_OFF + NSTAGE * PANEL_BYTES;  // the ring holds the A panels of both stages, then the B panels
+constexpr int LDS_BYTES = RING_OFF + NSTAGE * STAGE_BYTES;   // 157 KiB of the CU's 160 KiB (the group table is static LDS)
 
 template <int KIND> struct KindTraits;
 template <> struct KindTraits<KIND_I8> { static constexpr int ELEMS_PER_BYTE = 1, SCALE_DW = 0; using Acc = v16i; };
@@ -151,7 +152,7 @@ __device__ __forceinline__ Rsrc make_rsrc(const void *base, uint32_t bytes)
     return rs;
 }
 // Descriptors are wave-uniform by construction; this pins them to scalar registers where the
-// compiler has lost track of that.
+// compiler has lost track of that (the 16-byte requests of the K loop take theirs as built).
 __device__ __forceinline__ Rsrc scalar_rsrc(Rsrc rs)
 {
     Rsrc u;
@@ -163,13 +164,24 @@ __device__ __forceinline__ Rsrc scalar_rsrc(Rsrc rs)
 }
 __device__ __forceinline__ void load16_to_lds(Rsrc rs, uint32_t voff, uint32_t soff, uint32_t lds_addr)
 {
-    rs = scalar_rsrc(rs);
     soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
     lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
                  : "memory", "m0");
+}
+// The same with the LDS address given as a scalar base plus a compile-time displacement (one scalar add
+// straight into M0).
+template <int DISP>
+__device__ __forceinline__ void load16_to_lds_at(Rsrc rs, uint32_t voff, uint32_t soff, uint32_t lds_sbase)
+{
+    soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
+    lds_sbase = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_sbase);
+    asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_sbase), "v"(voff), "s"(rs), "s"(soff), "i"(DISP)
+                 : "memory", "m0", "scc");
 }
 __device__ __forceinline__ void load4_to_lds(Rsrc rs, uint32_t voff, uint32_t soff, uint32_t lds_addr)
 {
@@ -184,6 +196,16 @@ __device__ __forceinline__ void load4_to_lds(Rsrc rs, uint32_t voff, uint32_t so
 
 __device__ __forceinline__ v4i lds_read16(uint32_t off) { return *reinterpret_cast<const v4i *>(smem + off); }
 __device__ __forceinline__ uint32_t lds_read4(uint32_t off) { return *reinterpret_cast<const uint32_t *>(smem + off); }
+// The same reads from an absolute LDS address (a base that already holds the segment's start plus a
+// compile-time displacement, which becomes the instruction's offset field).
+__device__ __forceinline__ v4i lds_read16_abs(uint32_t addr)
+{
+    return *reinterpret_cast<const __attribute__((address_space(3))) v4i *>((uintptr_t)addr);
+}
+__device__ __forceinline__ uint32_t lds_read4_abs(uint32_t addr)
+{
+    return *reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>((uintptr_t)addr);
+}
 
 // Panel layout: row pitch 128 B; 16-byte chunk c of row `row` sits at chunk position
 // c ^ ((row >> 1) & 7), which spreads 16 consecutive rows over all 64 banks for 16-byte reads.
@@ -254,17 +276,31 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     const int r = lane & 31, g = lane >> 5;
 
     const int lda = p.K / KT::ELEMS_PER_BYTE;  // bytes per row of A and of B (K-contiguous)
-    const int ksteps = max((lda + BKB - 1) / BKB, 2);   // a one-step K runs a second, empty step: the pipeline has two stages
+    // an even number of steps per tile, so that a step's ring stage is its parity: an odd count runs one
+    // more, empty step (its requests fetch nothing, its products are zero)
+    const int ksteps = max(((lda + BKB - 1) / BKB + 1) & ~1, 2);
     const int n_tiles = (p.n_out + BN_OUT - 1) / BN_OUT;
     const int total_tiles = uniform(tab.tile_start[p.num_groups]) * n_tiles;  // rows past the groups are not ours
 
-    // LDS read offsets of this lane inside a stage.
+    // ---- LDS addresses of this lane's fragment reads.  Ring: stage s of the A panel at RING_OFF +
+    // s * PANEL_BYTES, of the B panel at RING_B_OFF + s * PANEL_BYTES; row pitch 128 B, 16-byte chunk c
+    // of row `row` at chunk position c ^ swizzle(row).  Lane (r, g) feeds K bytes [16g, 16g+16) of each
+    // 32-byte half of a 64-byte substep: chunks ks*4 + g and ks*4 + 2 + g.  The stage, the row block
+    // and the substep are compile-time displacements of the reads, so no address is computed in the
+    // K loop.
     const uint32_t swz = swizzle_of_row(r);
-    const uint32_t rd_a = (uint32_t)(wm * WM + r) * BKB, rd_b = (uint32_t)PANEL_BYTES + (uint32_t)(wn * WN + r) * BKB;
-    const uint32_t rd_sa = (uint32_t)(wm * WM + r) * 16;
+    uint32_t fr_a[4], fr_b[4];
+#pragma unroll
+    for (int x = 0; x < 4; x++) {   // x = 2*ks + half
+        const uint32_t chunk = (((uint32_t)((x >> 1) * 4 + (x & 1) * 2 + g)) ^ swz) << 4;
+        fr_a[x] = lds_base + (uint32_t)RING_OFF + (uint32_t)(wm * WM + r) * BKB + chunk;
+        fr_b[x] = lds_base + (uint32_t)RING_B_OFF + (uint32_t)(wn * WN + r) * BKB + chunk;
+    }
+    // (absolute LDS addresses, like the fragment bases)
+    const uint32_t rd_sa = lds_base + (uint32_t)(wm * WM + r) * 16;
     // B scales: TB = 1 like A's, 16 bytes per column; TB = 0 eight 512-byte rows per group,
     // [K64 block][column][2]
-    const uint32_t rd_sb = TB ? 4096u + (uint32_t)(wn * WN + r) * 16 : 4096u + (((uint32_t)(wn * WN + r) * 2) & ~3u);
+    const uint32_t rd_sb = lds_base + (TB ? 4096u + (uint32_t)(wn * WN + r) * 16 : 4096u + (((uint32_t)(wn * WN + r) * 2) & ~3u));
     // TB = 0 fragment reads: lane (q = lane / 16, i = lane % 16) addresses K-row 16*(q/2) + i/2 of
     // the substep part and the 8-byte half (i & 1) of 16-byte chunk wn*4 + j*2 + (q & 1), whose
     // position in the row is swizzled by twice the row's low bits (i / 2): the 32 lanes of one pass
@@ -273,21 +309,28 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     // For FP4 the panel has 256 K-rows of 128 bytes (two columns per byte) and the 4-bit form of
     // the load is a 16 x 16 nibble transpose: lane i addresses K-row i at 16 columns (8 bytes) and
     // lane j receives 16 consecutive K nibbles of column j; the chunk swizzle uses row bits 1..3.
+    // The column block j enters the address by an exclusive or: one base per column block.
     constexpr bool FP4K = KIND == KIND_F4;
     constexpr int EPB = KT::ELEMS_PER_BYTE;
     constexpr int BROW = BN / EPB;               // bytes per K-row of the TB = 0 panel
     constexpr int BCPR = BROW / 16;              // 16-byte chunks per K-row
     constexpr int BRPI = 64 / BCPR;              // K-rows filled by one direct-to-LDS instruction
     const int tq = lane >> 4, ti = lane & 15;
-    const uint32_t rd_bt = FP4K ? (uint32_t)PANEL_BYTES + (uint32_t)(32 * (tq >> 1) + ti) * 128u +
-                                      ((uint32_t)((wn * 2) ^ (ti >> 1)) << 4) + (uint32_t)(tq & 1) * 8u
-                                : (uint32_t)PANEL_BYTES + (uint32_t)(16 * (tq >> 1) + (ti >> 1)) * 256u +
-                                      ((uint32_t)((wn * 4 + (tq & 1)) ^ ((ti >> 1) << 1)) << 4) + (uint32_t)(ti & 1) * 8u;
+    const uint32_t rd_bt = FP4K ? (uint32_t)(32 * (tq >> 1) + ti) * 128u + ((uint32_t)((wn * 2) ^ (ti >> 1)) << 4) + (uint32_t)(tq & 1) * 8u
+                                : (uint32_t)(16 * (tq >> 1) + (ti >> 1)) * 256u + ((uint32_t)((wn * 4 + (tq & 1)) ^ ((ti >> 1) << 1)) << 4) +
+                                      (uint32_t)(ti & 1) * 8u;
+    uint32_t fr_bt[NT];
+#pragma unroll
+    for (int j = 0; j < NT; j++) fr_bt[j] = lds_base + (uint32_t)RING_B_OFF + (rd_bt ^ ((uint32_t)j << (FP4K ? 4 : 5)));
+    // wave-uniform LDS addresses of the first panel request of this wave (stage 0)
+    const uint32_t lds_req_a = lds_base + (uint32_t)RING_OFF + (uint32_t)(wm * WM + wn * 16) * BKB;
+    const uint32_t lds_req_b = lds_base + (uint32_t)RING_B_OFF + (uint32_t)(wave * NJ) * 1024u;
     const int ldb = TB ? lda : p.N / EPB;   // bytes between consecutive rows of B as stored
     const uint32_t b_bytes = (uint32_t)min((int64_t)p.N * lda, (int64_t)0x7FFFFFFF);   // one right-hand operand
+    const uint32_t b_step = (uint32_t)(BKB * EPB) * (uint32_t)ldb;                      // TB = 0: bytes of B between K-steps
     // Byte position inside its 128-byte row piece that this lane fetches in the K-contiguous panels
     // (even / odd request of a wave), for cutting the last step off at the row end.
-    const uint32_t cb0 = (uint32_t)((lane & 7) ^ (lane >> 4)) << 4, cb1 = cb0 ^ 64u;
+    const int cb0 = (int)(((lane & 7) ^ (lane >> 4)) << 4), cb1 = cb0 ^ 64;
     // Rows that belong to no group are written as zeros (the reference's golden pads them,
     // examples/utils/gen_data_fp4_mx_alltoallv_gmm.py:788-790): all workgroups share the range,
     // 16 bytes per thread and pass; usually it is empty.
@@ -309,7 +352,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     nwg = uniform(nwg);
 
     // Per-lane source offsets of the panel requests, relative to the descriptors' starts: the same
-    // for every tile, and the same for every second request of a wave up to a wave-uniform term.
+    // for every tile.
     //   A: request q = 2*h + jj fills rows wm*128 + h*64 + (wn*2 + jj)*8 .. +7 of the panel (this wave
     //   fetches rows of the half of the tile that its own group computes); lane l lands at row l/8,
     //   chunk position l%8 and must therefore fetch chunk (l%8) ^ swizzle(row).
@@ -319,29 +362,23 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     //   lands at row l/BCPR, chunk position l%BCPR and fetches tile chunk (l%BCPR) ^ swizzle, 16 bytes
     //   of columns; with SwiGLU chunk tc holds gate or up ((tc >> 1) & 1) columns j0 + (tc >> 2)*32 +
     //   (tc & 1)*16 .. +15.
-    // The swizzle of a request's rows depends on the request's parity only, so requests q and q + 2
-    // differ by a fixed number of rows: offset(q) = par[q & 1] + (q >> 1) * pair_step.
-    uint32_t a_par[2], b_par[2];
+    uint32_t off_a[NJ], off_b[NJ];
 #pragma unroll
-    for (int x = 0; x < 2; x++) {
-        const int row = wm * WM + (wn * 2 + x) * 8 + (lane >> 3);
-        a_par[x] = (uint32_t)row * (uint32_t)lda + ((uint32_t)(lane & 7) ^ swizzle_of_row(row)) * 16u;
+    for (int q = 0; q < NJ; q++) {
+        const int row = wm * WM + (q >> 1) * 64 + (wn * 2 + (q & 1)) * 8 + (lane >> 3);
+        off_a[q] = (uint32_t)row * (uint32_t)lda + ((uint32_t)(lane & 7) ^ swizzle_of_row(row)) * 16u;
         if (TB) {
-            const int brow = (wave * NJ + x) * 8 + (lane >> 3);
+            const int brow = (wave * NJ + q) * 8 + (lane >> 3);
             const uint32_t chunk = ((uint32_t)(lane & 7) ^ swizzle_of_row(brow)) * 16u;
             const int col = SWIGLU ? ((brow >> 5) & 1) * p.n_out + (brow >> 6) * 32 + (brow & 31) : brow;   // relative to j0
-            b_par[x] = (uint32_t)col * (uint32_t)lda + chunk;
+            off_b[q] = (uint32_t)col * (uint32_t)lda + chunk;
         } else {
-            const int kr = (wave * NJ + x) * BRPI + lane / BCPR;
+            const int kr = (wave * NJ + q) * BRPI + lane / BCPR;
             const int tc = (lane % BCPR) ^ (FP4K ? (kr >> 1) & 7 : (kr & 7) << 1);
             const int col = SWIGLU ? ((tc >> 1) & 1) * p.n_out + (tc >> 2) * 32 + (tc & 1) * 16 : tc * 16 * EPB;   // relative to j0
-            b_par[x] = (uint32_t)kr * (uint32_t)ldb + (uint32_t)(col / EPB);
+            off_b[q] = (uint32_t)kr * (uint32_t)ldb + (uint32_t)(col / EPB);
         }
     }
-    uint32_t off_a[NJ], off_b[NJ];
-    const uint32_t a_pair_step = 64u * (uint32_t)lda;                                   // rows between requests q and q + 2
-    const uint32_t b_pair_step = TB ? 16u * (uint32_t)lda : 2u * BRPI * (uint32_t)ldb;
-    for (int q = 0; q < NJ; q++) { off_a[q] = a_par[q & 1] + (uint32_t)(q >> 1) * a_pair_step; off_b[q] = b_par[q & 1] + (uint32_t)(q >> 1) * b_pair_step; }
 
     const int nk_tile = ksteps;
 #ifdef CCH_PROF
@@ -416,51 +453,77 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         }
     };
 
-    // ---- requests.  K-step kt of tile c into ring stage `stage`.
-    // Lanes whose 16 bytes start at or past the end of the row fetch nothing (LDS gets zeros).
-    auto issue_a = [&](const TileCtx &c, int kt, int stage, auto q_c) {
-        constexpr int q = decltype(q_c)::value;
-#ifdef CCH_V_NOLOAD
-        return;
-#endif
-        const uint32_t rem = (uint32_t)max(lda - kt * BKB, 0);
-        const uint32_t voff = ((q & 1) ? cb1 : cb0) < rem ? off_a[q] : NO_FETCH;
-        const uint32_t row0 = (uint32_t)(wm * WM + (q >> 1) * 64 + (wn * 2 + (q & 1)) * 8);
-        load16_to_lds(c.rs_a, voff, (uint32_t)kt * BKB, lds_base + (uint32_t)(RING_OFF + stage * STAGE_BYTES) + row0 * BKB);
+    // ---- requests.  Panel requests of K-step `kstep` (byte offset kstep*128 in a row) into ring stage
+    // STG.  Lanes whose 16 bytes start at or past the end of the row fetch nothing (LDS gets zeros):
+    // `tail` holds what is left of the row from the step's start, worked out once per pair of requests.
+    struct Tail {
+        int koff;
+        bool ok0, ok1;   // per lane: even / odd requests of this wave fetch
     };
-    auto issue_b = [&](const TileCtx &c, int kt, int stage, auto j_c) {
-        constexpr int j = decltype(j_c)::value;
+    auto tail_of = [&](int kstep) {
+        // (the K position is made opaque: for the fixed steps of the peeled requests the lane offsets
+        // would otherwise be worked out once and held in registers through the whole kernel)
+        Tail tl;
+        tl.koff = kstep * BKB;
+        asm volatile("" : "+s"(tl.koff));
+        const int rem = lda - tl.koff;
+        tl.ok0 = cb0 < rem;
+        tl.ok1 = cb1 < rem;
+        return tl;
+    };
+    auto issue_a = [&](const TileCtx &c, const Tail &tl, auto stg_c, auto q_c) {
+        constexpr int q = decltype(q_c)::value, STG = decltype(stg_c)::value;
 #ifdef CCH_V_NOLOAD
         return;
 #endif
-        const uint32_t lds = lds_base + (uint32_t)(RING_OFF + stage * STAGE_BYTES + PANEL_BYTES) + (uint32_t)(wave * NJ + j) * 1024u;
+        const uint32_t voff = ((q & 1) ? tl.ok1 : tl.ok0) ? off_a[q] : NO_FETCH;
+        load16_to_lds_at<STG * PANEL_BYTES + ((q >> 1) * 64 + (q & 1) * 8) * BKB>(c.rs_a, voff, (uint32_t)tl.koff, lds_req_a);
+    };
+    // TB = 0: the K position of a request is part of the lane offset, which the bounds check covers:
+    // K-rows past the operand's last one lie past its descriptor
+    auto issue_b = [&](const TileCtx &c, const Tail &tl, uint32_t boff, auto stg_c, auto j_c) {
+        constexpr int j = decltype(j_c)::value, STG = decltype(stg_c)::value;
+#ifdef CCH_V_NOLOAD
+        return;
+#endif
         if constexpr (TB) {
-            const uint32_t rem = (uint32_t)max(lda - kt * BKB, 0);
-            const uint32_t voff = ((j & 1) ? cb1 : cb0) < rem ? off_b[j] : NO_FETCH;
-            load16_to_lds(c.rs_b, voff, (uint32_t)kt * BKB, lds);
+            const uint32_t voff = ((j & 1) ? tl.ok1 : tl.ok0) ? off_b[j] : NO_FETCH;
+            load16_to_lds_at<STG * PANEL_BYTES + j * 1024>(c.rs_b, voff, (uint32_t)tl.koff, lds_req_b);
         } else {
-            // K-rows past the operand's last one lie past its descriptor
-            load16_to_lds(c.rs_b, off_b[j] + (uint32_t)kt * (BKB * EPB) * (uint32_t)ldb, 0u, lds);
+            load16_to_lds_at<STG * PANEL_BYTES + j * 1024>(c.rs_b, off_b[j] + boff, 0u, lds_req_b);
         }
     };
-    // Scale group `grp` of tile c (steps grp*SPG .. grp*SPG+SPG-1) into scale buffer `buf`: waves
+    auto boff_of = [&](int kstep) {
+        uint32_t boff = (uint32_t)kstep * b_step;
+        asm volatile("" : "+s"(boff));
+        return boff;
+    };
+    // A scale request as the matrix slot before it prepared it: descriptor (empty when no group is due:
+    // the request is issued all the same, so that the number of requests in flight never depends on
+    // the step), lane offset, LDS destination.
+    struct ScaleReq {
+        Rsrc rs;
+        uint32_t voff, dst;
+    };
+    // Scale group `grp` of tile c (steps grp*SPG .. grp*SPG+SPG-1) into the next scale buffer: waves
     // 0-3 fetch 16 bytes of each A row, one row per lane; waves 4-7 the same for the B rows
-    // (TB = 1) or 1 KiB each of the group's eight [column][2] rows (TB = 0).  When the group is
-    // not due the request is issued all the same, against an empty descriptor and into the sink,
-    // so that the number of requests in flight never depends on the step.
-    auto issue_scales = [&](int due, const TileCtx &c, int grp, int buf) {
+    // (TB = 1) or 1 KiB each of the group's eight [column][2] rows (TB = 0).
+    auto prep_scales = [&](int due, const TileCtx &c, int grp) {
+        ScaleReq rq;
+        due = uniform(due);
+        rq.rs = c.rs_sc;
+        rq.rs[2] = due ? rq.rs[2] : 0;
+        rq.voff = c.off_sc + ((TB || wave < 4) ? (uint32_t)grp * 16u : (uint32_t)grp * 16u * (uint32_t)p.N);   // TB = 0: 8 rows of 2N bytes
+        rq.dst = lds_base + (due ? (uint32_t)(SCALE_OFF + (gi & 1) * SCALE_BUF) + (uint32_t)(wave >= 4) * 4096u + (uint32_t)(wave & 3) * 1024u
+                                 : (uint32_t)SINK_OFF);
+        gi += due;
+        return rq;
+    };
+    auto issue_scales = [&](const ScaleReq &rq) {
 #ifdef CCH_V_NOLOAD
         return;
 #endif
-        if constexpr (MX) {
-            due = uniform(due);
-            Rsrc rs = c.rs_sc;
-            rs[2] = due ? rs[2] : 0;
-            const uint32_t goff = (TB || wave < 4) ? (uint32_t)grp * 16u : (uint32_t)grp * 16u * (uint32_t)p.N;   // 8 rows of 2N bytes
-            const uint32_t dst = due ? (uint32_t)(SCALE_OFF + buf * SCALE_BUF) + (uint32_t)(wave >= 4) * 4096u + (uint32_t)(wave & 3) * 1024u
-                                     : (uint32_t)SINK_OFF;
-            load16_to_lds(rs, c.off_sc + goff, 0u, lds_base + dst);
-        }
+        if constexpr (MX) load16_to_lds(rq.rs, rq.voff, 0u, rq.dst);
     };
     // Epilogue parameters of a tile (per-token / per-channel scales, or the destination rows).
     auto issue_params = [&](const TileCtx &c, int parity) {
@@ -481,21 +544,55 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                          (uint32_t)min(idx, c.m_end - 1 - c.m0) * 4u, 0u, dst);
         }
     };
-    // Requests by slot.  Step kt of tile c into `stage`:
-    //   L0  A rows of row blocks 2-3          C0  A rows of row blocks 0-1 (one request after each of the first MFMA blocks)
-    //   L1  B panel share, first half         C1  B panel share, second half (likewise)
-    auto issue_l0 = [&](const TileCtx &c, int kt, int stage) {
-        issue_a(c, kt, stage, IC<2>{});
-        issue_a(c, kt, stage, IC<3>{});
+
+    // LDS addresses of this lane's scale reads of the coming step (prepared in the matrix slot before
+    // its first memory slot): low dword for the A rows and the B columns, and - when rows can start 2
+    // bytes past a 4-byte boundary - the dword after the step's last one, which for the last dword of
+    // a group's 16 bytes is the first of the next group's.
+    uint32_t va_sa = 0, va_sb = 0, va_sa_hi = 0, va_sb_hi = 0;
+    // for the first step of a tile whose group 0 is in the buffer of parity gb & 1
+    auto prep_scale_reads = [&](int gb) {
+        if constexpr (MX) {
+            const uint32_t bufc = (uint32_t)(SCALE_OFF + (gb & 1) * SCALE_BUF), bufn = (uint32_t)(SCALE_OFF + ((gb + 1) & 1) * SCALE_BUF);
+            va_sa = rd_sa + bufc;
+            va_sb = rd_sb + bufc;
+            if constexpr (UA) {
+                va_sa_hi = rd_sa + (SPG == 1 ? bufn : bufc + (uint32_t)SCALE_DW * 4u);
+                va_sb_hi = rd_sb + (SPG == 1 ? bufn : bufc + (uint32_t)SCALE_DW * 4u);
+            }
+            asm volatile("" : "+v"(va_sa), "+v"(va_sb));
+            if constexpr (UA) asm volatile("" : "+v"(va_sa_hi), "+v"(va_sb_hi));
+        }
     };
-    auto issue_l1 = [&](const TileCtx &c, int kt, int stage) {
-        issue_b(c, kt, stage, IC<0>{});
-        issue_b(c, kt, stage, IC<1>{});
+    // from step kt to step kt + 1 of the same tile: a few bytes on, or to the start of the other
+    // buffer when the next step opens a group (the addresses move by wave-uniform amounts)
+    auto advance_scale_reads = [&](int gb, int kt) {
+        if constexpr (MX) {
+            const int grp = kt / SPG, ws = kt - grp * SPG;                          // this step's group and place in it
+            const int to_other = ((gb + grp) & 1) ? -SCALE_BUF : SCALE_BUF;          // from this group's buffer to the next group's
+            const bool opens = ws == SPG - 1;                                       // the next step opens a group
+            const int step_a = SCALE_DW * 4, step_b = TB ? SCALE_DW * 4 : 2 * SCALE_DW * 512;
+            int da = opens ? to_other - ws * step_a : step_a;
+            int db = opens ? to_other - ws * step_b : step_b;
+            asm volatile("" : "+s"(da), "+s"(db));
+            va_sa += (uint32_t)da;
+            va_sb += (uint32_t)db;
+            if constexpr (UA) {
+                // the dword after the next step's last one: the first of the buffer after its own when
+                // that step closes its group
+                const int ws1 = opens ? 0 : ws + 1;
+                int dh = ws1 == SPG - 1 ? (opens ? -to_other : to_other) - ws1 * step_a : step_a;
+                asm volatile("" : "+s"(dh));
+                va_sa_hi = va_sa + (uint32_t)dh;
+                va_sb_hi = va_sb + (uint32_t)dh;
+            }
+            asm volatile("" : "+v"(va_sa), "+v"(va_sb));
+            if constexpr (UA) asm volatile("" : "+v"(va_sa_hi), "+v"(va_sb_hi));
+        }
     };
 
     TileCtx cur, nxt;
     int t = (int)blockIdx.x < nwg ? (int)blockIdx.x : total_tiles, parity = 0;
-    int gstep = 0;        // K-steps executed by this workgroup so far; ring stage = gstep & 1
     decode(t, cur);
     nxt = cur;
     nxt.valid = 0;
@@ -503,16 +600,18 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     if (any) {
         // Everything the first tile's step 0 and step 1 need, except the last A rows of step 1 (slot
         // L0 of step 0 requests them); all of it has landed before the first step starts.
-        static_for<NJ>([&](auto j_c) { issue_b(cur, 0, 0, j_c); });
-        static_for<NJ>([&](auto q_c) { issue_a(cur, 0, 0, q_c); });
-        issue_scales(1, cur, 0, gi & 1);
-        gi += MX ? 1 : 0;
-        issue_params(cur, 0);
-        static_for<NJ>([&](auto j_c) { issue_b(cur, 1, 1, j_c); });
-        issue_a(cur, 1, 1, IC<0>{});
-        issue_a(cur, 1, 1, IC<1>{});
-        issue_scales(SPG == 2 && nk_tile > 2, cur, 1, gi & 1);
-        gi += (MX && SPG == 2 && nk_tile > 2) ? 1 : 0;
+        {
+            const Tail t0 = tail_of(0), t1 = tail_of(1);
+            static_for<NJ>([&](auto j_c) { issue_b(cur, t0, boff_of(0), IC<0>{}, j_c); });
+            static_for<NJ>([&](auto q_c) { issue_a(cur, t0, IC<0>{}, q_c); });
+            issue_scales(prep_scales(1, cur, 0));
+            issue_params(cur, 0);
+            static_for<NJ>([&](auto j_c) { issue_b(cur, t1, boff_of(1), IC<1>{}, j_c); });
+            issue_a(cur, t1, IC<1>{}, IC<0>{});
+            issue_a(cur, t1, IC<1>{}, IC<1>{});
+            issue_scales(prep_scales(SPG == 2 && nk_tile > 2, cur, 1));
+        }
+        prep_scale_reads(0);
         CCH_WAIT_VM_LGKM0(0);
         CCH_BARRIER();
         // the second group starts one slot behind the first
@@ -525,82 +624,77 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // row blocks, both 64-byte halves each.
         v8i fa[2][2], fb[NT][2];
         constexpr int NSC = SCALE_DW > 0 ? SCALE_DW : 1;
-        uint32_t sc[NSC][MT + NT];  // scale dwords of the current step, shifted so that byte 0 / 2 is this lane's
+        uint32_t sc[NSC][MT + NT];  // scale dwords of the current step, this lane's two bytes in bytes 0 and 2
 
-        auto read_frag = [&](uint32_t row_off, int ks) {
+        auto frag_a = [&](auto stg_c, int ks, int i) {
+            constexpr int STG = decltype(stg_c)::value;
 #ifdef CCH_V_NOLDS
-            return (v8i){(int)row_off, ks, 0, 0, 0, 0, 0, 0};
+            return (v8i){ks, i, 0, 0, 0, 0, 0, 0};
 #endif
-            // lane (r, g) feeds K bytes [16g, 16g+16) of each 32-byte half of the 64-byte substep
-            const uint32_t c0 = (((uint32_t)(ks * 4 + g)) ^ swz) << 4, c1 = (((uint32_t)(ks * 4 + 2 + g)) ^ swz) << 4;
-            const v4i lo = lds_read16(row_off + c0), hi = lds_read16(row_off + c1);
+            const v4i lo = lds_read16_abs(fr_a[ks * 2] + (uint32_t)(STG * PANEL_BYTES + i * 32 * BKB));
+            const v4i hi = lds_read16_abs(fr_a[ks * 2 + 1] + (uint32_t)(STG * PANEL_BYTES + i * 32 * BKB));
             return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         };
-        auto frag_a = [&](int stage, int ks, int i) { return read_frag((uint32_t)(RING_OFF + stage * STAGE_BYTES) + rd_a + i * 32 * BKB, ks); };
-        auto frag_b = [&](int stage, int ks, int j) {
+        auto frag_b = [&](auto stg_c, int ks, int j) {
+            constexpr int STG = decltype(stg_c)::value;
 #ifdef CCH_V_NOLDS
-            return (v8i){stage, ks, j, 0, 0, 0, 0, 0};
+            return (v8i){ks, j, 0, 0, 0, 0, 0, 0};
 #endif
             if constexpr (TB) {
-                return read_frag((uint32_t)(RING_OFF + stage * STAGE_BYTES) + rd_b + j * 32 * BKB, ks);
+                const v4i lo = lds_read16_abs(fr_b[ks * 2] + (uint32_t)(STG * PANEL_BYTES + j * 32 * BKB));
+                const v4i hi = lds_read16_abs(fr_b[ks * 2 + 1] + (uint32_t)(STG * PANEL_BYTES + j * 32 * BKB));
+                return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             } else {
                 typedef __attribute__((address_space(3))) v2i *LdsV2;
+                // FP4: four nibble transposes, K elements 32g+0..15, 32g+16..31, 64+32g+0..15, 64+32g+16..31 of
+                // the substep (K-rows of 128 B); else four byte transposes, K bytes 16g+0..7, 16g+8..15,
+                // 32+16g+0..7, 32+16g+8..15 (K-rows of 256 B): the same byte displacements either way
+                const uint32_t base = fr_bt[j] + (uint32_t)(STG * PANEL_BYTES) + (uint32_t)ks * 16384u;
                 v2i t0, t1, t2, t3;
                 if constexpr (FP4K) {
-                    // four nibble transposes: K elements 32g+0..15, 32g+16..31, 64+32g+0..15, 64+32g+16..31 of the substep
-                    const uint32_t base = (uint32_t)(RING_OFF + stage * STAGE_BYTES) + (rd_bt ^ ((uint32_t)j << 4)) + (uint32_t)ks * (128u * 128u);
-                    t0 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base));
-                    t1 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 16u * 128u));
-                    t2 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 64u * 128u));
-                    t3 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 80u * 128u));
+                    t0 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(base));
+                    t1 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(base + 2048u));
+                    t2 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(base + 8192u));
+                    t3 = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LdsV2)(uintptr_t)(base + 10240u));
                 } else {
-                    // four byte transposes: K bytes 16g+0..7, 16g+8..15, 32+16g+0..7, 32+16g+8..15 of the substep
-                    const uint32_t base = (uint32_t)(RING_OFF + stage * STAGE_BYTES) + (rd_bt ^ ((uint32_t)j << 5)) + (uint32_t)ks * (64u * 256u);
-                    t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base));
-                    t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 8u * 256u));
-                    t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 32u * 256u));
-                    t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(lds_base + base + 40u * 256u));
+                    t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(base));
+                    t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(base + 2048u));
+                    t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(base + 8192u));
+                    t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LdsV2)(uintptr_t)(base + 10240u));
                 }
                 return (v8i){t0[0], t0[1], t1[0], t1[1], t2[0], t2[1], t3[0], t3[1]};
             }
         };
-        // Scale dwords of K-step kt of the current tile, in two parts so that the LDS reads can be
-        // issued ahead of the fragment reads and the arithmetic done while those are under way.
-        // In the last two steps of a tile the bytes of the 32-element blocks that lie past K (fetched
-        // from the next row, or not at all) are cleared: their payload is zero, and a zero byte
-        // (2^-127) keeps the product zero where a stray 0xFF (NaN) would not.  Lane group g uses
-        // byte g and byte 2 + g of a dword: the shift lets the matrix instruction pick them with its
-        // byte selector (one byte permute per dword does both).
+        // Scale dwords of the step whose read addresses were prepared (prep_scale_reads), in two parts
+        // so that the LDS reads are issued ahead of the fragment reads and the arithmetic runs while
+        // those are under way.  In the last two steps of a tile the bytes of the 32-element blocks
+        // that lie past K (fetched from the next row, or not at all) are cleared: their payload is
+        // zero, and a zero byte (2^-127) keeps the product zero where a stray 0xFF (NaN) would not.
+        // Lane group g uses byte g and byte 2 + g of a step's dword: one byte permute brings them to
+        // bytes 0 and 2, where the matrix instruction's byte selector finds them.
         uint32_t raw_lo[NSC][MT + NT], raw_hi[NSC][MT + NT];
-        auto read_scales_raw = [&](int kt) {
+        auto read_scales_raw = [&]() {
 #ifdef CCH_V_NOSCALE
             return;
 #endif
             if constexpr (MX) {
-                const int grp = kt / SPG, w0 = (kt - grp * SPG) * SCALE_DW;   // dword of the step inside its group's 16 bytes
-                const uint32_t bufc = (uint32_t)(SCALE_OFF + ((gbase + grp) & 1) * SCALE_BUF);       // this group's buffer
-                const uint32_t bufn = (uint32_t)(SCALE_OFF + ((gbase + grp + 1) & 1) * SCALE_BUF);   // the next group's
 #pragma unroll
                 for (int d = 0; d < SCALE_DW; d++) {
-                    // A row fetched from 2 bytes before its start holds the step's four bytes across two
-                    // dwords; the second one of a group's last dword is the first of the next group's.
-                    const int w = w0 + d;
-                    const uint32_t lo_off = bufc + (uint32_t)w * 4u, hi_off = w == 3 ? bufn : bufc + (uint32_t)w * 4u + 4u;
 #pragma unroll
                     for (int s = 0; s < MT; s++) {
-                        raw_lo[d][s] = lds_read4(lo_off + rd_sa + s * 512);
-                        if constexpr (UA) raw_hi[d][s] = lds_read4(hi_off + rd_sa + s * 512);
+                        raw_lo[d][s] = lds_read4_abs(va_sa + d * 4 + s * 512);
+                        if constexpr (UA) raw_hi[d][s] = d == SCALE_DW - 1 ? lds_read4_abs(va_sa_hi + s * 512) : lds_read4_abs(va_sa + d * 4 + 4 + s * 512);
                     }
 #pragma unroll
                     for (int s = 0; s < NT; s++) {
                         if constexpr (TB) {
-                            raw_lo[d][MT + s] = lds_read4(lo_off + rd_sb + s * 512);
-                            if constexpr (UA) raw_hi[d][MT + s] = lds_read4(hi_off + rd_sb + s * 512);
+                            raw_lo[d][MT + s] = lds_read4_abs(va_sb + d * 4 + s * 512);
+                            if constexpr (UA)
+                                raw_hi[d][MT + s] = d == SCALE_DW - 1 ? lds_read4_abs(va_sb_hi + s * 512) : lds_read4_abs(va_sb + d * 4 + 4 + s * 512);
                         } else {
                             // the two K32 scales of K64 row 2x and of row 2x+1; each row holds two columns per dword
-                            const uint32_t sb0 = bufc + rd_sb + s * 64 + (uint32_t)((kt - grp * SPG) * (2 * SCALE_DW) + d * 2) * 512u;
-                            raw_lo[d][MT + s] = lds_read4(sb0);
-                            raw_hi[d][MT + s] = lds_read4(sb0 + 512);
+                            raw_lo[d][MT + s] = lds_read4_abs(va_sb + d * 1024 + s * 64);
+                            raw_hi[d][MT + s] = lds_read4_abs(va_sb + d * 1024 + 512 + s * 64);
                         }
                     }
                 }
@@ -675,64 +769,104 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             }
         };
 
-        // One K-step of the current tile.  MODE 0: steady state; 1: second to last step (its L1
-        // requests the next tile's step 0, scales and epilogue parameters); 2: last step (requests
-        // the next tile's step 0 / step 1 shares, no barrier at its end: the caller places it
-        // around the epilogue).  FIRST: first step of a tile (accumulators start from zero; the
-        // previous tile's output stores are among the younger requests that the waits count).
-        // MTH: halves of this wave's 128 rows that hold rows of the group (0, 1, 2).
-        auto step = [&](auto mode_c, auto first_c, auto mth_c, int kt) {
-            constexpr int MODE = decltype(mode_c)::value, MTH = decltype(mth_c)::value;
+        // One K-step of the current tile.  MODE 0: steady state; 1: second to last step (its requests
+        // are the next tile's step 0, scales and epilogue parameters); 2: last step (requests the next
+        // tile's step 0 / step 1 shares, no barrier at its end: the caller places it around the
+        // epilogue).  FIRST: first step of a tile (accumulators start from zero; the previous tile's
+        // output stores are among the younger requests that the waits count).  MTH: halves of this
+        // wave's 128 rows that hold rows of the group (0, 1, 2).  STG: ring stage of the step (tiles
+        // have an even number of steps, so a step's stage is its parity).
+        // The memory slots hold nothing but LDS reads, requests and the waits: every wave-uniform
+        // quantity they use is worked out in the matrix slot before them, where the wave has issue
+        // cycles to spare between MFMAs.
+        auto step = [&](auto mode_c, auto first_c, auto mth_c, auto stg_c, int kt) {
+            constexpr int MODE = decltype(mode_c)::value, MTH = decltype(mth_c)::value, STG = decltype(stg_c)::value;
             constexpr int FIRST = decltype(first_c)::value;
-            const int stage = gstep & 1, nstage = stage ^ 1;
             // Requests that may still be in flight when a wait of this step is reached, oldest first:
             //   [L0 C0 L1 C1 of the step before] [output stores] [this L0] [this C0] [this L1]
             constexpr int PREV_L1 = MODE == 2 ? NL1 + NPARAM : NL1;   // what the step before this one issued in its L1
             constexpr int STORES = FIRST ? NSTORES : 0;
             constexpr int THIS_L1 = MODE == 1 ? NL1 + NPARAM : NL1;
-            // tile and step that the requests of C0, L1 and C1 are for (two steps ahead)
+            // tile and step that the requests of C0, L1 and C1 are for (two steps ahead, into this stage)
             const TileCtx &rq = MODE == 0 ? cur : nxt;
             const int rq_kt = MODE == 0 ? kt + 2 : MODE - 1;
+            // The read bases are made opaque per step: base + displacement would otherwise be worked out
+            // once for every displacement and held in a register each through the whole loop.
+#pragma unroll
+            for (int x = 0; x < 4; x++) {
+                asm volatile("" : "+v"(fr_a[x]));
+                if constexpr (TB) asm volatile("" : "+v"(fr_b[x]));
+            }
+            if constexpr (!TB) {
+#pragma unroll
+                for (int j = 0; j < NT; j++) asm volatile("" : "+v"(fr_bt[j]));
+            }
             // ------------------------------------------------------------------ L0
             if constexpr (MTH > 0) {
-                read_scales_raw(kt);
+                read_scales_raw();
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-                    for (int j = 0; j < NT; j++) fb[j][ks] = frag_b(stage, ks, j);
+                    for (int j = 0; j < NT; j++) fb[j][ks] = frag_b(stg_c, ks, j);
                 __builtin_amdgcn_sched_barrier(0);
                 finish_scales(IC<MODE != 0>{}, kt);   // while the B fragments arrive; its inputs die before the A fragments need registers
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-                    for (int i = 0; i < 2; i++) fa[i][ks] = frag_a(stage, ks, i);
+                    for (int i = 0; i < 2; i++) fa[i][ks] = frag_a(stg_c, ks, i);
             }
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (MODE == 2) issue_l0(nxt, 0, nstage);
-            else issue_l0(cur, kt + 1, nstage);
+            // the last A rows of the next step, into the other stage
+            {
+                const Tail tl = tail_of(MODE == 2 ? 0 : kt + 1);
+                issue_a(MODE == 2 ? nxt : cur, tl, IC<STG ^ 1>{}, IC<2>{});
+                issue_a(MODE == 2 ? nxt : cur, tl, IC<STG ^ 1>{}, IC<3>{});
+            }
             __builtin_amdgcn_sched_barrier(0);
             { PROF_BEGIN(t_); CCH_WAIT_LGKM0(); PROF_END(t_, pf_l0); }
             { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b0); }
             // ------------------------------------------------------------------ C0
             // (the first A rows of the step after the next are requested between the MFMA blocks: their
             // place, the first rows of this stage's half, was read for the last time in L0)
+            ScaleReq sreq;
+            Tail rq_tl;
+            uint32_t rq_boff = 0;
             if constexpr (MTH > 0) {
                 CCH_SETPRIO(CCH_PRIO_C);
                 mfma_block(IC<FIRST>{}, IC<0>{}, IC<0>{}, fa[0][0]);
                 __builtin_amdgcn_sched_barrier(0);
-                issue_a(rq, rq_kt, stage, IC<0>{});
+                rq_tl = tail_of(rq_kt);
+                if constexpr (!TB) rq_boff = boff_of(rq_kt);
+                issue_a(rq, rq_tl, stg_c, IC<0>{});
                 __builtin_amdgcn_sched_barrier(0);
                 mfma_block(IC<FIRST>{}, IC<0>{}, IC<1>{}, fa[1][0]);
                 __builtin_amdgcn_sched_barrier(0);
-                issue_a(rq, rq_kt, stage, IC<1>{});
+                issue_a(rq, rq_tl, stg_c, IC<1>{});
                 __builtin_amdgcn_sched_barrier(0);
                 mfma_block(IC<0>{}, IC<1>{}, IC<0>{}, fa[0][1]);
                 mfma_block(IC<0>{}, IC<1>{}, IC<1>{}, fa[1][1]);
                 CCH_SETPRIO(CCH_PRIO_L);
             } else {
-                issue_a(rq, rq_kt, stage, IC<0>{});
-                issue_a(rq, rq_kt, stage, IC<1>{});
+                rq_tl = tail_of(rq_kt);
+                if constexpr (!TB) rq_boff = boff_of(rq_kt);
+                issue_a(rq, rq_tl, stg_c, IC<0>{});
+                issue_a(rq, rq_tl, stg_c, IC<1>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // Scale group n of a tile is requested three steps before its first step (a reader of the
+            // group before it needs its first bytes one step early); group 0 comes with the tile's
+            // first step, and MXFP4's group 1 (steps 2-3) with its second.  Prepared here for L1.
+            if constexpr (MX) {
+                if constexpr (MODE == 0) {
+                    sreq = prep_scales(((kt + 3) & (SPG - 1)) == 0 && kt + 3 < nk_tile, cur, (kt + 3) / SPG);
+                } else if constexpr (MODE == 1) {
+                    nbase = gi;
+                    sreq = prep_scales(1, nxt, 0);
+                } else {
+                    sreq = prep_scales(SPG == 2 && nk_tile > 2, nxt, 1);
+                }
+                asm volatile("" : "+s"(sreq.rs), "+v"(sreq.voff), "+s"(sreq.dst));
             }
             __builtin_amdgcn_sched_barrier(0);
             // the last A rows of this step (requested in the previous step's L0) must have landed:
@@ -744,27 +878,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-                    for (int i = 0; i < 2; i++) fa[i][ks] = frag_a(stage, ks, 2 + i);
+                    for (int i = 0; i < 2; i++) fa[i][ks] = frag_a(stg_c, ks, 2 + i);
             }
             __builtin_amdgcn_sched_barrier(0);
-            // Scale group n of a tile is requested three steps before its first step (a reader of the
-            // group before it needs its first bytes one step early, see read_scales_raw); group 0 comes
-            // with the tile's first step, and MXFP4's group 1 (steps 2-3) with its second.
-            issue_l1(rq, rq_kt, stage);
-            if constexpr (MODE == 0) {
-                const int due = ((kt + 3) & (SPG - 1)) == 0 && kt + 3 < nk_tile;
-                issue_scales(due, cur, (kt + 3) / SPG, gi & 1);
-                gi += MX ? due : 0;
-            } else if constexpr (MODE == 1) {
-                nbase = gi;
-                issue_scales(1, nxt, 0, gi & 1);
-                gi += MX ? 1 : 0;
-                issue_params(nxt, parity ^ 1);
-            } else {
-                const int due = SPG == 2 && nk_tile > 2;
-                issue_scales(due, nxt, 1, gi & 1);
-                gi += MX ? due : 0;
-            }
+            issue_b(rq, rq_tl, rq_boff, stg_c, IC<0>{});
+            issue_b(rq, rq_tl, rq_boff, stg_c, IC<1>{});
+            issue_scales(sreq);
+            if constexpr (MODE == 1) issue_params(nxt, parity ^ 1);
             __builtin_amdgcn_sched_barrier(0);
             // B and the first A rows of the next step (requested in the previous step's C0, L1 and C1)
             // must have landed: younger than them are the stores and this step's L0, C0 and L1
@@ -775,19 +895,23 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 CCH_SETPRIO(CCH_PRIO_C);
                 mfma_block(IC<FIRST>{}, IC<0>{}, IC<2>{}, fa[0][0]);
                 __builtin_amdgcn_sched_barrier(0);
-                issue_b(rq, rq_kt, stage, IC<2>{});
+                issue_b(rq, rq_tl, rq_boff, stg_c, IC<2>{});
                 __builtin_amdgcn_sched_barrier(0);
                 mfma_block(IC<FIRST>{}, IC<0>{}, IC<3>{}, fa[1][0]);
                 __builtin_amdgcn_sched_barrier(0);
-                issue_b(rq, rq_kt, stage, IC<3>{});
+                issue_b(rq, rq_tl, rq_boff, stg_c, IC<3>{});
                 __builtin_amdgcn_sched_barrier(0);
                 mfma_block(IC<0>{}, IC<1>{}, IC<2>{}, fa[0][1]);
                 mfma_block(IC<0>{}, IC<1>{}, IC<3>{}, fa[1][1]);
                 CCH_SETPRIO(CCH_PRIO_L);
             } else {
-                issue_b(rq, rq_kt, stage, IC<2>{});
-                issue_b(rq, rq_kt, stage, IC<3>{});
+                issue_b(rq, rq_tl, rq_boff, stg_c, IC<2>{});
+                issue_b(rq, rq_tl, rq_boff, stg_c, IC<3>{});
             }
+            __builtin_amdgcn_sched_barrier(0);
+            // where the next step (of this tile, or the next tile's first) reads its scales
+            if constexpr (MODE == 2) prep_scale_reads(nbase);
+            else advance_scale_reads(gbase, kt);
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (MODE != 2) { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b3); }
             if constexpr (FIRST && MTH < 2) {
@@ -807,7 +931,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 #pragma unroll
                     for (int j = 0; j < NT; j++) asm volatile("" : "+v"(acc[i][j]));
             }
-            gstep++;
         };
         // Halves of this wave's rows that hold rows of the group: the K loop is instantiated for
         // each count, and a wave whose rows lie wholly past the end of a short group issues its
@@ -817,18 +940,22 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             // The step count is made opaque per tile: addresses that depend on it (the scale
             // reads of the peeled steps) would otherwise be hoisted out of the tile loop and
             // held in registers through the K loop.
-            int nk = ksteps;
+            int nk = nk_tile;
             asm volatile("" : "+s"(nk));
             if (nk > 2) {
-                step(IC<0>{}, IC<1>{}, mth_c, 0);
-                for (int kt = 1; kt + 2 < nk; kt++) step(IC<0>{}, IC<0>{}, mth_c, kt);
+                step(IC<0>{}, IC<1>{}, mth_c, IC<0>{}, 0);
+                step(IC<0>{}, IC<0>{}, mth_c, IC<1>{}, 1);
+                for (int kt = 2; kt + 2 < nk; kt += 2) {
+                    step(IC<0>{}, IC<0>{}, mth_c, IC<0>{}, kt);
+                    step(IC<0>{}, IC<0>{}, mth_c, IC<1>{}, kt + 1);
+                }
                 decode(t + nwg, nxt);
-                step(IC<1>{}, IC<0>{}, mth_c, nk - 2);
+                step(IC<1>{}, IC<0>{}, mth_c, IC<0>{}, nk - 2);
             } else {
                 decode(t + nwg, nxt);
-                step(IC<1>{}, IC<1>{}, mth_c, 0);
+                step(IC<1>{}, IC<1>{}, mth_c, IC<0>{}, 0);
             }
-            step(IC<2>{}, IC<0>{}, mth_c, nk - 1);
+            step(IC<2>{}, IC<0>{}, mth_c, IC<1>{}, nk - 1);
         };
         const int mth = uniform(min(max((cur.m_end - cur.m0 - wm * WM + 63) >> 6, 0), 2));
         if (mth == 2) k_loop(IC<2>{});
