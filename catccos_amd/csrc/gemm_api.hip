@@ -15,7 +15,6 @@ static std::atomic<int> g_force_generic{0};
 static std::atomic<int> g_require_tiled{0};
 static std::atomic<int> g_tile_order{-1};   // -1: chosen per problem
 static std::atomic<int> g_balance{0};
-static std::atomic<int> g_nt_small{1};
 static std::atomic<int> g_nt_out{-1};      // -1: chosen per problem
 
 static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
@@ -23,11 +22,10 @@ static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
     if (prob.T == 0 || prob.n_out == 0) return CCH_OK;
     GemmProblem p = prob;
     const int order = g_tile_order.load();
-    p.tile_order = order >= 0 ? order : (p.group_sizes != nullptr && p.num_groups > 1);
+    p.tile_order = order >= 0 ? order : 2;
     p.balance_rounds = g_balance.load();
     const int nto = g_nt_out.load();
     p.nt_out = nto >= 0 ? nto : (kind == KIND_F4);
-    p.nt_b_max_tiles = (p.group_sizes != nullptr && p.num_groups > 1) ? g_nt_small.load() : 0;
     const bool forced = g_force_generic.load() != 0;
     const char *why = forced ? "force_generic_gemm is set" : gemm_tile_unsupported(p, kind, epi);
     if (why == nullptr) return launch_gemm_tile(p, kind, epi, stream);
@@ -67,10 +65,6 @@ int cch_set_option(const char *name, int value)
     }
     if (strcmp(name, "require_tiled_gemm") == 0) {
         g_require_tiled.store(value);
-        return CCH_OK;
-    }
-    if (strcmp(name, "gemm_nt_small_experts") == 0) {
-        g_nt_small.store(value);
         return CCH_OK;
     }
     if (strcmp(name, "gemm_nt_output") == 0) {

@@ -34,10 +34,10 @@ struct GemmProblem {
     int sld;                 // scale bytes per row: 2*ceil(K/64)
     int64_t b_stride;        // bytes between experts in b
     int64_t sb_stride;       // bytes between experts in sb
-    int nt_b_max_tiles;      // tiled kernels: non-temporal weight requests for experts with at most this many row tiles (0: never)
     int nt_out;              // tiled kernels: output stores carry the non-temporal hint
     int balance_rounds;      // tiled kernels: use only as many workgroups as the round count needs
-    int tile_order;          // tiled kernels: 0 = row-major over (row tile, column tile); 1 = runs of consecutive tiles per XCD
+    int tile_order;          // tiled kernels: 0 = row-major over (row tile, column tile); 1 = runs of consecutive tiles per XCD;
+                             // 2 = a block of 4 row tiles x 8 column tiles per XCD where the shape allows (else 1 for groups, 0 without)
 };
 
 // Row ranges and tile counts of the groups, kept in LDS by every workgroup.

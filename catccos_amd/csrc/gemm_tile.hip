@@ -395,17 +395,19 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         c.valid = t < total_tiles;
         const uint32_t lim = c.valid ? 0x7FFFFFFFu : 0u;
         t = max(min(t, total_tiles - 1), 0);
-        if (p.tile_order == 1 && (nwg & 7) == 0 && t < total_tiles - total_tiles % nwg) {
-            // Workgroup w of a round runs on XCD w % 8: give each XCD a run of gridDim.x / 8
-            // consecutive tiles of the round (whole row tiles next to each other), so that its L2
-            // fetches one or two A panels and the B panels of one or two experts per round.
+        const bool whole_round = t < total_tiles - total_tiles % nwg;   // the last, partial round stays row-major
+        if (p.tile_order == 2 && nwg == 256 && (n_tiles == 8 || n_tiles == 16 || n_tiles == 32 || n_tiles == 64) && whole_round) {
+            // Workgroup w of a round runs on XCD w % 8.  Each XCD takes a block of 4 row tiles x 8
+            // column tiles of the round (256 / n_tiles row tiles by n_tiles column tiles): a weight
+            // panel then has up to four users in one L2 and a token panel eight.
+            const int G = nwg, j = t / G, w = t - j * G, x = w & 7, i = w >> 3, cb = n_tiles >> 3;
+            t = j * G + ((x / cb) * 4 + (i >> 3)) * n_tiles + (x % cb) * 8 + (i & 7);
+        } else if ((p.tile_order == 1 || (p.tile_order == 2 && p.group_sizes != nullptr && p.num_groups > 1)) && (nwg & 7) == 0 && whole_round) {
+            // Each XCD takes a run of nwg / 8 consecutive tiles of the round (whole row tiles next
+            // to each other), so that its L2 fetches one or two A panels and the B panels of one or
+            // two experts per round.
             const int G = nwg, j = t / G, w = t - j * G;
             t = j * G + (w & 7) * (G >> 3) + (w >> 3);
-        } else if (p.tile_order == 2 && nwg == 256 && n_tiles == 16 && t < total_tiles - total_tiles % nwg) {
-            // Each XCD takes a block of 4 row tiles x 8 column tiles of the round: a weight panel then
-            // has up to four users in one L2 and a token panel eight.
-            const int G = nwg, j = t / G, w = t - j * G, x = w & 7, i = w >> 3;
-            t = j * G + ((x >> 1) * 4 + (i >> 3)) * n_tiles + (x & 1) * 8 + (i & 7);
         }
         const int tr = t / n_tiles, nt = t - tr * n_tiles;
         c.e = uniform(find_group(tab, p.num_groups, tr));

@@ -227,7 +227,8 @@ def dyn_quant_i8_rows(x_bf16, src=None, topk=1, mode=DQ_DEVICE, smooth=None, smo
     return q, scale
 
 
-def gemm_i8_dequant(a, b, per_tok, per_ch, trans_b=0, rows=None, want_bf16=False):
+def gemm_i8_dequant(a, b, per_tok, per_ch, trans_b=0, rows=None, want_bf16=False, blocked=False):
+    """`blocked` picks the cache-blocked routine (the CPU baseline; same values), see oracle.c."""
     a = np.ascontiguousarray(a, dtype=np.int8)
     b = np.ascontiguousarray(b, dtype=np.int8)
     per_tok = np.ascontiguousarray(per_tok, dtype=np.float32)
@@ -238,12 +239,12 @@ def gemm_i8_dequant(a, b, per_tok, per_ch, trans_b=0, rows=None, want_bf16=False
     cnt = nr if rows is not None else m
     out = np.empty((cnt, n), dtype=np.float32)
     out16 = np.empty((cnt, n), dtype=np.uint16) if want_bf16 else None
-    lib().orc_gemm_i8_dequant(_p(a), _p(b), _p(per_tok), _p(per_ch), _i64(m), _i64(n), _i64(k), int(trans_b),
-                              _p(r), _i64(nr), _p(out), _p(out16))
+    fn = lib().orc_gemm_i8_dequant_blocked if blocked else lib().orc_gemm_i8_dequant
+    fn(_p(a), _p(b), _p(per_tok), _p(per_ch), _i64(m), _i64(n), _i64(k), int(trans_b), _p(r), _i64(nr), _p(out), _p(out16))
     return (out, out16) if want_bf16 else out
 
 
-def gmm_i8_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, fp16_step=False, rows=None, want_bf16=False):
+def gmm_i8_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, fp16_step=False, rows=None, want_bf16=False, blocked=False):
     x = np.ascontiguousarray(x, dtype=np.int8)
     w = np.ascontiguousarray(w, dtype=np.int8)
     gs = np.ascontiguousarray(group_sizes, dtype=np.int32)
@@ -256,13 +257,16 @@ def gmm_i8_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, fp16_step=False, r
     cnt = nr if rows is not None else t
     out = np.empty((cnt, n // 2), dtype=np.float32)
     out16 = np.empty((cnt, n // 2), dtype=np.uint16) if want_bf16 else None
-    lib().orc_gmm_i8_dequant_swiglu(_p(x), _p(w), _p(gs), _i64(e), _i64(t), _i64(k), _i64(n), _p(per_tok),
-                                    _p(per_ch), int(fp16_step), _p(r), _i64(nr), _p(out), _p(out16))
+    fn = lib().orc_gmm_i8_dequant_swiglu_blocked if blocked else lib().orc_gmm_i8_dequant_swiglu
+    fn(_p(x), _p(w), _p(gs), _i64(e), _i64(t), _i64(k), _i64(n), _p(per_tok), _p(per_ch), int(fp16_step), _p(r), _i64(nr),
+       _p(out), _p(out16))
     return (out, out16) if want_bf16 else out
 
 
-def mx_gmm(a, sa, b, sb, n, k, fmt=E4M3, trans_b=0, group_sizes=None, rows=None, want_bf16=False, want_f64=False):
-    """Dense (group_sizes None, b one expert) or grouped MX GEMM golden; see oracle.c:orc_mx_gmm."""
+def mx_gmm(a, sa, b, sb, n, k, fmt=E4M3, trans_b=0, group_sizes=None, rows=None, want_bf16=False, want_f64=False, blocked=False):
+    """Dense (group_sizes None, b one expert) or grouped MX GEMM golden; see oracle.c:orc_mx_gmm.
+    `blocked` picks the cache-blocked routine (the CPU baseline; same values, no fp64 copy)."""
+    assert not (blocked and want_f64)
     a = np.ascontiguousarray(a, dtype=np.uint8)
     sa = np.ascontiguousarray(sa, dtype=np.uint8)
     b = np.ascontiguousarray(b, dtype=np.uint8)
@@ -280,8 +284,12 @@ def mx_gmm(a, sa, b, sb, n, k, fmt=E4M3, trans_b=0, group_sizes=None, rows=None,
     out = np.empty((cnt, n), dtype=np.float32)
     out16 = np.empty((cnt, n), dtype=np.uint16) if want_bf16 else None
     out64 = np.empty((cnt, n), dtype=np.float64) if want_f64 else None
-    lib().orc_mx_gmm(_p(a), _p(sa), _p(b), _p(sb), _p(gs), _i64(e), _i64(t), _i64(n), _i64(k), fmt, int(trans_b),
-                     _p(r), _i64(nr), _p(out), _p(out16), _p(out64))
+    if blocked:
+        lib().orc_mx_gmm_blocked(_p(a), _p(sa), _p(b), _p(sb), _p(gs), _i64(e), _i64(t), _i64(n), _i64(k), fmt, int(trans_b),
+                                 _p(r), _i64(nr), _p(out), _p(out16))
+    else:
+        lib().orc_mx_gmm(_p(a), _p(sa), _p(b), _p(sb), _p(gs), _i64(e), _i64(t), _i64(n), _i64(k), fmt, int(trans_b),
+                         _p(r), _i64(nr), _p(out), _p(out16), _p(out64))
     res = [out]
     if want_bf16:
         res.append(out16)

@@ -750,6 +750,293 @@ void orc_mx_gmm(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uin
     free(row_expert);
 }
 
+/* ------------------------------------------------ blocked CPU baselines */
+
+/*
+ * The routines above compute one output row at a time and decode every
+ * weight again for every row: fine as a golden, a straw man as a CPU
+ * baseline.  The *_blocked routines below produce THE SAME VALUES (same
+ * operands, same k-ascending accumulation with one fused multiply-add per
+ * term in fp32, exact int32 sums for int8) with the work organised the way a
+ * CPU GEMM is: per expert the selected rows of A are decoded once, each
+ * thread owns a block of BLK_N output columns, decodes a BLK_K x BLK_N panel
+ * of the expert's weights once and runs a 4 x 16 register tile over it.
+ * pinned by: equality with orc_mx_gmm / orc_gemm_i8_dequant /
+ *            orc_gmm_i8_dequant_swiglu on ragged shapes, both layouts, all
+ *            payload formats (tests/test_oracle_blocked.py).
+ */
+#define BLK_N 128
+#define BLK_K 256
+typedef float vf8 __attribute__((vector_size(32), aligned(4)));
+typedef int32_t vi8 __attribute__((vector_size(32), aligned(4)));
+
+/* selected output indices ordered by expert: order[start[e] .. start[e+1]) */
+static void rows_by_expert(const int64_t *row_expert, const int64_t *rows, int64_t nrows, int64_t E,
+                           int64_t *start, int64_t *order)
+{
+    for (int64_t e = 0; e <= E; e++) start[e] = 0;
+    for (int64_t i = 0; i < nrows; i++) {
+        int64_t e = row_expert[rows ? rows[i] : i];
+        if (e >= 0) start[e + 1]++;
+    }
+    for (int64_t e = 0; e < E; e++) start[e + 1] += start[e];
+    int64_t *fill = (int64_t *)malloc((size_t)(E + 1) * 8);
+    memcpy(fill, start, (size_t)(E + 1) * 8);
+    for (int64_t i = 0; i < nrows; i++) {
+        int64_t e = row_expert[rows ? rows[i] : i];
+        if (e >= 0) order[fill[e]++] = i;
+    }
+    free(fill);
+}
+
+/* c[cnt][BLK_N] += a[cnt][lda] (columns k0..k0+kc) x panel[kc][BLK_N], fp32, k ascending */
+static void tile_f32(const float *a, int64_t lda, int64_t cnt, const float *panel, int64_t kc, float *c)
+{
+    int64_t r = 0;
+    for (; r + 4 <= cnt; r += 4)
+        for (int64_t n0 = 0; n0 < BLK_N; n0 += 16) {
+            vf8 acc[4][2];
+            for (int i = 0; i < 4; i++)
+                for (int h = 0; h < 2; h++) acc[i][h] = *(const vf8 *)(c + (r + i) * BLK_N + n0 + 8 * h);
+            for (int64_t k = 0; k < kc; k++) {
+                const vf8 b0 = *(const vf8 *)(panel + k * BLK_N + n0), b1 = *(const vf8 *)(panel + k * BLK_N + n0 + 8);
+                for (int i = 0; i < 4; i++) {
+                    const float av = a[(r + i) * lda + k];
+                    const vf8 a8 = {av, av, av, av, av, av, av, av};
+                    acc[i][0] += a8 * b0;
+                    acc[i][1] += a8 * b1;
+                }
+            }
+            for (int i = 0; i < 4; i++)
+                for (int h = 0; h < 2; h++) *(vf8 *)(c + (r + i) * BLK_N + n0 + 8 * h) = acc[i][h];
+        }
+    for (; r < cnt; r++)
+        for (int64_t n0 = 0; n0 < BLK_N; n0 += 8) {
+            vf8 acc = *(const vf8 *)(c + r * BLK_N + n0);
+            for (int64_t k = 0; k < kc; k++) {
+                const float av = a[r * lda + k];
+                const vf8 a8 = {av, av, av, av, av, av, av, av};
+                acc += a8 * *(const vf8 *)(panel + k * BLK_N + n0);
+            }
+            *(vf8 *)(c + r * BLK_N + n0) = acc;
+        }
+}
+
+static void tile_i32(const int32_t *a, int64_t lda, int64_t cnt, const int32_t *panel, int64_t kc, int32_t *c)
+{
+    int64_t r = 0;
+    for (; r + 4 <= cnt; r += 4)
+        for (int64_t n0 = 0; n0 < BLK_N; n0 += 16) {
+            vi8 acc[4][2];
+            for (int i = 0; i < 4; i++)
+                for (int h = 0; h < 2; h++) acc[i][h] = *(const vi8 *)(c + (r + i) * BLK_N + n0 + 8 * h);
+            for (int64_t k = 0; k < kc; k++) {
+                const vi8 b0 = *(const vi8 *)(panel + k * BLK_N + n0), b1 = *(const vi8 *)(panel + k * BLK_N + n0 + 8);
+                for (int i = 0; i < 4; i++) {
+                    const int32_t av = a[(r + i) * lda + k];
+                    const vi8 a8 = {av, av, av, av, av, av, av, av};
+                    acc[i][0] += a8 * b0;
+                    acc[i][1] += a8 * b1;
+                }
+            }
+            for (int i = 0; i < 4; i++)
+                for (int h = 0; h < 2; h++) *(vi8 *)(c + (r + i) * BLK_N + n0 + 8 * h) = acc[i][h];
+        }
+    for (; r < cnt; r++)
+        for (int64_t n = 0; n < BLK_N; n++) {
+            int32_t s = c[r * BLK_N + n];
+            for (int64_t k = 0; k < kc; k++) s += a[r * lda + k] * panel[k * BLK_N + n];
+            c[r * BLK_N + n] = s;
+        }
+}
+
+/* Same arguments and results as orc_mx_gmm (without the fp64 copy). */
+void orc_mx_gmm_blocked(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb,
+                        const int32_t *group_sizes, int64_t E, int64_t T, int64_t N, int64_t K, int fmt, int trans_b,
+                        const int64_t *rows, int64_t nrows, float *out_f32, uint16_t *out_bf16)
+{
+    const int fp4 = fmt == ORC_FMT_E2M1;
+    const int64_t nblk = (K + 31) / 32;
+    const int64_t sld = ((nblk + 1) / 2) * 2;
+    const int64_t b_bytes = fp4 ? (trans_b ? N * ((K + 1) / 2) : K * ((N + 1) / 2)) : K * N;
+    const int64_t sb_bytes = sld * N;
+    int64_t *row_expert = (int64_t *)malloc((size_t)(T > 0 ? T : 1) * 8);
+    if (group_sizes) {
+        int64_t r = 0;
+        for (int64_t e = 0; e < E; e++)
+            for (int32_t i = 0; i < group_sizes[e] && r < T; i++) row_expert[r++] = e;
+        for (; r < T; r++) row_expert[r] = -1;
+    } else {
+        for (int64_t r = 0; r < T; r++) row_expert[r] = 0;
+    }
+    if (!rows) nrows = T;
+    int64_t *start = (int64_t *)malloc((size_t)(E + 1) * 8);
+    int64_t *order = (int64_t *)malloc((size_t)(nrows > 0 ? nrows : 1) * 8);
+    rows_by_expert(row_expert, rows, nrows, E, start, order);
+    /* rows that belong to no group are zero */
+    for (int64_t i = 0; i < nrows; i++)
+        if (row_expert[rows ? rows[i] : i] < 0)
+            for (int64_t n = 0; n < N; n++) {
+                if (out_f32) out_f32[i * N + n] = 0.0f;
+                if (out_bf16) out_bf16[i * N + n] = 0;
+            }
+    const int64_t ncb = (N + BLK_N - 1) / BLK_N;
+    for (int64_t e = 0; e < E; e++) {
+        const int64_t cnt = start[e + 1] - start[e];
+        if (cnt == 0) continue;
+        const int64_t *ord = order + start[e];
+        const uint8_t *be = b + e * b_bytes;
+        const uint8_t *sbe = sb + e * sb_bytes;
+        float *adeq = (float *)malloc((size_t)cnt * K * 4);
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < cnt; i++) {
+            const int64_t m = rows ? rows[ord[i]] : ord[i];
+            for (int64_t k = 0; k < K; k++)
+                adeq[i * K + k] = orc_decode(payload_at(a, K, m, k, fp4), fmt) * orc_e8m0_decode(sa[m * sld + k / 32]);
+        }
+#pragma omp parallel
+        {
+            float *panel = (float *)malloc((size_t)BLK_K * BLK_N * 4);
+            float *c = (float *)malloc((size_t)cnt * BLK_N * 4);
+#pragma omp for schedule(dynamic, 1)
+            for (int64_t cb = 0; cb < ncb; cb++) {
+                const int64_t n0 = cb * BLK_N, nc = N - n0 < BLK_N ? N - n0 : BLK_N;
+                memset(c, 0, (size_t)cnt * BLK_N * 4);
+                for (int64_t k0 = 0; k0 < K; k0 += BLK_K) {
+                    const int64_t kc = K - k0 < BLK_K ? K - k0 : BLK_K;
+                    for (int64_t kk = 0; kk < kc; kk++) {
+                        const int64_t k = k0 + kk, kb = k / 32;
+                        float *prow = panel + kk * BLK_N;
+                        for (int64_t j = 0; j < nc; j++) {
+                            const int64_t n = n0 + j;
+                            prow[j] = trans_b ? orc_decode(payload_at(be, K, n, k, fp4), fmt) * orc_e8m0_decode(sbe[n * sld + kb])
+                                              : orc_decode(payload_at(be, N, k, n, fp4), fmt) *
+                                                    orc_e8m0_decode(sbe[(kb >> 1) * N * 2 + n * 2 + (kb & 1)]);
+                        }
+                        for (int64_t j = nc; j < BLK_N; j++) prow[j] = 0.0f;
+                    }
+                    tile_f32(adeq + k0, K, cnt, panel, kc, c);
+                }
+                for (int64_t i = 0; i < cnt; i++)
+                    for (int64_t j = 0; j < nc; j++) {
+                        if (out_f32) out_f32[ord[i] * N + n0 + j] = c[i * BLK_N + j];
+                        if (out_bf16) out_bf16[ord[i] * N + n0 + j] = orc_f32_to_bf16(c[i * BLK_N + j]);
+                    }
+            }
+            free(panel);
+            free(c);
+        }
+        free(adeq);
+    }
+    free(order); free(start); free(row_expert);
+}
+
+/* int8 x int8 -> int32 for the selected rows of one expert (or of the dense problem): acc[cnt][N] */
+static void i8_expert_blocked(const int8_t *x, const int8_t *w, int64_t N, int64_t K, int trans_b, const int64_t *rows,
+                              const int64_t *ord, int64_t cnt, int32_t *acc)
+{
+    int32_t *a32 = (int32_t *)malloc((size_t)cnt * K * 4);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < cnt; i++) {
+        const int64_t m = rows ? rows[ord[i]] : ord[i];
+        for (int64_t k = 0; k < K; k++) a32[i * K + k] = x[m * K + k];
+    }
+    const int64_t ncb = (N + BLK_N - 1) / BLK_N;
+#pragma omp parallel
+    {
+        int32_t *panel = (int32_t *)malloc((size_t)BLK_K * BLK_N * 4);
+        int32_t *c = (int32_t *)malloc((size_t)cnt * BLK_N * 4);
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t cb = 0; cb < ncb; cb++) {
+            const int64_t n0 = cb * BLK_N, nc = N - n0 < BLK_N ? N - n0 : BLK_N;
+            memset(c, 0, (size_t)cnt * BLK_N * 4);
+            for (int64_t k0 = 0; k0 < K; k0 += BLK_K) {
+                const int64_t kc = K - k0 < BLK_K ? K - k0 : BLK_K;
+                for (int64_t kk = 0; kk < kc; kk++) {
+                    int32_t *prow = panel + kk * BLK_N;
+                    for (int64_t j = 0; j < nc; j++) prow[j] = trans_b ? w[(n0 + j) * K + k0 + kk] : w[(k0 + kk) * N + n0 + j];
+                    for (int64_t j = nc; j < BLK_N; j++) prow[j] = 0;
+                }
+                tile_i32(a32 + k0, K, cnt, panel, kc, c);
+            }
+            for (int64_t i = 0; i < cnt; i++)
+                for (int64_t j = 0; j < nc; j++) acc[i * N + n0 + j] = c[i * BLK_N + j];
+        }
+        free(panel);
+        free(c);
+    }
+    free(a32);
+}
+
+/* Same arguments and results as orc_gemm_i8_dequant. */
+void orc_gemm_i8_dequant_blocked(const int8_t *a, const int8_t *b, const float *per_tok, const float *per_ch,
+                                 int64_t M, int64_t N, int64_t K, int trans_b, const int64_t *rows, int64_t nrows,
+                                 float *out_f32, uint16_t *out_bf16)
+{
+    if (!rows) nrows = M;
+    int64_t *ord = (int64_t *)malloc((size_t)(nrows > 0 ? nrows : 1) * 8);
+    for (int64_t i = 0; i < nrows; i++) ord[i] = i;
+    int32_t *acc = (int32_t *)malloc((size_t)(nrows > 0 ? nrows : 1) * N * 4);
+    i8_expert_blocked(a, b, N, K, trans_b, rows, ord, nrows, acc);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < nrows; i++) {
+        const int64_t m = rows ? rows[i] : i;
+        for (int64_t n = 0; n < N; n++) {
+            float v = (float)acc[i * N + n] * per_tok[m] * per_ch[n];
+            if (out_f32) out_f32[i * N + n] = v;
+            if (out_bf16) out_bf16[i * N + n] = orc_f32_to_bf16(v);
+        }
+    }
+    free(acc); free(ord);
+}
+
+/* Same arguments and results as orc_gmm_i8_dequant_swiglu. */
+void orc_gmm_i8_dequant_swiglu_blocked(const int8_t *x, const int8_t *w, const int32_t *group_sizes, int64_t E,
+                                       int64_t T, int64_t K, int64_t N, const float *per_tok, const float *per_ch,
+                                       int fp16_step, const int64_t *rows, int64_t nrows, float *out_f32,
+                                       uint16_t *out_bf16)
+{
+    const int64_t H = N / 2;
+    int64_t *row_expert = (int64_t *)malloc((size_t)(T > 0 ? T : 1) * 8);
+    int64_t r = 0;
+    for (int64_t e = 0; e < E; e++)
+        for (int32_t i = 0; i < group_sizes[e] && r < T; i++) row_expert[r++] = e;
+    for (; r < T; r++) row_expert[r] = -1;
+    if (!rows) nrows = T;
+    int64_t *start = (int64_t *)malloc((size_t)(E + 1) * 8);
+    int64_t *order = (int64_t *)malloc((size_t)(nrows > 0 ? nrows : 1) * 8);
+    rows_by_expert(row_expert, rows, nrows, E, start, order);
+    for (int64_t i = 0; i < nrows; i++)
+        if (row_expert[rows ? rows[i] : i] < 0)
+            for (int64_t j = 0; j < H; j++) {
+                if (out_f32) out_f32[i * H + j] = 0.0f;
+                if (out_bf16) out_bf16[i * H + j] = 0;
+            }
+    for (int64_t e = 0; e < E; e++) {
+        const int64_t cnt = start[e + 1] - start[e];
+        if (cnt == 0) continue;
+        const int64_t *ord = order + start[e];
+        int32_t *acc = (int32_t *)malloc((size_t)cnt * N * 4);
+        i8_expert_blocked(x, w + e * K * N, N, K, 0, rows, ord, cnt, acc);
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < cnt; i++) {
+            const int64_t m = rows ? rows[ord[i]] : ord[i];
+            for (int64_t j = 0; j < H; j++) {
+                float g = (float)acc[i * N + j] * per_ch[e * N + j];
+                float u = (float)acc[i * N + j + H] * per_ch[e * N + j + H];
+                if (fp16_step) { g = f32_to_f16_to_f32(g); u = f32_to_f16_to_f32(u); }
+                g *= per_tok[m];
+                u *= per_tok[m];
+                float v = g * sigmoidf_(g) * u;
+                if (out_f32) out_f32[ord[i] * H + j] = v;
+                if (out_bf16) out_bf16[ord[i] * H + j] = orc_f32_to_bf16(v);
+            }
+        }
+        free(acc);
+    }
+    free(order); free(start); free(row_expert);
+}
+
 /* ---------------------------------------------- token-count prefix sums */
 
 /* comm_block_scheduler_alltoallv_gmm.hpp:113-121: rows that source core

@@ -184,7 +184,7 @@ def test_mx_gemm_scale_extremes():
 
 # ---------------------------------------------------------------- MX grouped
 
-@pytest.mark.parametrize("fmt", ["e4m3", "e2m1"])
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
 @pytest.mark.parametrize("cfg", [(4, 1024, 256, 256, None), (5, 900, 512, 384, [0, 300, 1, 0, 500]), (32, 4096, 512, 512, None)])
 @pytest.mark.parametrize("trans_b", [0, 1])
 def test_mx_gmm(fmt, cfg, trans_b, path):
@@ -263,8 +263,40 @@ def test_mx_gemm_tiled(fmt, shape, trans_b, tiled_only):
     assert_close(got, want, ("mx tiled", fmt, shape, trans_b))
 
 
-@pytest.mark.parametrize("fmt", ["e4m3", "e2m1"])
-@pytest.mark.parametrize("cfg", [(5, 900, 1024, 416, [0, 300, 1, 0, 500]), (8, 3000, 768, 1056, None)])
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
+@pytest.mark.parametrize("trans_b", [0, 1])
+@pytest.mark.parametrize("shape", _reference_shapes("ascend950_mxfp8_matmul_reduce_scatter"))
+def test_mx_gemm_reference_shape_list_tiled(shape, trans_b, fmt, tiled_only):
+    """Every (M, K, N) of the reference's MXFP8 list (K = 1216, 960 and 1984 end inside a 128-byte step
+    and their scale rows start 2 bytes past a 4-byte boundary; K = 128 is a single step) on the MFMA
+    path - a fall-back is an error here - in both layouts of B, and with the FP4 and E5M2 payloads at
+    the same shapes."""
+    m, k, n = shape
+    rng = np.random.default_rng(m + k + n + trans_b)
+    pa, sa, pb, sb = mx_operands(rng, m, n, k, fmt, trans_b, 0.02 if fmt == "e2m1" else 1.0)
+    want = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], trans_b)
+    got = out_f32(cc.mx_matmul(dev(pa), dev(sa), dev(pb), dev(sb), fmt, trans_b))
+    assert_close(got, want, (shape, trans_b, fmt))
+
+
+@pytest.mark.parametrize("trans_b", [0, 1])
+@pytest.mark.parametrize("shape", _reference_shapes("ascend950_mxfp8_matmul_reduce_scatter"))
+def test_i8_dequant_reference_mx_shapes_tiled(shape, trans_b, tiled_only):
+    """The int8 kernels at the same shapes (K tails of 64 and 96 bytes, a single K step)."""
+    m, k, n = shape
+    rng = np.random.default_rng(m + k + n + 17 * trans_b)
+    a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    pt = rng.uniform(0.001, 0.02, m).astype(np.float32)
+    pc = rng.uniform(0.001, 0.02, n).astype(np.float32)
+    want = orc.gemm_i8_dequant(a, b, pt, pc)
+    bb = np.ascontiguousarray(b.T) if trans_b else b
+    got = out_f32(cc.w8a8_matmul_dequant(dev(a), dev(bb), dev(pt), dev(pc), trans_b))
+    assert_close(got, want, ("i8 tiled", shape, trans_b))
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
+@pytest.mark.parametrize("cfg", [(5, 900, 1024, 416, [0, 300, 1, 0, 500]), (8, 3000, 768, 1056, None), (6, 1500, 1216, 520, None)])
 @pytest.mark.parametrize("trans_b", [0, 1])
 def test_mx_gmm_tiled(fmt, cfg, trans_b, tiled_only):
     e, t, k, n, gs = cfg
@@ -492,14 +524,12 @@ def test_grouped_tile_order_covers_every_tile_once():
     outs = {}
     cc.set_option("require_tiled_gemm", 1)
     try:
-        for order in (0, 1, -1, 2, 3):
-            # 2: the default order again, with a balanced count of workgroups taking tiles instead of every CU
-            # 3: the default order without non-temporal weight requests (3 as threshold: with them for every
-            #    expert of up to three row tiles; the default is one)
-            cc.set_option("gemm_balance_rounds", 1 if order == 2 else 0)
-            cc.set_option("gemm_nt_small_experts", 3 if order == 3 else 0 if order == 0 else 1)
-            cc.set_option("gemm_nt_output", 1 if order == 3 else 0 if order == 0 else -1)
-            cc.set_option("gemm_tile_order", -1 if order >= 2 else order)
+        for order in (0, 1, 2, -1, 3, 4):
+            # 3: the default order again, with a balanced count of workgroups taking tiles instead of every CU
+            # 4: the default order with non-temporal output stores
+            cc.set_option("gemm_balance_rounds", 1 if order == 3 else 0)
+            cc.set_option("gemm_nt_output", 1 if order == 4 else 0 if order == 0 else -1)
+            cc.set_option("gemm_tile_order", -1 if order >= 3 else order)
             # the output starts as NaN: a tile that no workgroup computes would keep it
             out = torch.full((t, n), float("nan"), dtype=torch.bfloat16, device="cuda")
             cc.mx_grouped_matmul_mapped(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), dev(ident), out, "e4m3", 0)
@@ -507,11 +537,11 @@ def test_grouped_tile_order_covers_every_tile_once():
     finally:
         cc.set_option("gemm_tile_order", -1)
         cc.set_option("gemm_balance_rounds", 0)
-        cc.set_option("gemm_nt_small_experts", 1)
         cc.set_option("gemm_nt_output", -1)
         cc.set_option("require_tiled_gemm", 0)
     assert not np.isnan(outs[1]).any()
-    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[-1]) and np.array_equal(outs[1], outs[2]) and np.array_equal(outs[1], outs[3])
+    for order in (1, 2, -1, 3, 4):
+        assert np.array_equal(outs[0], outs[order]), order
     assert_close(outs[1], gold, "per-XCD tile order")
 
 

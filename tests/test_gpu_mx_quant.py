@@ -112,8 +112,8 @@ def test_hardware_cast_equals_integer_encoder():
     assert torch.equal(p1, p2) and torch.equal(s1, s2)
 
 
-def test_full_size_config1_properties_and_sampled_rows():
-    """[4096,7168] N(0,1) with 0.1% x100 outliers: sampled rows bit-exact, and the
+def test_full_size_config1_whole_tensor_and_properties():
+    """[4096,7168] N(0,1) with 0.1% x100 outliers: every byte of the whole tensor bit-exact, and the
     size-independent properties: re-quantising the dequantised tensor is the identity,
     doubling the input shifts every scale byte by one and leaves the payload unchanged."""
     m, k = 4096, 7168
@@ -121,9 +121,8 @@ def test_full_size_config1_properties_and_sampled_rows():
     xd = to_dev(x)
     p, s = cc.mx_quant(xd, "e4m3")
     torch.cuda.synchronize()
-    rows = np.random.default_rng(0).choice(m, 192, replace=False)
-    po, so = orc.mx_quant_rows(x[rows], orc.E4M3, orc.RNE)
-    assert np.array_equal(p.cpu().numpy()[rows], po) and np.array_equal(s.cpu().numpy()[rows], so)
+    po, so = orc.mx_quant_rows(x, orc.E4M3, orc.RNE)   # the whole tensor (the oracle takes well under a second)
+    assert np.array_equal(p.cpu().numpy(), po) and np.array_equal(s.cpu().numpy(), so)
     deq = p.view(torch.float8_e4m3fn).to(torch.float32) * torch.exp2(s.to(torch.float32) - 127).repeat_interleave(32, 1)
     p2, s2 = cc.mx_quant(deq.to(torch.bfloat16), "e4m3")
     assert torch.equal(p2, p) and torch.equal(s2, s)
