@@ -410,6 +410,15 @@ def main():
         tt4 = [queue_time_ms(lambda: cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), 30, 60.0)]
         extra["moe_w8a8_swiglu_cfg4"] = {"tops": round(2.0 * t4 * n4 * k4 / (np.mean(tt4) * 1e-3) / 1e12, 1), "us": round(float(np.mean(tt4)) * 1e3, 1)}
         extra["moe_w8a8_swiglu_cfg4"]["frac_of_int8_peak"] = round(extra["moe_w8a8_swiglu_cfg4"]["tops"] / FP8_PEAK_TFLOPS, 4)
+        # the same with the activation leaving as MXFP8 from the epilogue, against the two-kernel chain it replaces
+        tf4 = queue_time_ms(lambda: cc.gmm_dequant_swiglu_mx(x4, w4, gs4, pt4, pc4, TRANS_B, "e4m3"), 30, 60.0)
+        tc4 = queue_time_ms(lambda: cc.mx_quant(cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), "e4m3"), 30, 60.0)
+        pf4, sf4 = cc.gmm_dequant_swiglu_mx(x4, w4, gs4, pt4, pc4, TRANS_B, "e4m3")
+        pq4, sq4 = cc.mx_quant(cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), "e4m3")
+        extra["moe_w8a8_swiglu_mxfp8_out_cfg4"] = {"us": round(tf4 * 1e3, 1), "two_kernel_chain_us": round(tc4 * 1e3, 1),
+                                                   "tops": round(2.0 * t4 * n4 * k4 / (tf4 * 1e-3) / 1e12, 1),
+                                                   "parity": {"bit_exact_vs_quantised_bf16_output": bool(torch.equal(pf4, pq4) and torch.equal(sf4, sq4))}}
+        del pf4, sf4, pq4, sq4
         if cpu:
             o4 = cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B).float().cpu().numpy()
             h4 = [t.cpu().numpy() for t in (x4, w4, gs4, pt4, pc4)]

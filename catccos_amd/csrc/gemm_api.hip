@@ -145,6 +145,37 @@ int cch_gmm_i8_dequant_swiglu_out(const void *x, const void *w, const int32_t *g
     return run(p, KIND_I8, EPI_DEQUANT_SWIGLU, static_cast<hipStream_t>(stream));
 }
 
+int cch_gmm_i8_dequant_swiglu_mx(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok,
+                                 const float *per_ch, void *payload, void *scales, int64_t num_experts, int64_t t, int64_t n,
+                                 int64_t k, int trans_b, int fmt, void *stream)
+{
+    int rc = check_shape("cch_gmm_i8_dequant_swiglu_mx", t, n, k);
+    if (rc) return rc;
+    CCH_REQUIRE(fmt == CCH_FMT_E4M3 || fmt == CCH_FMT_E5M2 || fmt == CCH_FMT_E2M1, "cch_gmm_i8_dequant_swiglu_mx: fmt %d (E4M3, E5M2 or E2M1)", fmt);
+    CCH_REQUIRE(trans_b == 0 || trans_b == 1, "cch_gmm_i8_dequant_swiglu_mx: trans_b %d", trans_b);
+    CCH_REQUIRE(n % 2 == 0, "cch_gmm_i8_dequant_swiglu_mx: n=%lld must be even (gate | up halves)", (long long)n);
+    CCH_REQUIRE(fmt != CCH_FMT_E2M1 || n % 4 == 0, "cch_gmm_i8_dequant_swiglu_mx: n=%lld: FP4 rows hold two codes per byte", (long long)n);
+    CCH_REQUIRE(num_experts >= 1 && num_experts <= MAX_GROUPS, "cch_gmm_i8_dequant_swiglu_mx: num_experts=%lld outside 1..%d", (long long)num_experts, MAX_GROUPS);
+    if (t == 0 || n == 0) return CCH_OK;
+    CCH_REQUIRE(payload && scales && per_tok && per_ch && group_sizes && (k == 0 || (x && w)), "cch_gmm_i8_dequant_swiglu_mx: null pointer");
+    GemmProblem p{};
+    p.a = static_cast<const uint8_t *>(x);
+    p.b = static_cast<const uint8_t *>(w);
+    p.per_tok = per_tok;
+    p.per_ch = per_ch;
+    p.out = static_cast<uint16_t *>(payload);
+    p.out_scales = static_cast<uint8_t *>(scales);
+    p.mx_out = 1;
+    p.mx_out_fmt = fmt;
+    p.group_sizes = group_sizes;
+    p.num_groups = (int)num_experts;
+    p.T = (int)t; p.N = (int)n; p.K = (int)k; p.n_out = (int)(n / 2);
+    p.mx_out_sld = (int)(2 * ((p.n_out + 63) / 64));
+    p.trans_b = trans_b;
+    p.b_stride = n * k;
+    return run(p, KIND_I8, EPI_DEQUANT_SWIGLU, static_cast<hipStream_t>(stream));
+}
+
 int cch_gmm_i8_dequant(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok, const float *per_ch,
                        void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k, int trans_b, void *stream)
 {

@@ -25,6 +25,12 @@ struct GemmProblem {
     const int32_t *out_row_map;  // device int32[T] or nullptr: row of `out` that receives row i (negative: dropped)
     int64_t out_rows;        // rows of `out` when out_row_map is given
     int out_fp16;            // output elements are IEEE half instead of bf16 (both rounded to nearest even)
+    int mx_out;              // SwiGLU epilogue only: 1 = the activation leaves MX-quantised along its rows (what the
+                             // row quantiser would make of the bf16 output): payload [T, n_out] codes of format
+                             // mx_out_fmt at `out` (FP4: two per byte), E8M0 scales [T, mx_out_sld] at `out_scales`
+    int mx_out_fmt;          // CCH_FMT_E4M3, CCH_FMT_E5M2 or CCH_FMT_E2M1
+    int mx_out_sld;          // scale bytes per output row: 2*ceil(n_out/64), padding bytes are 127
+    uint8_t *out_scales;
     const int32_t *group_sizes;  // device int32[E] or nullptr (dense, E = 1)
     int num_groups;
     int T, N, K;             // K in elements

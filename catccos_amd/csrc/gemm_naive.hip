@@ -98,6 +98,52 @@ __global__ __launch_bounds__(256) void gemm_naive_kernel(GemmProblem p)
     p.out[out_row * p.n_out + col] = p.out_fp16 ? __builtin_bit_cast(uint16_t, (_Float16)v) : (uint16_t)f32_to_bf16_bits(v);
 }
 
+// The grouped int8 GEMM with dequantisation and SwiGLU whose activation leaves MX-quantised: what the
+// row quantiser makes of the bf16 output of the kernel above, without the bf16 tensor in between.
+// 32 neighbouring lanes hold one block of a row (the last block of a row may be shorter).
+template <int FMT>
+__global__ __launch_bounds__(256) void gemm_naive_swiglu_mx_kernel(GemmProblem p)
+{
+    using T = FmtTraits<FMT>;
+    __shared__ GroupTable tab;
+    if (threadIdx.x == 0) build_group_table(tab, p.group_sizes, p.num_groups, p.T, 1);
+    __syncthreads();
+    const int col = blockIdx.x * 256 + threadIdx.x;
+    const int row = blockIdx.y;
+    const bool live = col < p.n_out;
+    const int e = find_group(tab, p.num_groups, row);
+    float v = 0.0f;
+    if (live && e < p.num_groups) {
+        float g = dot_column<KIND_I8>(p, row, e, col) * p.per_ch[(size_t)e * p.N + col];
+        float u = dot_column<KIND_I8>(p, row, e, col + p.n_out) * p.per_ch[(size_t)e * p.N + col + p.n_out];
+        g *= p.per_tok[row];
+        u *= p.per_tok[row];
+        v = g * (1.0f / (1.0f + expf(-g))) * u;
+    }
+    const uint32_t h = live ? f32_to_bf16_bits(v) : 0u;
+    uint32_t amax = h & 0x7FFFu;
+#pragma unroll
+    for (int d = 1; d < 32; d <<= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, d, 32));
+    int ex;
+    bool is_nan;
+    const uint32_t sbyte = shared_exp_byte<FMT>(amax, ex, is_nan);
+    // 2^-ex in two exact factors (2^-127 is no normal float)
+    const float y = bf16_bits_to_f32(h) * pow2i(-min(ex, 126)) * (ex > 126 ? 0.5f : 1.0f);
+    const uint32_t code = is_nan ? T::NANCODE : encode_small<FMT, CCH_ROUND_RNE>(y);
+    uint8_t *payload = reinterpret_cast<uint8_t *>(p.out);
+    if constexpr (is_fp4_v<FMT>) {
+        const uint32_t hi = (uint32_t)__shfl_down((int)code, 1, 32);
+        if (live && (col & 1) == 0) payload[((size_t)row * p.n_out + col) >> 1] = (uint8_t)(code | ((col + 1 < p.n_out ? hi : 0u) << 4));
+    } else {
+        if (live) payload[(size_t)row * p.n_out + col] = (uint8_t)code;
+    }
+    if (live && (col & 31) == 0) {
+        p.out_scales[(size_t)row * p.mx_out_sld + (col >> 5)] = (uint8_t)sbyte;
+        const int nblk = (p.n_out + 31) >> 5;
+        if ((nblk & 1) && (col >> 5) == nblk - 1) p.out_scales[(size_t)row * p.mx_out_sld + nblk] = 127;
+    }
+}
+
 template <int KIND, int EPI>
 static int launch_naive_t(const GemmProblem &p, hipStream_t stream)
 {
@@ -110,6 +156,16 @@ static int launch_naive_t(const GemmProblem &p, hipStream_t stream)
 
 int launch_gemm_naive(const GemmProblem &p, int kind, int epi, hipStream_t stream)
 {
+    if (p.mx_out) {
+        if (kind != KIND_I8 || epi != EPI_DEQUANT_SWIGLU) return fail(CCH_ENOSUP, "MX-quantised output exists for the int8 SwiGLU epilogue only");
+        if (p.T == 0 || p.n_out == 0) return CCH_OK;
+        if (p.T > 65535) return fail(CCH_ENOSUP, "generic GEMM path takes at most 65535 rows per call (got %d)", p.T);
+        dim3 grid((unsigned)((p.n_out + 255) / 256), (unsigned)p.T);
+        if (p.mx_out_fmt == CCH_FMT_E4M3) hipLaunchKernelGGL((gemm_naive_swiglu_mx_kernel<CCH_FMT_E4M3>), grid, dim3(256), 0, stream, p);
+        else if (p.mx_out_fmt == CCH_FMT_E5M2) hipLaunchKernelGGL((gemm_naive_swiglu_mx_kernel<CCH_FMT_E5M2>), grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((gemm_naive_swiglu_mx_kernel<CCH_FMT_E2M1>), grid, dim3(256), 0, stream, p);
+        return launch_status("gemm_naive_swiglu_mx_kernel");
+    }
     if (kind == KIND_I8 && epi == EPI_DEQUANT) return launch_naive_t<KIND_I8, EPI_DEQUANT>(p, stream);
     if (kind == KIND_I8 && epi == EPI_DEQUANT_SWIGLU) return launch_naive_t<KIND_I8, EPI_DEQUANT_SWIGLU>(p, stream);
     if (kind == KIND_F8 && epi == EPI_PLAIN) return launch_naive_t<KIND_F8, EPI_PLAIN>(p, stream);

@@ -47,6 +47,7 @@
 #include "common.h"
 #include "gemm_common.h"
 #include "mx_formats.h"
+#include "mx_quant_block.h"
 
 namespace cch {
 
@@ -55,6 +56,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -335,11 +337,20 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     // examples/utils/gen_data_fp4_mx_alltoallv_gmm.py:788-790): all workgroups share the range,
     // 16 bytes per thread and pass; usually it is empty.
     const bool has_map = EPI == EPI_PLAIN && p.out_row_map != nullptr;   // rows go where the map says
+    const bool mx_out = SWIGLU && p.mx_out;
+    const int out_row_bytes = mx_out ? (p.mx_out_fmt == CCH_FMT_E2M1 ? p.n_out / 2 : p.n_out) : p.n_out * 2;
     if (p.group_sizes && !has_map) {
-        const size_t begin = (size_t)uniform(tab.row_start[p.num_groups]) * p.n_out / 8, end = (size_t)p.T * p.n_out / 8;
+        const int first = uniform(tab.row_start[p.num_groups]);
+        const size_t begin = (size_t)first * out_row_bytes / 16, end = (size_t)p.T * out_row_bytes / 16;
         v4u *o16 = reinterpret_cast<v4u *>(p.out);
         for (size_t i = begin + (size_t)blockIdx.x * TILE_THREADS + threadIdx.x; i < end; i += (size_t)gridDim.x * TILE_THREADS)
             o16[i] = (v4u){0, 0, 0, 0};
+        if (mx_out) {
+            // a block of zeros has the scale 2^0
+            const size_t sb0 = (size_t)first * p.mx_out_sld, sb1 = (size_t)p.T * p.mx_out_sld;
+            for (size_t i = sb0 + (size_t)blockIdx.x * TILE_THREADS + threadIdx.x; i < sb1; i += (size_t)gridDim.x * TILE_THREADS)
+                p.out_scales[i] = 127;
+        }
     }
 
     // Workgroups that take tiles: all of them, or (balance) just enough for the same number of
@@ -983,8 +994,8 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             // registers that the K loop needs.
             int lane_e = lane;
             asm volatile("" : "+v"(lane_e));
-            const __amdgpu_buffer_rsrc_t rs_out =
-                __builtin_amdgcn_make_buffer_rsrc(p.out + (has_map ? (size_t)0 : (size_t)cur.m0 * p.n_out), 0, 0x7FFFFFFF, 0x00020000);
+            const __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(
+                reinterpret_cast<uint8_t *>(p.out) + (has_map ? (size_t)0 : (size_t)cur.m0 * out_row_bytes), 0, 0x7FFFFFFF, 0x00020000);
             float chs[NT];
             if (EPI != EPI_PLAIN) {
 #pragma unroll
@@ -1045,6 +1056,43 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                         const int mapped = (int)lds_read4(prm + (uint32_t)row * 4u);
                         ok = ok && (!has_map || (mapped >= 0 && mapped < (int)p.out_rows));   // dropped or out of range: not written
                         out_row = has_map ? (uint32_t)mapped : out_row;
+                    }
+                    if constexpr (SWIGLU) {
+                        if (mx_out) {
+                            // The four lanes of a quad hold the 32 columns of one row that this wave owns:
+                            // one MX block.  Its maximum, shared exponent and codes as the row quantiser
+                            // makes them from the bf16 values.
+                            const uint32_t w[4] = {(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]};
+                            const uint32_t amax = block_amax_bits(w);
+                            uint32_t code[2], sbyte;
+                            int e;
+                            bool is_nan;
+                            if (p.mx_out_fmt == CCH_FMT_E2M1) {
+                                sbyte = shared_exp_byte<CCH_FMT_E2M1>(amax, e, is_nan);
+                                quant8_hw<CCH_FMT_E2M1>(w, e, is_nan, code);
+                            } else if (p.mx_out_fmt == CCH_FMT_E5M2) {
+                                sbyte = shared_exp_byte<CCH_FMT_E5M2>(amax, e, is_nan);
+                                quant8_hw<CCH_FMT_E5M2>(w, e, is_nan, code);
+                            } else {
+                                sbyte = shared_exp_byte<CCH_FMT_E4M3>(amax, e, is_nan);
+                                quant8_hw<CCH_FMT_E4M3>(w, e, is_nan, code);
+                            }
+                            const uint32_t elem = out_row * (uint32_t)p.n_out + (uint32_t)col;
+                            if (p.mx_out_fmt == CCH_FMT_E2M1)
+                                __builtin_amdgcn_raw_buffer_store_b32(code[0], rs_out, (int)(ok ? elem >> 1 : NO_FETCH), 0, 0);
+                            else
+                                __builtin_amdgcn_raw_buffer_store_b64((v2u){code[0], code[1]}, rs_out, (int)(ok ? elem : NO_FETCH), 0, 0);
+                            // the quad's first lane writes the block's scale, and behind the last block of a row
+                            // with an odd count of blocks the padding byte
+                            const __amdgpu_buffer_rsrc_t rs_sc_out = __builtin_amdgcn_make_buffer_rsrc(
+                                p.out_scales + (size_t)cur.m0 * p.mx_out_sld, 0, 0x7FFFFFFF, 0x00020000);
+                            const uint32_t blk = (uint32_t)col >> 5, soff = out_row * (uint32_t)p.mx_out_sld + blk;
+                            const bool first = ok && chunk == 0;
+                            __builtin_amdgcn_raw_buffer_store_b8((uint8_t)sbyte, rs_sc_out, (int)(first ? soff : NO_FETCH), 0, 0);
+                            if ((p.n_out & 32) != 0 && (int)blk == (p.n_out >> 5) - 1)
+                                __builtin_amdgcn_raw_buffer_store_b8((uint8_t)127, rs_sc_out, (int)(first ? soff + 1 : NO_FETCH), 0, 0);
+                            continue;
+                        }
                     }
                     const uint32_t off = ok ? (out_row * (uint32_t)p.n_out + (uint32_t)col) * 2u : NO_FETCH;
                     const v4u sv = (v4u){(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]};
@@ -1117,6 +1165,7 @@ const char *gemm_tile_unsupported(const GemmProblem &p, int kind, int epi)
     // rows are fetched in 16-byte pieces
     if (p.K < 1 || p.K % (16 * epb) != 0) return "K must be a multiple of 16 bytes per row";
     if (p.n_out % 8 != 0 || !aligned(p.out, 16)) return "output rows must take 16-byte stores (n_out % 8 == 0, out 16-byte aligned)";
+    if (p.mx_out && (epi != EPI_DEQUANT_SWIGLU || p.n_out % 32 != 0 || p.out_fp16)) return "MX-quantised output needs whole 32-column blocks";
     if ((int64_t)BM * p.n_out * 2 >= ((int64_t)1 << 31)) return "output row tile beyond 2 GiB";
     // mapped output rows are addressed from the start of `out` with 32-bit offsets
     if (p.out_row_map && (epi != EPI_PLAIN || p.out_rows * p.n_out * 2 >= ((int64_t)1 << 31) || !aligned(p.out_row_map, 4)))

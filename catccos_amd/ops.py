@@ -257,7 +257,14 @@ def gmm_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, trans_b=0, out_dtype=
     return _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, True, out_dtype)
 
 
-def _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, swiglu, out_dtype=torch.bfloat16):
+def gmm_dequant_swiglu_mx(x, w, group_sizes, per_tok, per_ch, trans_b=0, fmt="e4m3"):
+    """gmm_dequant_swiglu with the activation MX-quantised along its rows in the kernel's epilogue:
+    returns (payload uint8 [T, N/2] (FP4: [T, N/4]), scales uint8 [T, scale_cols(N/2)]), the same bytes
+    as mx_quant(gmm_dequant_swiglu(...), fmt)."""
+    return _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, True, torch.bfloat16, mx_fmt=_fmt(fmt))
+
+
+def _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, swiglu, out_dtype=torch.bfloat16, mx_fmt=None):
     code = _out_code(out_dtype)
     _require_gpu(x, w, group_sizes, per_tok, per_ch)
     _check_2d("x", x, torch.int8)
@@ -275,6 +282,15 @@ def _gmm_i8(x, w, group_sizes, per_tok, per_ch, trans_b, swiglu, out_dtype=torch
     per_ch = per_ch.contiguous().float()
     if per_tok.numel() != t or tuple(per_ch.shape) != (e, n):
         raise ValueError("per_tok must be [T] and per_ch [E,N]")
+    if mx_fmt is not None:
+        if n % 2 or (mx_fmt == FMT_E2M1 and n % 4):
+            raise ValueError("n must be even (a multiple of 4 for FP4 output)")
+        h = n // 2
+        payload = torch.empty((t, h // 2 if mx_fmt == FMT_E2M1 else h), dtype=torch.uint8, device=x.device)
+        scales = torch.empty((t, scale_cols(h)), dtype=torch.uint8, device=x.device)
+        check(_abi.lib().cch_gmm_i8_dequant_swiglu_mx(_ptr(x), _ptr(w), _ptr(group_sizes), _ptr(per_tok), _ptr(per_ch), _ptr(payload),
+                                                      _ptr(scales), e, t, n, k, int(trans_b), mx_fmt, _stream()))
+        return payload, scales
     out = torch.empty((t, n // 2 if swiglu else n), dtype=out_dtype, device=x.device)
     fn = _abi.lib().cch_gmm_i8_dequant_swiglu_out if swiglu else _abi.lib().cch_gmm_i8_dequant_out
     check(fn(_ptr(x), _ptr(w), _ptr(group_sizes), _ptr(per_tok), _ptr(per_ch), _ptr(out), e, t, n, k, int(trans_b), code,

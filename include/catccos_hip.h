@@ -144,6 +144,19 @@ int cch_gmm_i8_dequant_swiglu(const void *x, const void *w, const int32_t *group
 int cch_gmm_i8_dequant_swiglu_out(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok,
                                   const float *per_ch, void *out, int64_t num_experts, int64_t t, int64_t n, int64_t k,
                                   int trans_b, int out_dtype, void *stream);
+/* The same with the activation leaving MX-quantised along its rows instead of as bf16: what
+ * cch_mx_quant_rows (round to nearest even) makes of the bf16 output above, bit for bit, without the
+ * bf16 tensor in between - the reference's SwiGLU-from-UB stage followed by its MX quantiser
+ * (examples/aux_ops/ascend950_swiglu_from_ub.h:216-389,
+ * include/catccos/comm/block/comm_block_mx_quant.hpp:213-266), as the input of the down-projection
+ * MX grouped matmul.
+ *   payload: codes of `fmt` (CCH_FMT_E4M3, CCH_FMT_E5M2; CCH_FMT_E2M1 two per byte), [t, n/2] elements;
+ *   scales:  E8M0 [t, 2*ceil(n/2/64)], one per 32 columns, padding bytes 127.
+ * Rows past sum(group_sizes) hold zero codes and scale bytes 127.  The tiled kernels take it when n/2 is
+ * a multiple of 32 (besides their other conditions); other shapes run on the generic kernels. */
+int cch_gmm_i8_dequant_swiglu_mx(const void *x, const void *w, const int32_t *group_sizes, const float *per_tok,
+                                 const float *per_ch, void *payload, void *scales, int64_t num_experts, int64_t t, int64_t n,
+                                 int64_t k, int trans_b, int fmt, void *stream);
 
 /* ---- MX (FP8 / FP4 payload, E8M0 scales) dense GEMM (config 3) ---------------
  * Replaces the compute half of MatmulReduceScatterMxTla::operator()<AIC>

@@ -1,0 +1,94 @@
+"""The grouped int8 matmul + dequant + SwiGLU whose activation leaves MX-quantised from the kernel's
+epilogue: its bytes must equal the oracle's row quantiser applied to the bf16 tensor that the unfused
+entry point writes, bit for bit (payload and scales, padding bytes, rows that belong to no group)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+import catccos_amd as cc
+
+pytestmark = pytest.mark.gpu
+FMT = {"e4m3": orc.E4M3, "e5m2": orc.E5M2, "e2m1": orc.E2M1}
+
+
+def bits(t):
+    torch.cuda.synchronize()
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def case(e, t, k, n, gs, seed):
+    rng = np.random.default_rng(seed)
+    x = torch.from_numpy(rng.integers(-127, 128, (t, k)).astype(np.int8)).cuda()
+    w = rng.integers(-127, 128, (e, k, n)).astype(np.int8)
+    pt = torch.from_numpy(rng.uniform(0.001, 0.02, t).astype(np.float32)).cuda()
+    # a wide range of channel scales, so that blocks differ in their shared exponents
+    pc = torch.from_numpy((rng.uniform(0.001, 0.02, (e, n)) * 2.0 ** rng.integers(-6, 3, (e, n))).astype(np.float32)).cuda()
+    return x, w, pt, pc, torch.from_numpy(np.array(gs, np.int32)).cuda()
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
+@pytest.mark.parametrize("trans_b", [0, 1])
+@pytest.mark.parametrize("cfg", [(4, 700, 512, 1088, [300, 0, 143, 250]),     # n/2 = 544: 17 blocks (odd: a padding byte), 7 rows of no group
+                                 (3, 300, 256, 512, [1, 0, 299]),
+                                 (6, 2000, 768, 2048, [700, 13, 0, 256, 900, 131])])
+def test_fused_bytes_equal_quantised_bf16_tiled(fmt, trans_b, cfg):
+    e, t, k, n, gs = cfg
+    x, w, pt, pc, gsd = case(e, t, k, n, gs, seed=t + k + trans_b)
+    wd = torch.from_numpy(np.ascontiguousarray(w.transpose(0, 2, 1)) if trans_b else w).cuda()
+    cc.set_option("require_tiled_gemm", 1)
+    try:
+        plain = cc.gmm_dequant_swiglu(x, wd, gsd, pt, pc, trans_b)
+        pay, sc = cc.gmm_dequant_swiglu_mx(x, wd, gsd, pt, pc, trans_b, fmt)
+    finally:
+        cc.set_option("require_tiled_gemm", 0)
+    want_p, want_s = orc.mx_quant_rows(bits(plain), FMT[fmt])
+    assert np.array_equal(sc.cpu().numpy(), want_s)
+    assert np.array_equal(pay.cpu().numpy(), want_p)
+    # and the device's own row quantiser agrees (the same bytes by another kernel)
+    p2, s2 = cc.mx_quant(plain, fmt)
+    assert torch.equal(p2, pay) and torch.equal(s2, sc)
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e2m1"])
+@pytest.mark.parametrize("trans_b", [0, 1])
+def test_fused_bytes_generic_path_and_ragged_blocks(fmt, trans_b):
+    """n/2 = 100: three whole blocks and one of four columns, outside what the tiled kernels take."""
+    e, t, k, n, gs = 3, 70, 96, 200, [30, 0, 33]
+    x, w, pt, pc, gsd = case(e, t, k, n, gs, seed=5 + trans_b)
+    wd = torch.from_numpy(np.ascontiguousarray(w.transpose(0, 2, 1)) if trans_b else w).cuda()
+    plain = cc.gmm_dequant_swiglu(x, wd, gsd, pt, pc, trans_b)
+    pay, sc = cc.gmm_dequant_swiglu_mx(x, wd, gsd, pt, pc, trans_b, fmt)
+    want_p, want_s = orc.mx_quant_rows(bits(plain), FMT[fmt])
+    assert np.array_equal(sc.cpu().numpy(), want_s)
+    assert np.array_equal(pay.cpu().numpy(), want_p)
+
+
+def test_fused_generic_equals_oracle_chain():
+    """Generic kernels at a tiled-capable shape against the oracle end to end: oracle GEMM + SwiGLU to bf16,
+    then the oracle's quantiser (the generic kernel's exp and division are the IEEE ones; a one-ulp bf16
+    difference from the oracle's libm moves at most that element's code by one step)."""
+    e, t, k, n, gs = 2, 96, 128, 256, [40, 56]
+    x, w, pt, pc, gsd = case(e, t, k, n, gs, seed=77)
+    cc.set_option("force_generic_gemm", 1)
+    try:
+        pay, sc = cc.gmm_dequant_swiglu_mx(x, torch.from_numpy(w).cuda(), gsd, pt, pc, 0, "e4m3")
+    finally:
+        cc.set_option("force_generic_gemm", 0)
+    _, gold16 = orc.gmm_i8_dequant_swiglu(x.cpu().numpy(), w, np.array(gs, np.int32), pt.cpu().numpy(), pc.cpu().numpy(), want_bf16=True)
+    want_p, want_s = orc.mx_quant_rows(gold16, orc.E4M3)
+    got = orc.mx_dequant_rows(pay.cpu().numpy(), sc.cpu().numpy(), n // 2, orc.E4M3)
+    want = orc.mx_dequant_rows(want_p, want_s, n // 2, orc.E4M3)
+    assert np.mean(sc.cpu().numpy() == want_s) > 0.99
+    assert np.mean(pay.cpu().numpy() == want_p) > 0.99
+    m = orc.compare(got, want)
+    assert m["max_rel_floor_rms"] <= 0.15, m   # one code step of E4M3 is 1/8 relative
+
+
+def test_bad_arguments():
+    x, w, pt, pc, gsd = case(2, 8, 32, 64, [4, 4], seed=1)
+    wd = torch.from_numpy(w).cuda()
+    with pytest.raises(ValueError):
+        cc.gmm_dequant_swiglu_mx(x, wd, gsd, pt, pc, 0, "e1m2x")
+    with pytest.raises(cc.CatccosError):
+        cc.gmm_dequant_swiglu_mx(x, wd, gsd, pt, pc, 0, "e1m2")
