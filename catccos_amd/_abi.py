@@ -35,6 +35,7 @@ PROTOTYPES = {
     "cch_mx_quant_rows_f16": [_P, _P, _P, _I64, _I64, _I, _I, _P],
     "cch_mx_quant_b": [_P, _P, _P, _I64, _I64, _I, _I, _I, _P],
     "cch_mx_quant_scatter_packed": [_P, _P, _P, _I64, _I64, _I, _I, _I, _P],
+    "cch_mx_quant_scatter_packed_rows": [_P, _P, _P, _I64, _I64, _I64, _I, _I, _I, _P],
     "cch_moe_token_unpermute": [_P, _P, _P, _P, _I64, _I64, _I64, _I, _P],
     "cch_moe_init_routing_workspace_bytes": [_I64, _I],
     "cch_moe_init_routing": [_P, _I64, _I, _P, _P, _P, _I, _P, _I64, _P],

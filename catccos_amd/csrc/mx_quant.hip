@@ -39,7 +39,7 @@ template <int FMT, int RND, bool HWCVT, bool VEC, bool PAIR, bool SCATTER = fals
 __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
     const uint16_t *__restrict__ x, uint8_t *__restrict__ payload, uint8_t *__restrict__ scales, int rows, int K,
     int nblk, int sld, int pld, int wpr, int total_ws, const int32_t *__restrict__ dst_idx = nullptr, int topk = 1,
-    int sstride = 0)
+    int sstride = 0, int out_rows = 0x7FFFFFFF)
 {
     static_assert(!(SCATTER && PAIR), "the scatter variant stores one wave-step at a time");
     if (!SCATTER) sstride = sld;
@@ -63,8 +63,10 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
             bt.w[u][0] = bt.w[u][1] = bt.w[u][2] = bt.w[u][3] = 0;
             if constexpr (SCATTER) {
 #pragma unroll
-                for (int t = 0; t < QUANT_MAX_TOPK; t++)
+                for (int t = 0; t < QUANT_MAX_TOPK; t++) {
                     bt.dst[u][t] = (bt.row[u] >= 0 && t < topk) ? dst_idx[(size_t)bt.row[u] * topk + t] : -1;
+                    if (bt.dst[u][t] >= out_rows) bt.dst[u][t] = -1;   // a row past the output is skipped like a negative one
+                }
             }
             if (bt.row[u] >= 0 && bt.k0[u] < K) {
                 const uint16_t *src = x + (size_t)bt.row[u] * K + bt.k0[u];
@@ -205,10 +207,12 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_kernel(
 // of the pair as dwords gathered with row shifts.
 // SCATTER: as in mx_quant_rows_kernel, the row goes to rows dst_idx[r*topk + 0 .. topk-1]; `sld`
 // is then the distance between scale rows of the packed output.
-template <int FMT, bool SCATTER = false>
+// HALF: the input is IEEE half instead of bf16 (same layout, same stores; the shared exponent comes
+// from the block maximum widened to fp32 and the codes from the packed-half conversions).
+template <int FMT, bool SCATTER = false, bool HALF = false>
 __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_fast_kernel(
     const uint16_t *__restrict__ x, uint8_t *__restrict__ payload, uint8_t *__restrict__ scales, int K, int sld, int pld,
-    int ppr, int npairs, const int32_t *__restrict__ dst_idx = nullptr, int topk = 1)
+    int ppr, int npairs, const int32_t *__restrict__ dst_idx = nullptr, int topk = 1, int out_rows = 0x7FFFFFFF)
 {
     constexpr bool FP4 = is_fp4_v<FMT>;
     const int lane = threadIdx.x & 63;
@@ -226,7 +230,10 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_fast_kernel(
         v[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 512));
         if constexpr (SCATTER) {
 #pragma unroll
-            for (int t = 0; t < QUANT_MAX_TOPK; t++) d.row[t] = t < topk ? dst_idx[(size_t)r * topk + t] : -1;
+            for (int t = 0; t < QUANT_MAX_TOPK; t++) {
+                d.row[t] = t < topk ? dst_idx[(size_t)r * topk + t] : -1;
+                if (d.row[t] >= out_rows) d.row[t] = -1;   // a row past the output is skipped like a negative one
+            }
         }
     };
     auto convert = [&](int p, const u32x4 (&v)[2], const Dest &d) {
@@ -235,11 +242,19 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_fast_kernel(
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             const uint32_t w[4] = {v[h][0], v[h][1], v[h][2], v[h][3]};
-            const uint32_t amax_bits = block_amax_bits(w);
+            const uint32_t amax_bits = block_amax_bits(w);   // |half| patterns order like |bf16| patterns
             int e;
             bool is_nan;
-            const uint32_t sbyte = shared_exp_byte<FMT>(amax_bits, e, is_nan);
-            quant8_hw<FMT>(w, e, is_nan, q[h]);
+            uint32_t sbyte;
+            if constexpr (HALF) {
+                is_nan = amax_bits >= 0x7C00u;   // Inf or NaN in the block
+                sbyte = shared_exp_byte_f32<FMT>(half_bits_to_f32(amax_bits), is_nan, e);
+                quant8_f16_hw<FMT>(w, e, q[h]);
+                if (is_nan) q[h][0] = q[h][1] = FP4 ? 0x77777777u : 0x7F7F7F7Fu;
+            } else {
+                sbyte = shared_exp_byte<FMT>(amax_bits, e, is_nan);
+                quant8_hw<FMT>(w, e, is_nan, q[h]);
+            }
             // lanes 4j hold block j's scale byte: gather 4 of them into lanes 0, 16, 32, 48
             const uint32_t b1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)sbyte, 0x104, 0xF, 0xF, true);  // row_shl:4
             const uint32_t b2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)sbyte, 0x108, 0xF, 0xF, true);  // row_shl:8
@@ -287,6 +302,32 @@ __global__ __launch_bounds__(QUANT_THREADS) void mx_quant_rows_fast_kernel(
         if (p2 >= npairs) break;
         p0 = p2;
     }
+}
+
+// Fast form for IEEE half input (round to nearest even): returns 1 when the shape or the alignment
+// is not the fast kernel's, so that the caller takes its general kernel.
+template <int FMT>
+static int launch_rows_fast_half(const void *x, void *payload, void *scales, int64_t m, int64_t k, hipStream_t stream)
+{
+    if (!(k % 1024 == 0 && aligned(x, 16) && aligned(payload, 16) && aligned(scales, 4) && m * (k / 1024) < ((int64_t)1 << 30))) return 1;
+    const int64_t nblk = k / 32, sld = 2 * ((nblk + 1) / 2), pld = is_fp4_v<FMT> ? k / 2 : k;
+    int dev = 0, cus = 0;
+    CCH_HIP(hipGetDevice(&dev));
+    CCH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int64_t npairs = m * (k / 1024);
+    const unsigned grid = (unsigned)std::min<int64_t>((npairs + QUANT_THREADS / 64 - 1) / (QUANT_THREADS / 64), (int64_t)cus * QUANT_BLOCKS_PER_CU);
+    hipLaunchKernelGGL((mx_quant_rows_fast_kernel<FMT, false, true>), dim3(grid), dim3(QUANT_THREADS), 0, stream,
+                       static_cast<const uint16_t *>(x), static_cast<uint8_t *>(payload), static_cast<uint8_t *>(scales), (int)k, (int)sld,
+                       (int)pld, (int)(k / 1024), (int)npairs);
+    return launch_status("mx_quant_rows_fast_kernel (half input)");
+}
+
+int mx_quant_rows_fast_half(const void *x, void *payload, void *scales, int64_t m, int64_t k, int fmt, hipStream_t stream)
+{
+    if (fmt == CCH_FMT_E4M3) return launch_rows_fast_half<CCH_FMT_E4M3>(x, payload, scales, m, k, stream);
+    if (fmt == CCH_FMT_E5M2) return launch_rows_fast_half<CCH_FMT_E5M2>(x, payload, scales, m, k, stream);
+    if (fmt == CCH_FMT_E2M1) return launch_rows_fast_half<CCH_FMT_E2M1>(x, payload, scales, m, k, stream);
+    return 1;
 }
 
 template <int FMT, int RND, bool HWCVT>
@@ -414,7 +455,7 @@ static int launch_b(const void *b, void *payload, void *scales, int64_t k, int64
 // padded scale bytes.
 template <int FMT, int RND, bool HWCVT>
 static int launch_scatter(const void *x, const int32_t *dst_idx, void *packed, int64_t tokens, int64_t k, int topk,
-                          hipStream_t stream)
+                          int out_rows, hipStream_t stream)
 {
     const bool fp4 = is_fp4_v<FMT>;
     const int64_t nblk = (k + 31) / 32, sld = 2 * ((nblk + 1) / 2), pbytes = fp4 ? (k + 1) / 2 : k;
@@ -433,7 +474,7 @@ static int launch_scatter(const void *x, const int32_t *dst_idx, void *packed, i
         const unsigned grid = (unsigned)std::min<int64_t>((npairs + QUANT_THREADS / 64 - 1) / (QUANT_THREADS / 64), max_blocks);
         hipLaunchKernelGGL((mx_quant_rows_fast_kernel<FMT, true>), dim3(grid), dim3(QUANT_THREADS), 0, stream,
                            static_cast<const uint16_t *>(x), out, out + pbytes, (int)k, (int)row_bytes, (int)row_bytes,
-                           (int)(k / 1024), (int)npairs, dst_idx, topk);
+                           (int)(k / 1024), (int)npairs, dst_idx, topk, out_rows);
         return launch_status("mx_quant_rows_fast_kernel (scatter)");
     }
     const int64_t rows_per_launch = std::max<int64_t>(1, (int64_t)(1 << 30) / wpr);
@@ -447,11 +488,11 @@ static int launch_scatter(const void *x, const int32_t *dst_idx, void *packed, i
         if (vec)
             hipLaunchKernelGGL((mx_quant_rows_kernel<FMT, RND, HWCVT, true, false, true>), dim3(grid), dim3(QUANT_THREADS), 0,
                                stream, xs, out, out + pbytes, (int)rows, (int)k, (int)nblk, (int)sld, (int)row_bytes, (int)wpr,
-                               (int)total_ws, ds, topk, (int)row_bytes);
+                               (int)total_ws, ds, topk, (int)row_bytes, out_rows);
         else
             hipLaunchKernelGGL((mx_quant_rows_kernel<FMT, RND, HWCVT, false, false, true>), dim3(grid), dim3(QUANT_THREADS), 0,
                                stream, xs, out, out + pbytes, (int)rows, (int)k, (int)nblk, (int)sld, (int)row_bytes, (int)wpr,
-                               (int)total_ws, ds, topk, (int)row_bytes);
+                               (int)total_ws, ds, topk, (int)row_bytes, out_rows);
         int rc = launch_status("mx_quant_rows_kernel (scatter)");
         if (rc) return rc;
     }
@@ -474,7 +515,15 @@ bool quant_set_option(const char *name, int value)
 extern "C" int cch_mx_quant_scatter_packed(const void *x, const int32_t *expanded_row_idx, void *packed_out, int64_t tokens,
                                            int64_t k, int top_k, int fmt, int rounding, void *stream)
 {
+    return cch_mx_quant_scatter_packed_rows(x, expanded_row_idx, packed_out, 0x7FFFFFFF, tokens, k, top_k, fmt, rounding, stream);
+}
+
+extern "C" int cch_mx_quant_scatter_packed_rows(const void *x, const int32_t *expanded_row_idx, void *packed_out, int64_t out_rows,
+                                                int64_t tokens, int64_t k, int top_k, int fmt, int rounding, void *stream)
+{
     using namespace cch;
+    CCH_REQUIRE(out_rows >= 0, "cch_mx_quant_scatter_packed: out_rows=%lld", (long long)out_rows);
+    const int orows = (int)std::min<int64_t>(out_rows, 0x7FFFFFFF);
     CCH_REQUIRE(tokens >= 0 && k >= 0, "cch_mx_quant_scatter_packed: negative shape tokens=%lld k=%lld", (long long)tokens,
                 (long long)k);
     CCH_REQUIRE(k < (int64_t)1 << 30, "cch_mx_quant_scatter_packed: k=%lld too large", (long long)k);
@@ -487,17 +536,17 @@ extern "C" int cch_mx_quant_scatter_packed(const void *x, const int32_t *expande
     const bool lut = rounding == CCH_ROUND_LUT;
     switch (fmt) {
         case CCH_FMT_E4M3:
-            return lut ? launch_scatter<CCH_FMT_E4M3, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s)
-                       : launch_scatter<CCH_FMT_E4M3, CCH_ROUND_RNE, true>(x, expanded_row_idx, packed_out, tokens, k, top_k, s);
+            return lut ? launch_scatter<CCH_FMT_E4M3, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, orows, s)
+                       : launch_scatter<CCH_FMT_E4M3, CCH_ROUND_RNE, true>(x, expanded_row_idx, packed_out, tokens, k, top_k, orows, s);
         case CCH_FMT_E5M2:
-            return lut ? launch_scatter<CCH_FMT_E5M2, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s)
-                       : launch_scatter<CCH_FMT_E5M2, CCH_ROUND_RNE, true>(x, expanded_row_idx, packed_out, tokens, k, top_k, s);
+            return lut ? launch_scatter<CCH_FMT_E5M2, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, orows, s)
+                       : launch_scatter<CCH_FMT_E5M2, CCH_ROUND_RNE, true>(x, expanded_row_idx, packed_out, tokens, k, top_k, orows, s);
         case CCH_FMT_E2M1:
-            return lut ? launch_scatter<CCH_FMT_E2M1, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s)
-                       : launch_scatter<CCH_FMT_E2M1, CCH_ROUND_RNE, true>(x, expanded_row_idx, packed_out, tokens, k, top_k, s);
+            return lut ? launch_scatter<CCH_FMT_E2M1, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, orows, s)
+                       : launch_scatter<CCH_FMT_E2M1, CCH_ROUND_RNE, true>(x, expanded_row_idx, packed_out, tokens, k, top_k, orows, s);
         case CCH_FMT_E1M2:  // no hardware conversion for this format: integer encoder for both rules
-            return lut ? launch_scatter<CCH_FMT_E1M2, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s)
-                       : launch_scatter<CCH_FMT_E1M2, CCH_ROUND_RNE, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, s);
+            return lut ? launch_scatter<CCH_FMT_E1M2, CCH_ROUND_LUT, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, orows, s)
+                       : launch_scatter<CCH_FMT_E1M2, CCH_ROUND_RNE, false>(x, expanded_row_idx, packed_out, tokens, k, top_k, orows, s);
         default:
             return fail(CCH_EINVAL, "cch_mx_quant_scatter_packed: unknown format %d", fmt);
     }

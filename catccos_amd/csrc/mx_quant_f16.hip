@@ -13,79 +13,14 @@
 
 #include "common.h"
 #include "mx_formats.h"
+#include "mx_quant_block.h"
 
 namespace cch {
 
+// mx_quant.hip: 1 when the fast streaming kernel does not take the shape, else its launch status
+int mx_quant_rows_fast_half(const void *x, void *payload, void *scales, int64_t m, int64_t k, int fmt, hipStream_t stream);
+
 constexpr int F16Q_THREADS = 512;
-
-__device__ __forceinline__ float half_bits_to_f32(uint32_t h)
-{
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
-}
-
-// E8M0 byte and applied exponent from the block maximum as fp32 (the rule of shared_exp_byte,
-// on the fp32 exponent field: a subnormal half maximum is a normal fp32 number).
-template <int FMT>
-__device__ __forceinline__ uint32_t shared_exp_byte_f32(float amax, bool is_nan, int &e_out)
-{
-    using T = FmtTraits<FMT>;
-    int e = (int)((__float_as_uint(amax) >> 23) & 0xFFu) - 127 - T::EMAX;
-    e = max(-128, min(127, e));
-    if (amax < 1e-12f) e = 0;
-    e_out = max(e, -127);
-    return is_nan ? 0xFFu : (uint32_t)max(e + 127, 0);
-}
-
-typedef short s16x2 __attribute__((ext_vector_type(2)));
-typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-// Round-to-nearest-even payloads of 8 packed halves (w[i] = elements 2i, 2i+1) with gfx950's fused
-// conversions, which divide by the power-of-two scale and round straight from packed half.  The
-// FP4 form saturates; the FP8 forms return NaN above the format maximum, so magnitudes are first
-// clamped, as 16-bit integers, to the half pattern of MAXV * 2^e = 1.75 * 2^(e + EMAX) (for a
-// subnormal block maximum that limit is subnormal too: the pattern 0x700 shifted down).
-template <int FMT>
-__device__ __forceinline__ void quant8_f16_hw(const uint32_t (&w)[4], int e, uint32_t (&out)[2])
-{
-    using T = FmtTraits<FMT>;
-    const float scale = __uint_as_float((uint32_t)(e + 127) << 23);
-    if constexpr (FMT == CCH_FMT_E2M1) {
-        uint32_t r = 0;
-        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(f16x2, w[0]), scale, 0);
-        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(f16x2, w[1]), scale, 1);
-        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(f16x2, w[2]), scale, 2);
-        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(f16x2, w[3]), scale, 3);
-        out[0] = r;
-        out[1] = 0;
-    } else {
-        const int fe = e + T::EMAX + 15;   // half exponent field of the limit
-        const uint32_t t16 = fe > 30 ? 0x7BFFu : fe >= 1 ? (((uint32_t)fe << 10) | 0x300u) : (0x700u >> min(1 - fe, 11));
-        const u16x2 lim = {(unsigned short)t16, (unsigned short)t16};
-        f16x2 c[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const u16x2 mag = __builtin_elementwise_min(__builtin_bit_cast(u16x2, w[i] & 0x7FFF7FFFu), lim);
-            c[i] = __builtin_bit_cast(f16x2, __builtin_bit_cast(uint32_t, mag) | (w[i] & 0x80008000u));
-        }
-        s16x2 r0 = {0, 0}, r1 = {0, 0};
-        if constexpr (FMT == CCH_FMT_E4M3) {
-            r0 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r0, c[0], scale, false);
-            r0 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r0, c[1], scale, true);
-            r1 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r1, c[2], scale, false);
-            r1 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r1, c[3], scale, true);
-        } else {
-            r0 = __builtin_amdgcn_cvt_scalef32_pk_bf8_f16(r0, c[0], scale, false);
-            r0 = __builtin_amdgcn_cvt_scalef32_pk_bf8_f16(r0, c[1], scale, true);
-            r1 = __builtin_amdgcn_cvt_scalef32_pk_bf8_f16(r1, c[2], scale, false);
-            r1 = __builtin_amdgcn_cvt_scalef32_pk_bf8_f16(r1, c[3], scale, true);
-        }
-        out[0] = __builtin_bit_cast(uint32_t, r0);
-        out[1] = __builtin_bit_cast(uint32_t, r1);
-    }
-}
 
 // Grid-stride over (row, 8-element group): `tpr` groups per row, a multiple of four so that the
 // four lanes of a block sit in one quad.  VEC: k % 8 == 0 and 16-byte aligned rows.
@@ -221,6 +156,11 @@ extern "C" int cch_mx_quant_rows_f16(const void *x, void *payload, void *scales,
     CCH_REQUIRE(x && payload && scales, "cch_mx_quant_rows_f16: null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool lut = rounding == CCH_ROUND_LUT;
+    if (!lut) {
+        // whole 1024-element pieces per row and aligned buffers: the streaming form shared with the bf16 quantiser
+        const int rc = mx_quant_rows_fast_half(x, payload, scales, m, k, fmt, s);
+        if (rc != 1) return rc;
+    }
     switch (fmt) {
         case CCH_FMT_E4M3:
             return lut ? launch_f16<CCH_FMT_E4M3, CCH_ROUND_LUT>(x, payload, scales, m, k, s)

@@ -71,7 +71,7 @@ def packed_row_bytes(k, fmt="e4m3"):
 def mx_quant_scatter_packed(x, expanded_row_idx, packed_out, top_k, fmt="e4m3", rounding=ROUND_RNE):
     """Quantises every row of x (bf16 [tokens, K]) once and writes [payload | scales] to rows
     expanded_row_idx[t * top_k + r] of packed_out (uint8 [rows, packed_row_bytes(K)]), skipping
-    negative entries.  Rows that no route names keep their contents.  Returns packed_out."""
+    negative entries and entries at or past `rows`.  Rows that no route names keep their contents.  Returns packed_out."""
     fmt = _fmt(fmt)
     _require_gpu(x, expanded_row_idx, packed_out)
     if x.dim() != 2 or x.dtype != torch.bfloat16:
@@ -82,12 +82,12 @@ def mx_quant_scatter_packed(x, expanded_row_idx, packed_out, top_k, fmt="e4m3", 
     row_bytes = ((k + 1) // 2 if fmt in _FP4 else k) + scale_cols(k)
     if packed_out.dim() != 2 or packed_out.dtype != torch.uint8 or packed_out.shape[1] != row_bytes or not packed_out.is_contiguous():
         raise ValueError("packed_out must be a contiguous uint8 [rows, %d] tensor" % row_bytes)
-    if top_k and tokens and int(expanded_row_idx.max()) >= packed_out.shape[0]:
-        raise ValueError("expanded_row_idx names a row past packed_out")
+    # the kernel skips entries at or past packed_out's rows (like negative ones): no pass over the table
+    # here, which would stall the stream
     x = x.contiguous()
     idx = expanded_row_idx.contiguous()
-    check(_abi.lib().cch_mx_quant_scatter_packed(_ptr(x), _ptr(idx), _ptr(packed_out), tokens, k, int(top_k), fmt, rounding,
-                                                 _stream()))
+    check(_abi.lib().cch_mx_quant_scatter_packed_rows(_ptr(x), _ptr(idx), _ptr(packed_out), packed_out.shape[0], tokens, k, int(top_k),
+                                                      fmt, rounding, _stream()))
     return packed_out
 
 

@@ -219,6 +219,11 @@ int cch_mx_gmm_mapped(const void *a, const void *sa, const void *b, const void *
  * Destination rows must be distinct (two routes writing one row race, as in the reference). */
 int cch_mx_quant_scatter_packed(const void *x, const int32_t *expanded_row_idx, void *packed_out, int64_t tokens,
                                 int64_t k, int top_k, int fmt, int rounding, void *stream);
+/* The same with the number of rows of packed_out stated: an entry of expanded_row_idx at or past
+ * out_rows is skipped like a negative one instead of being written outside the buffer (a caller that
+ * cannot vouch for its routing table needs no pass over it on the host). */
+int cch_mx_quant_scatter_packed_rows(const void *x, const int32_t *expanded_row_idx, void *packed_out, int64_t out_rows,
+                                     int64_t tokens, int64_t k, int top_k, int fmt, int rounding, void *stream);
 
 /* ---- MoE token un-permute (combine side of the MoE path) ----
  * Replaces KernelMoeTokenUnpermute (examples/aux_ops/moe_token_unpermute/

@@ -80,5 +80,23 @@ def test_scatter_empty_and_errors():
     x = torch.zeros((2, 64), dtype=torch.bfloat16, device="cuda")
     with pytest.raises(cc.CatccosError):
         cc.mx_quant_scatter_packed(x, torch.zeros(18, dtype=torch.int32, device="cuda"), packed, 9)
-    with pytest.raises(ValueError):
-        cc.mx_quant_scatter_packed(x, torch.full((4,), 7, dtype=torch.int32, device="cuda"), packed, 2)
+    # entries at or past the rows of packed_out are skipped like negative ones (both kernels), nothing is written outside
+    cc.mx_quant_scatter_packed(x, torch.full((4,), 7, dtype=torch.int32, device="cuda"), packed, 2)
+    torch.cuda.synchronize()
+    assert (packed == 9).all()
+
+
+@pytest.mark.parametrize("shape", [(40, 2048, 2), (9, 96, 3)], ids=["streaming-kernel", "general-kernel"])
+def test_scatter_skips_rows_past_the_output(shape):
+    tokens, k, topk = shape
+    rng = np.random.default_rng(tokens)
+    xb = rand_rows(rng, tokens, k, 2.0)
+    out_rows = tokens * topk - 7            # seven routes name rows that do not exist
+    idx = rng.permutation(tokens * topk).astype(np.int32)
+    # guard rows behind the buffer that the call is told about
+    whole = torch.full((out_rows + 8, cc.packed_row_bytes(k)), 0x5A, dtype=torch.uint8, device="cuda")
+    cc.mx_quant_scatter_packed(dev_bf16(xb), torch.from_numpy(idx).cuda(), whole[:out_rows], topk)
+    torch.cuda.synchronize()
+    want = orc.mx_quant_scatter_packed(xb, np.where(idx >= out_rows, -1, idx), out_rows, topk, orc.E4M3, orc.RNE, fill=0x5A)
+    assert np.array_equal(whole[:out_rows].cpu().numpy(), want)
+    assert (whole[out_rows:] == 0x5A).all()
