@@ -121,6 +121,35 @@ def event_time_ms(fn, steps, warmup, warm_ms=0.0):
     return wall, per
 
 
+def clock_under_load(fn, seconds=1.5):
+    """Shader clock and power as rocm-smi reports them while fn() runs back to back: the figure that prices
+    the published peak (quoted at the 2.4 GHz boost clock) for this kernel.  Returns {} where rocm-smi is
+    missing or prints something else."""
+    import re
+    import subprocess
+    import torch
+    out = {}
+    t0 = time.perf_counter()
+    texts = []
+    try:
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(200):
+                fn()
+            if time.perf_counter() - t0 > 0.6 and len(texts) < 2:
+                texts.append(subprocess.run(["rocm-smi", "--showclocks", "--showpower"], capture_output=True, text=True, timeout=20).stdout)
+        torch.cuda.synchronize()
+        sclk = [int(m) for t in texts for m in re.findall(r"sclk clock level: \d+: \((\d+)Mhz\)", t)]
+        power = [float(m) for t in texts for m in re.findall(r"Power \(W\): ([0-9.]+)", t)]
+        if sclk:
+            out["sclk_mhz_under_load"] = sclk
+        if power:
+            out["power_w_under_load"] = power
+    except Exception as exc:   # a reporting aid only
+        torch.cuda.synchronize()
+        out["error"] = repr(exc)[:120]
+    return out
+
+
 def queue_time_ms(fn, launches, warm_ms):
     """Average duration of fn() over a queue of back-to-back launches between one pair of events
     (gaps between kernels included), after at least warm_ms of the same load."""
@@ -189,10 +218,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=100, help="untimed launches (about 55 ms: the clock's ramp from idle)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--no-clock", action="store_true", help="skip the 1.5 s of back-to-back launches under which rocm-smi is asked for the clock")
     ap.add_argument("--set-option", action="append", default=[], metavar="NAME=VALUE",
                     help="library switch for an A/B run, e.g. gemm_tile_order=0 (cch_set_option)")
-    ap.add_argument("--only", choices=["copy", "quant"], help="profiling aid: run only a 512 MiB device copy (counter "
-                    "calibration) or only the config-1 MX quantiser, print a short JSON line and exit")
+    ap.add_argument("--lib", metavar="PATH", help="another build of libcatccos_hip.so (a measurement build, see catccos_amd/build.py)")
+    ap.add_argument("--only", choices=["copy", "quant", "cfg2", "cfg3", "cfg4", "cfg5"], help="profiling aid: run only a 512 MiB device copy "
+                    "(counter calibration), only the config-1 MX quantiser, or only one of the other configurations' GEMMs; "
+                    "print a short JSON line and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the grouped GEMM; this build has no multi-GPU path "
@@ -200,6 +232,9 @@ def main():
 
     import numpy as np
     import torch
+    if args.lib:
+        from catccos_amd import _abi as abi0
+        abi0.LIB_PATH = os.path.abspath(args.lib)
     import catccos_amd as cc
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (MI355X); none is visible")
@@ -230,341 +265,370 @@ def main():
         cc.set_option(name, int(val))
     gs_host = zipf_groups(rng, T, E)
     gs = torch.from_numpy(gs_host).to(dev)
-    x0 = (torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16)
-    a, sa = cc.mx_quant(x0, "e4m3")
-    b = torch.empty((E, K, N), dtype=torch.uint8, device=dev)
-    sb = torch.empty((E, K // 64, N, 2), dtype=torch.uint8, device=dev)
-    for e in range(E):
-        w0 = (torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16)
-        b[e], sb[e] = cc.mx_quant_b(w0, "e4m3", trans_b=TRANS_B)
-    del x0, w0
-    torch.cuda.synchronize()
-
-    out = [None]
-
-    def step():
-        out[0] = cc.mx_grouped_matmul(a, sa, b, sb, gs, "e4m3", TRANS_B)
-
-    # `warmup` launches as asked for, then more of the same until the shader clock has settled (see event_time_ms)
-    wall_ms, per_ms = event_time_ms(step, args.steps, args.warmup, warm_ms=100.0)
-    kernel_ms = float(np.mean(per_ms))
+    only_cfg = args.only if args.only in ("cfg2", "cfg3", "cfg4", "cfg5") else None
     flop = 2.0 * T * N * K
-    value = flop / (wall_ms * 1e-3) / 1e12
-    achieved = flop / (kernel_ms * 1e-3) / 1e12
-
-    # size-independent sanity of the timed result: sampled rows against the oracle happen in the CPU leg below
-    result = {
-        "metric": "MXFP8 GMM TFLOP/s (% MFMA peak); MX-quant HBM GB/s (% of peak)",
-        "value": round(value, 2),
-        "unit": "TFLOP/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(wall_ms, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "mxfp8 (e4m3 x e4m3, e8m0 scales, f32 accumulate, bf16 out)",
-        "data": "synthetic",
-        "config": {"workload": "MXFP8 grouped matmul, config-5 shapes with E4M3 payload", "experts": E, "tokens": T, "k": K,
-                   "n": N, "trans_b": TRANS_B, "group_sizes": gs_host.tolist()},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / FP8_PEAK_TFLOPS, 4), "traffic": GMM_TRAFFIC_BYTES,
-                     "kernel": "gemm_tile_kernel<KIND_F8, EPI_PLAIN, E4M3, TB=0>", "algorithmic_flop_per_launch": flop,
-                     "kernel_ms_min": round(float(np.min(per_ms)), 4), "kernel_ms_median": round(float(np.median(per_ms)), 4),
-                     "kernel_ms_mean": round(kernel_ms, 4)},
-    }
-
-    # ------------------------------------------------------------ CPU baseline on a bounded sample of rows
-    cpu = not args.no_cpu_baseline
-    if cpu:
-        import oracle as orc
-        a_h, sa_h = a.cpu().numpy(), sa.cpu().numpy()
-        b_h, sb_h = b.cpu().numpy(), sb.cpu().numpy()
-        out_h = out[0].float().cpu().numpy()
-        used = int(gs_host.sum())
-        rows, gold, rec = cpu_leg(lambda r: orc.mx_gmm(a_h, sa_h, b_h, sb_h, N, K, orc.E4M3, TRANS_B, group_sizes=gs_host, rows=r, blocked=True),
-                                  2.0 * used * N * K, used, lambda n: sample_rows(rng_s, gs_host, n), 20.0, "TFLOP/s")
-        rec["parity_on_sample"] = parity_record(out_h[rows], gold)
-        rec["parity_on_sample"]["rows_past_the_groups_are_zero"] = bool(np.all(out_h[used:] == 0))
-        result["cpu_baseline"] = rec
-        del a_h, sa_h, b_h, sb_h, out_h, gold
-
-    # ------------------------------------------------------------ the other configurations, same library
-    if not args.no_extra:
-        extra = {}
-        # config 1: MX quantiser, rotating buffer sets larger than the 256 MB Infinity Cache
-        M1, K1 = 4096, 7168
-        sets = quant_inputs(dev, M1, K1, 6)
-        q_us = quant_batch_time_us(sets, 120, 1500)
-        qbytes = M1 * K1 * 2 + M1 * K1 + M1 * K1 // 32
-        q_gbs = qbytes / (q_us * 1e-6) / 1e9
-        extra["mx_quant_cfg1"] = {"gb_per_s": round(q_gbs, 1), "frac_of_hbm_peak": round(q_gbs / HBM_PEAK_GBS, 4),
-                                  "us": round(q_us, 2), "bytes": qbytes, "buffers": "6 rotating input sets (352 MB), 120 queued launches"}
-        # the same kernel on one input set that stays in the Infinity Cache: the rate a caller sees whose tensor was just written
-        hot_us = quant_batch_time_us(sets[:1], 120, 1500)
-        extra["mx_quant_cfg1"]["hot_cache"] = {"gb_per_s": round(qbytes / (hot_us * 1e-6) / 1e9, 1), "us": round(hot_us, 2),
-                                               "buffers": "one input set (59 MB) read again and again"}
-        if cpu:
-            # whole-tensor check and CPU rate of the same tensor
-            x_h = sets[0].view(torch.int16).cpu().numpy().view(np.uint16)
-            t0 = time.perf_counter()
-            pq_h, sq_h = orc.mx_quant_rows(x_h, orc.E4M3)
-            dt = time.perf_counter() - t0
-            pq_d, sq_d = cc.mx_quant(sets[0], "e4m3")
-            extra["mx_quant_cfg1"]["cpu_baseline"] = {"value": round(qbytes / dt / 1e9, 2), "unit": "GB/s", "cores": orc.num_threads(), "kind": "port",
-                                                      "sample": "the whole [4096, 7168] tensor, %.2f s" % dt}
-            extra["mx_quant_cfg1"]["parity"] = {"bit_exact_whole_tensor": bool(np.array_equal(pq_d.cpu().numpy(), pq_h) and
-                                                                               np.array_equal(sq_d.cpu().numpy(), sq_h)),
-                                                "payload_bytes": int(pq_h.size), "scale_bytes": int(sq_h.size)}
-        # the half-input twin of the quantiser on the same values
-        sets16 = [x.to(torch.float16) for x in sets]
-        h_us = quant_batch_time_us(sets16, 120, 1500, "cch_mx_quant_rows_f16")
-        extra["mx_quant_f16_input_cfg1_shape"] = {"gb_per_s": round(qbytes / (h_us * 1e-6) / 1e9, 1),
-                                                  "frac_of_hbm_peak": round(qbytes / (h_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                                                  "us": round(h_us, 2), "bytes": qbytes}
-        if cpu:
-            t0 = time.perf_counter()
-            ph_h, sh_h = orc.mx_quant_rows_f16(sets16[0].view(torch.int16).cpu().numpy().view(np.uint16), orc.E4M3)
-            dt = time.perf_counter() - t0
-            ph_d, sh_d = cc.mx_quant(sets16[0], "e4m3")
-            extra["mx_quant_f16_input_cfg1_shape"]["cpu_baseline"] = {"value": round(qbytes / dt / 1e9, 2), "unit": "GB/s", "cores": orc.num_threads(),
-                                                                      "kind": "port", "sample": "the whole [4096, 7168] tensor, %.2f s" % dt}
-            extra["mx_quant_f16_input_cfg1_shape"]["parity"] = {"bit_exact_whole_tensor": bool(np.array_equal(ph_d.cpu().numpy(), ph_h) and
-                                                                                             np.array_equal(sh_d.cpu().numpy(), sh_h))}
-        del sets16
-        # the same rows quantised once and scattered as packed [payload | scales] rows to their top-2 destinations
-        idx1 = torch.randperm(M1 * 2, device=dev).to(torch.int32)
-        packed1 = torch.empty((M1 * 2, cc.packed_row_bytes(K1)), dtype=torch.uint8, device=dev)
-        st1 = torch.cuda.current_stream().cuda_stream
-        from catccos_amd import _abi as abi1
-
-        def sc_launch(i):
-            abi1.check(abi1.lib().cch_mx_quant_scatter_packed(sets[i % len(sets)].data_ptr(), idx1.data_ptr(), packed1.data_ptr(),
-                                                              M1, K1, 2, 0, 0, st1))
-
-        for i in range(600):
-            sc_launch(i)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for i in range(120):
-            sc_launch(i)
-        e1.record()
-        torch.cuda.synchronize()
-        sc_us = e0.elapsed_time(e1) * 1e3 / 120
-        sc_bytes = M1 * K1 * 2 + 2 * M1 * cc.packed_row_bytes(K1)
-        extra["mx_quant_scatter_top2_cfg1_rows"] = {"gb_per_s": round(sc_bytes / sc_us / 1e3, 1),
-                                                    "frac_of_hbm_peak": round(sc_bytes / sc_us / 1e3 / HBM_PEAK_GBS, 4),
-                                                    "us": round(sc_us, 2), "bytes": sc_bytes}
-        if cpu:
-            sc_launch(0)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            pk_h = orc.mx_quant_scatter_packed(x_h, idx1.cpu().numpy(), M1 * 2, 2, orc.E4M3)
-            dt = time.perf_counter() - t0
-            extra["mx_quant_scatter_top2_cfg1_rows"]["cpu_baseline"] = {"value": round(sc_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": orc.num_threads(),
-                                                                        "kind": "port", "sample": "all 4096 tokens, top-2, %.2f s" % dt}
-            extra["mx_quant_scatter_top2_cfg1_rows"]["parity"] = {"bit_exact_whole_tensor": bool(np.array_equal(packed1.cpu().numpy(), pk_h))}
-        del sets, packed1
-        # config 2: int8 W8A8 + dequant
-        m2, k2, n2 = 8192, 4096, 8192
-        a2 = torch.randint(-127, 128, (m2, k2), dtype=torch.int8, device=dev)
-        b2 = torch.randint(-127, 128, (k2, n2), dtype=torch.int8, device=dev)
-        pt2 = torch.rand(m2, device=dev) * 0.019 + 0.001
-        pc2 = torch.rand(n2, device=dev) * 0.019 + 0.001
-        t2 = [queue_time_ms(lambda: cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, TRANS_B), 30, 60.0)]
-        extra["w8a8_dequant_cfg2"] = {"tops": round(2.0 * m2 * n2 * k2 / (np.mean(t2) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t2)) * 1e3, 1)}
-        extra["w8a8_dequant_cfg2"]["frac_of_int8_peak"] = round(extra["w8a8_dequant_cfg2"]["tops"] / FP8_PEAK_TFLOPS, 4)
-        if cpu:
-            o2 = cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, TRANS_B).float().cpu().numpy()
-            a2h, b2h, pt2h, pc2h = a2.cpu().numpy(), b2.cpu().numpy(), pt2.cpu().numpy(), pc2.cpu().numpy()
-            rows, gold, rec = cpu_leg(lambda r: orc.gemm_i8_dequant(a2h, b2h, pt2h, pc2h, TRANS_B, rows=r, blocked=True), 2.0 * m2 * n2 * k2, m2,
-                                      lambda n: np.sort(rng_s.choice(m2, n, replace=False)).astype(np.int64), 6.0, "TOP/s")
-            extra["w8a8_dequant_cfg2"]["cpu_baseline"] = rec
-            extra["w8a8_dequant_cfg2"]["parity"] = parity_record(o2[rows], gold)
-            del o2, a2h, b2h, gold
-        del a2, b2
-        # config 3: MXFP8 dense
-        m3, k3, n3 = 4096, 2048, 7168
-        a3, sa3 = cc.mx_quant(torch.randn(m3, k3, device=dev).to(torch.bfloat16), "e4m3")
-        b3, sb3 = cc.mx_quant_b(torch.randn(k3, n3, device=dev).to(torch.bfloat16), "e4m3", trans_b=TRANS_B)
-        t3 = [queue_time_ms(lambda: cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", TRANS_B), 30, 60.0)]
-        extra["mxfp8_dense_cfg3"] = {"tflops": round(2.0 * m3 * n3 * k3 / (np.mean(t3) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t3)) * 1e3, 1)}
-        extra["mxfp8_dense_cfg3"]["frac_of_fp8_peak"] = round(extra["mxfp8_dense_cfg3"]["tflops"] / FP8_PEAK_TFLOPS, 4)
-        if cpu:
-            o3 = cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", TRANS_B).float().cpu().numpy()
-            h3 = [t.cpu().numpy() for t in (a3, sa3, b3, sb3)]
-            rows, gold, rec = cpu_leg(lambda r: orc.mx_gmm(h3[0], h3[1], h3[2], h3[3], n3, k3, orc.E4M3, TRANS_B, rows=r, blocked=True), 2.0 * m3 * n3 * k3, m3,
-                                      lambda n: np.sort(rng_s.choice(m3, n, replace=False)).astype(np.int64), 6.0, "TFLOP/s")
-            extra["mxfp8_dense_cfg3"]["cpu_baseline"] = rec
-            extra["mxfp8_dense_cfg3"]["parity"] = parity_record(o3[rows], gold)
-            del o3, h3, gold
-        # config 4: MoE W8A8 grouped + dequant + SwiGLU
-        e4, t4, k4, n4 = 16, 8192, 7168, 4096
-        gs4 = torch.from_numpy(zipf_groups(rng, t4, e4)).to(dev)
-        x4 = torch.randint(-127, 128, (t4, k4), dtype=torch.int8, device=dev)
-        w4 = torch.randint(-127, 128, (e4, k4, n4), dtype=torch.int8, device=dev)
-        pt4 = torch.rand(t4, device=dev) * 0.019 + 0.001
-        pc4 = torch.rand(e4, n4, device=dev) * 0.019 + 0.001
-        tt4 = [queue_time_ms(lambda: cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), 30, 60.0)]
-        extra["moe_w8a8_swiglu_cfg4"] = {"tops": round(2.0 * t4 * n4 * k4 / (np.mean(tt4) * 1e-3) / 1e12, 1), "us": round(float(np.mean(tt4)) * 1e3, 1)}
-        extra["moe_w8a8_swiglu_cfg4"]["frac_of_int8_peak"] = round(extra["moe_w8a8_swiglu_cfg4"]["tops"] / FP8_PEAK_TFLOPS, 4)
-        # the same with the activation leaving as MXFP8 from the epilogue, against the two-kernel chain it replaces
-        tf4 = queue_time_ms(lambda: cc.gmm_dequant_swiglu_mx(x4, w4, gs4, pt4, pc4, TRANS_B, "e4m3"), 30, 60.0)
-        tc4 = queue_time_ms(lambda: cc.mx_quant(cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), "e4m3"), 30, 60.0)
-        pf4, sf4 = cc.gmm_dequant_swiglu_mx(x4, w4, gs4, pt4, pc4, TRANS_B, "e4m3")
-        pq4, sq4 = cc.mx_quant(cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), "e4m3")
-        extra["moe_w8a8_swiglu_mxfp8_out_cfg4"] = {"us": round(tf4 * 1e3, 1), "two_kernel_chain_us": round(tc4 * 1e3, 1),
-                                                   "tops": round(2.0 * t4 * n4 * k4 / (tf4 * 1e-3) / 1e12, 1),
-                                                   "parity": {"bit_exact_vs_quantised_bf16_output": bool(torch.equal(pf4, pq4) and torch.equal(sf4, sq4))}}
-        del pf4, sf4, pq4, sq4
-        if cpu:
-            o4 = cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B).float().cpu().numpy()
-            h4 = [t.cpu().numpy() for t in (x4, w4, gs4, pt4, pc4)]
-            used4 = int(h4[2].sum())
-            rows, gold, rec = cpu_leg(lambda r: orc.gmm_i8_dequant_swiglu(h4[0], h4[1], h4[2], h4[3], h4[4], rows=r, blocked=True), 2.0 * used4 * n4 * k4,
-                                      used4, lambda n: sample_rows(rng_s, h4[2], n), 8.0, "TOP/s")
-            extra["moe_w8a8_swiglu_cfg4"]["cpu_baseline"] = rec
-            extra["moe_w8a8_swiglu_cfg4"]["parity"] = parity_record(o4[rows], gold)
-            extra["moe_w8a8_swiglu_cfg4"]["parity"]["rows_past_the_groups_are_zero"] = bool(np.all(o4[used4:] == 0))
-            del o4, h4, gold
-        del x4, w4
-        # input side of config 4: per-token dynamic int8 quantisation of the bf16 tokens (queued launches through the C ABI)
-        from catccos_amd import _abi
-        xs4 = [torch.randn(t4, k4, device=dev).to(torch.bfloat16) for _ in range(4)]
-        q4 = torch.empty((t4, k4), dtype=torch.int8, device=dev)
-        s4 = torch.empty((t4,), dtype=torch.float32, device=dev)
-        st4 = torch.cuda.current_stream().cuda_stream
-
-        def dq_launch(i):
-            _abi.check(_abi.lib().cch_dyn_quant_i8_rows(xs4[i % 4].data_ptr(), None, q4.data_ptr(), s4.data_ptr(), t4, t4, k4, 1, 0, st4))
-
-        for i in range(800):
-            dq_launch(i)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for i in range(60):
-            dq_launch(i)
-        e1.record()
-        torch.cuda.synchronize()
-        dq_us = e0.elapsed_time(e1) * 1e3 / 60
-        dq_bytes = t4 * k4 * 3 + t4 * 4
-        extra["dyn_quant_i8_cfg4_tokens"] = {"gb_per_s": round(dq_bytes / dq_us / 1e3, 1), "frac_of_hbm_peak": round(dq_bytes / dq_us / 1e3 / HBM_PEAK_GBS, 4),
-                                             "us": round(dq_us, 2), "bytes": dq_bytes}
-        if cpu:
-            dq_launch(0)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            qh, sh = orc.dyn_quant_i8_rows(xs4[0].view(torch.int16).cpu().numpy().view(np.uint16))
-            dt = time.perf_counter() - t0
-            extra["dyn_quant_i8_cfg4_tokens"]["cpu_baseline"] = {"value": round(dq_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": orc.num_threads(),
-                                                                 "kind": "port", "sample": "all 8192 tokens, %.2f s" % dt}
-            extra["dyn_quant_i8_cfg4_tokens"]["parity"] = {"bit_exact_whole_tensor": bool(np.array_equal(q4.cpu().numpy(), qh) and
-                                                                                        np.array_equal(s4.cpu().numpy(), sh))}
-        del xs4, q4
-        # combine side: top-2 weighted un-permute of 8192 expert-output rows back to 4096 tokens
-        tok_u, hid_u, topk_u = 4096, 7168, 2
-        ys = [torch.randn(tok_u * topk_u, hid_u, device=dev).to(torch.bfloat16) for _ in range(3)]
-        idx_u = torch.randperm(tok_u * topk_u, device=dev).to(torch.int32)
-        pr_u = torch.rand(tok_u * topk_u, device=dev)
-        out_u = torch.empty((tok_u, hid_u), dtype=torch.bfloat16, device=dev)
-
-        def un_launch(i):
-            _abi.check(_abi.lib().cch_moe_token_unpermute(ys[i % 3].data_ptr(), idx_u.data_ptr(), pr_u.data_ptr(), out_u.data_ptr(),
-                                                          tok_u * topk_u, tok_u, hid_u, topk_u, st4))
-
-        for i in range(600):
-            un_launch(i)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for i in range(60):
-            un_launch(i)
-        e1.record()
-        torch.cuda.synchronize()
-        un_us = e0.elapsed_time(e1) * 1e3 / 60
-        un_bytes = tok_u * topk_u * hid_u * 2 + tok_u * hid_u * 2 + tok_u * topk_u * 8
-        extra["moe_token_unpermute_top2"] = {"gb_per_s": round(un_bytes / un_us / 1e3, 1), "frac_of_hbm_peak": round(un_bytes / un_us / 1e3 / HBM_PEAK_GBS, 4),
-                                             "us": round(un_us, 2), "bytes": un_bytes}
-        if cpu:
-            un_launch(0)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            uh = orc.moe_token_unpermute(ys[0].view(torch.int16).cpu().numpy().view(np.uint16), idx_u.cpu().numpy(), pr_u.cpu().numpy(), topk_u)
-            dt = time.perf_counter() - t0
-            extra["moe_token_unpermute_top2"]["cpu_baseline"] = {"value": round(un_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": orc.num_threads(),
-                                                                 "kind": "port", "sample": "all 4096 tokens, %.2f s" % dt}
-            extra["moe_token_unpermute_top2"]["parity"] = {"bit_exact_whole_tensor": bool(np.array_equal(
-                out_u.view(torch.int16).cpu().numpy().view(np.uint16), uh))}
-        del ys, out_u
-        # routing sort of config 4's routes (8192 tokens, top-2, 16 experts): three short launches through the C ABI
-        rt_rows, rt_e = 8192 * 2, 16
-        rt_idx = torch.randint(0, rt_e, (rt_rows,), dtype=torch.int32, device=dev)
-        rt_d2s = torch.empty(rt_rows, dtype=torch.int32, device=dev)
-        rt_s2d = torch.empty_like(rt_d2s)
-        rt_cnt = torch.empty(rt_e, dtype=torch.int32, device=dev)
-        rt_wsb = int(_abi.lib().cch_moe_init_routing_workspace_bytes(rt_rows, rt_e))
-        rt_ws = torch.empty(max(rt_wsb, 4), dtype=torch.uint8, device=dev)
-
-        def rt_launch():
-            _abi.check(_abi.lib().cch_moe_init_routing(rt_idx.data_ptr(), rt_rows, rt_e, rt_d2s.data_ptr(), rt_s2d.data_ptr(),
-                                                       rt_cnt.data_ptr(), 0, rt_ws.data_ptr(), rt_wsb, st4))
-
-        for _ in range(200):
-            rt_launch()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(100):
-            rt_launch()
-        e1.record()
-        torch.cuda.synchronize()
-        extra["moe_init_routing_cfg4_routes"] = {"us": round(e0.elapsed_time(e1) * 1e3 / 100, 2), "routes": rt_rows, "experts": rt_e,
-                                                 "launches_per_call": 3}
-        if cpu:
-            t0 = time.perf_counter()
-            d2s_h, s2d_h, cnt_h = orc.moe_init_routing(rt_idx.cpu().numpy(), rt_e)
-            dt = time.perf_counter() - t0
-            extra["moe_init_routing_cfg4_routes"]["cpu_baseline"] = {"value": round(dt * 1e6, 1), "unit": "us", "cores": 1, "kind": "port",
-                                                                     "sample": "all 16384 routes (numpy stable argsort and bincount)"}
-            extra["moe_init_routing_cfg4_routes"]["parity"] = {"bit_exact_whole_tensor": bool(
-                np.array_equal(rt_d2s.cpu().numpy(), d2s_h) and np.array_equal(rt_s2d.cpu().numpy(), s2d_h) and np.array_equal(rt_cnt.cpu().numpy(), cnt_h))}
-        # config 5: MXFP4 grouped (same groups as the headline)
-        a5, sa5 = cc.mx_quant((torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16), "e2m1")
-        b5 = torch.empty((E, K, N // 2), dtype=torch.uint8, device=dev)
-        sb5 = torch.empty((E, K // 64, N, 2), dtype=torch.uint8, device=dev)
+    cpu = not args.no_cpu_baseline and only_cfg is None
+    result = {"only": only_cfg}
+    if only_cfg is None:
+        x0 = (torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16)
+        a, sa = cc.mx_quant(x0, "e4m3")
+        b = torch.empty((E, K, N), dtype=torch.uint8, device=dev)
+        sb = torch.empty((E, K // 64, N, 2), dtype=torch.uint8, device=dev)
         for e in range(E):
-            b5[e], sb5[e] = cc.mx_quant_b((torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16), "e2m1", trans_b=TRANS_B)
-        t5 = [queue_time_ms(lambda: cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", TRANS_B), 30, 60.0)]
-        extra["mxfp4_grouped_cfg5"] = {"tflops": round(flop / (np.mean(t5) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t5)) * 1e3, 1)}
-        extra["mxfp4_grouped_cfg5"]["frac_of_fp4_peak"] = round(extra["mxfp4_grouped_cfg5"]["tflops"] / FP4_PEAK_TFLOPS, 4)
-        if cpu:
-            o5 = cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", TRANS_B).float().cpu().numpy()
-            h5 = [t.cpu().numpy() for t in (a5, sa5, b5, sb5)]
-            used5 = int(gs_host.sum())
-            rows, gold, rec = cpu_leg(lambda r: orc.mx_gmm(h5[0], h5[1], h5[2], h5[3], N, K, orc.E2M1, TRANS_B, group_sizes=gs_host, rows=r, blocked=True),
-                                      2.0 * used5 * N * K, used5, lambda n: sample_rows(rng_s, gs_host, n), 10.0, "TFLOP/s")
-            extra["mxfp4_grouped_cfg5"]["cpu_baseline"] = rec
-            extra["mxfp4_grouped_cfg5"]["parity"] = parity_record(o5[rows], gold)
-            del o5, h5, gold
-        del a5, sa5, b5, sb5
-        # Yardstick, not part of this build: the vendor library's dense FP8 GEMM (per-tensor scales, E4M3,
-        # bf16 out) on the headline's shape as one group, and this kernel on the same bytes with unit scales.
+            w0 = (torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16)
+            b[e], sb[e] = cc.mx_quant_b(w0, "e4m3", trans_b=TRANS_B)
+        del x0, w0
+        torch.cuda.synchronize()
+
+        out = [None]
+
+        def step():
+            out[0] = cc.mx_grouped_matmul(a, sa, b, sb, gs, "e4m3", TRANS_B)
+
+        # `warmup` launches as asked for, then more of the same until the shader clock has settled (see event_time_ms)
+        wall_ms, per_ms = event_time_ms(step, args.steps, args.warmup, warm_ms=100.0)
+        kernel_ms = float(np.mean(per_ms))
+        flop = 2.0 * T * N * K
+        value = flop / (wall_ms * 1e-3) / 1e12
+        achieved = flop / (kernel_ms * 1e-3) / 1e12
+
+        clk = clock_under_load(step) if not args.no_clock else {}
+        # an instrumented build of the library (--lib, built with -DCCH_PROF) counts the shader cycles every wave spends in the
+        # waits and barriers of the K loop: mean per wave of the last launch, first and second wave group apart
         try:
-            ya = (torch.randn(T, K, device=dev) * 0.5).to(torch.float8_e4m3fn)
-            yb = (torch.randn(N, K, device=dev) * 0.5).to(torch.float8_e4m3fn)
-            one = torch.tensor(1.0, device=dev)
-            t_lib = queue_time_ms(lambda: torch._scaled_mm(ya, yb.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16), 100, 150.0)
-            ysa = torch.full((T, K // 32), 127, dtype=torch.uint8, device=dev)
-            ysb = torch.full((N, K // 32), 127, dtype=torch.uint8, device=dev)
-            t_own = queue_time_ms(lambda: cc.mx_matmul(ya.view(torch.uint8), ysa, yb.view(torch.uint8), ysb, "e4m3", 1), 100, 150.0)
-            extra["yardstick_dense_fp8_16384x4096x7168"] = {
-                "library_scaled_mm_tflops": round(flop / (t_lib * 1e-3) / 1e12, 1), "this_kernel_same_data_tflops": round(flop / (t_own * 1e-3) / 1e12, 1),
-                "note": "library = torch._scaled_mm (per-tensor scales); both with B as [N,K]"}
-        except Exception as exc:   # the library call is optional: a box without it still reports everything else
-            extra["yardstick_dense_fp8_16384x4096x7168"] = {"error": repr(exc)[:200]}
+            import ctypes
+            from catccos_amd import _abi as abi_p
+            rd = abi_p.lib().cch_prof_read
+            rd.argtypes = [ctypes.c_void_p]
+            step()
+            torch.cuda.synchronize()
+            buf = (ctypes.c_uint64 * (256 * 64))()
+            if rd(buf) == 0:
+                d = np.frombuffer(buf, dtype=np.uint64).reshape(256, 8, 8).astype(np.float64)
+                names = ["total", "lgkm_wait_L0", "barrier_after_L0", "vm_wait_C0", "barrier_after_C0", "vm_wait_L1", "barrier_after_L1", "barrier_after_C1"]
+                clk["shader_cycles_per_wave"] = {g: {n: int(v) for n, v in zip(names, d[:, sl, :].mean(axis=(0, 1)))}
+                                                 for g, sl in (("waves_0_3", slice(0, 4)), ("waves_4_7", slice(4, 8)))}
+        except AttributeError:
+            pass
+        # size-independent sanity of the timed result: sampled rows against the oracle happen in the CPU leg below
+        result = {
+            "metric": "MXFP8 GMM TFLOP/s (% MFMA peak); MX-quant HBM GB/s (% of peak)",
+            "value": round(value, 2),
+            "unit": "TFLOP/s",
+            "n_gpus": 1,
+            "steps": args.steps,
+            "warmup": args.warmup,
+            "ms_per_step": round(wall_ms, 4),
+            "higher_is_better": True,
+            "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "mxfp8 (e4m3 x e4m3, e8m0 scales, f32 accumulate, bf16 out)",
+            "data": "synthetic",
+            "config": {"workload": "MXFP8 grouped matmul, config-5 shapes with E4M3 payload", "experts": E, "tokens": T, "k": K,
+                       "n": N, "trans_b": TRANS_B, "group_sizes": gs_host.tolist()},
+            "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(achieved / FP8_PEAK_TFLOPS, 4), "traffic": GMM_TRAFFIC_BYTES,
+                         "kernel": "gemm_tile_kernel<KIND_F8, EPI_PLAIN, E4M3, TB=0>", "algorithmic_flop_per_launch": flop,
+                         "kernel_ms_min": round(float(np.min(per_ms)), 4), "kernel_ms_median": round(float(np.median(per_ms)), 4),
+                         "kernel_ms_mean": round(kernel_ms, 4), **clk},
+        }
+
+        # ------------------------------------------------------------ CPU baseline on a bounded sample of rows
+        if cpu:
+            import oracle as orc
+            a_h, sa_h = a.cpu().numpy(), sa.cpu().numpy()
+            b_h, sb_h = b.cpu().numpy(), sb.cpu().numpy()
+            out_h = out[0].float().cpu().numpy()
+            used = int(gs_host.sum())
+            rows, gold, rec = cpu_leg(lambda r: orc.mx_gmm(a_h, sa_h, b_h, sb_h, N, K, orc.E4M3, TRANS_B, group_sizes=gs_host, rows=r, blocked=True),
+                                      2.0 * used * N * K, used, lambda n: sample_rows(rng_s, gs_host, n), 20.0, "TFLOP/s")
+            rec["parity_on_sample"] = parity_record(out_h[rows], gold)
+            rec["parity_on_sample"]["rows_past_the_groups_are_zero"] = bool(np.all(out_h[used:] == 0))
+            result["cpu_baseline"] = rec
+            del a_h, sa_h, b_h, sb_h, out_h, gold
+
+        # ------------------------------------------------------------ the other configurations, same library
+    if not args.no_extra or only_cfg:
+        extra = {}
+        if only_cfg is None:
+            # config 1: MX quantiser, rotating buffer sets larger than the 256 MB Infinity Cache
+            M1, K1 = 4096, 7168
+            sets = quant_inputs(dev, M1, K1, 6)
+            q_us = quant_batch_time_us(sets, 120, 1500)
+            qbytes = M1 * K1 * 2 + M1 * K1 + M1 * K1 // 32
+            q_gbs = qbytes / (q_us * 1e-6) / 1e9
+            extra["mx_quant_cfg1"] = {"gb_per_s": round(q_gbs, 1), "frac_of_hbm_peak": round(q_gbs / HBM_PEAK_GBS, 4),
+                                      "us": round(q_us, 2), "bytes": qbytes, "buffers": "6 rotating input sets (352 MB), 120 queued launches"}
+            # the same kernel on one input set that stays in the Infinity Cache: the rate a caller sees whose tensor was just written
+            hot_us = quant_batch_time_us(sets[:1], 120, 1500)
+            extra["mx_quant_cfg1"]["hot_cache"] = {"gb_per_s": round(qbytes / (hot_us * 1e-6) / 1e9, 1), "us": round(hot_us, 2),
+                                                   "buffers": "one input set (59 MB) read again and again"}
+            if cpu:
+                # whole-tensor check and CPU rate of the same tensor
+                x_h = sets[0].view(torch.int16).cpu().numpy().view(np.uint16)
+                t0 = time.perf_counter()
+                pq_h, sq_h = orc.mx_quant_rows(x_h, orc.E4M3)
+                dt = time.perf_counter() - t0
+                pq_d, sq_d = cc.mx_quant(sets[0], "e4m3")
+                extra["mx_quant_cfg1"]["cpu_baseline"] = {"value": round(qbytes / dt / 1e9, 2), "unit": "GB/s", "cores": orc.num_threads(), "kind": "port",
+                                                          "sample": "the whole [4096, 7168] tensor, %.2f s" % dt}
+                extra["mx_quant_cfg1"]["parity"] = {"bit_exact_whole_tensor": bool(np.array_equal(pq_d.cpu().numpy(), pq_h) and
+                                                                                   np.array_equal(sq_d.cpu().numpy(), sq_h)),
+                                                    "payload_bytes": int(pq_h.size), "scale_bytes": int(sq_h.size)}
+            # the half-input twin of the quantiser on the same values
+            sets16 = [x.to(torch.float16) for x in sets]
+            h_us = quant_batch_time_us(sets16, 120, 1500, "cch_mx_quant_rows_f16")
+            extra["mx_quant_f16_input_cfg1_shape"] = {"gb_per_s": round(qbytes / (h_us * 1e-6) / 1e9, 1),
+                                                      "frac_of_hbm_peak": round(qbytes / (h_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                                                      "us": round(h_us, 2), "bytes": qbytes}
+            if cpu:
+                t0 = time.perf_counter()
+                ph_h, sh_h = orc.mx_quant_rows_f16(sets16[0].view(torch.int16).cpu().numpy().view(np.uint16), orc.E4M3)
+                dt = time.perf_counter() - t0
+                ph_d, sh_d = cc.mx_quant(sets16[0], "e4m3")
+                extra["mx_quant_f16_input_cfg1_shape"]["cpu_baseline"] = {"value": round(qbytes / dt / 1e9, 2), "unit": "GB/s", "cores": orc.num_threads(),
+                                                                          "kind": "port", "sample": "the whole [4096, 7168] tensor, %.2f s" % dt}
+                extra["mx_quant_f16_input_cfg1_shape"]["parity"] = {"bit_exact_whole_tensor": bool(np.array_equal(ph_d.cpu().numpy(), ph_h) and
+                                                                                                 np.array_equal(sh_d.cpu().numpy(), sh_h))}
+            del sets16
+            # the same rows quantised once and scattered as packed [payload | scales] rows to their top-2 destinations
+            idx1 = torch.randperm(M1 * 2, device=dev).to(torch.int32)
+            packed1 = torch.empty((M1 * 2, cc.packed_row_bytes(K1)), dtype=torch.uint8, device=dev)
+            st1 = torch.cuda.current_stream().cuda_stream
+            from catccos_amd import _abi as abi1
+
+            def sc_launch(i):
+                abi1.check(abi1.lib().cch_mx_quant_scatter_packed(sets[i % len(sets)].data_ptr(), idx1.data_ptr(), packed1.data_ptr(),
+                                                                  M1, K1, 2, 0, 0, st1))
+
+            for i in range(600):
+                sc_launch(i)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(120):
+                sc_launch(i)
+            e1.record()
+            torch.cuda.synchronize()
+            sc_us = e0.elapsed_time(e1) * 1e3 / 120
+            sc_bytes = M1 * K1 * 2 + 2 * M1 * cc.packed_row_bytes(K1)
+            extra["mx_quant_scatter_top2_cfg1_rows"] = {"gb_per_s": round(sc_bytes / sc_us / 1e3, 1),
+                                                        "frac_of_hbm_peak": round(sc_bytes / sc_us / 1e3 / HBM_PEAK_GBS, 4),
+                                                        "us": round(sc_us, 2), "bytes": sc_bytes}
+            if cpu:
+                sc_launch(0)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                pk_h = orc.mx_quant_scatter_packed(x_h, idx1.cpu().numpy(), M1 * 2, 2, orc.E4M3)
+                dt = time.perf_counter() - t0
+                extra["mx_quant_scatter_top2_cfg1_rows"]["cpu_baseline"] = {"value": round(sc_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": orc.num_threads(),
+                                                                            "kind": "port", "sample": "all 4096 tokens, top-2, %.2f s" % dt}
+                extra["mx_quant_scatter_top2_cfg1_rows"]["parity"] = {"bit_exact_whole_tensor": bool(np.array_equal(packed1.cpu().numpy(), pk_h))}
+            del sets, packed1
+        if only_cfg in (None, "cfg2"):
+            # config 2: int8 W8A8 + dequant
+            m2, k2, n2 = 8192, 4096, 8192
+            a2 = torch.randint(-127, 128, (m2, k2), dtype=torch.int8, device=dev)
+            b2 = torch.randint(-127, 128, (k2, n2), dtype=torch.int8, device=dev)
+            pt2 = torch.rand(m2, device=dev) * 0.019 + 0.001
+            pc2 = torch.rand(n2, device=dev) * 0.019 + 0.001
+            t2 = [queue_time_ms(lambda: cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, TRANS_B), 30, 60.0)]
+            extra["w8a8_dequant_cfg2"] = {"tops": round(2.0 * m2 * n2 * k2 / (np.mean(t2) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t2)) * 1e3, 1)}
+            extra["w8a8_dequant_cfg2"]["frac_of_int8_peak"] = round(extra["w8a8_dequant_cfg2"]["tops"] / FP8_PEAK_TFLOPS, 4)
+            if cpu:
+                o2 = cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, TRANS_B).float().cpu().numpy()
+                a2h, b2h, pt2h, pc2h = a2.cpu().numpy(), b2.cpu().numpy(), pt2.cpu().numpy(), pc2.cpu().numpy()
+                rows, gold, rec = cpu_leg(lambda r: orc.gemm_i8_dequant(a2h, b2h, pt2h, pc2h, TRANS_B, rows=r, blocked=True), 2.0 * m2 * n2 * k2, m2,
+                                          lambda n: np.sort(rng_s.choice(m2, n, replace=False)).astype(np.int64), 6.0, "TOP/s")
+                extra["w8a8_dequant_cfg2"]["cpu_baseline"] = rec
+                extra["w8a8_dequant_cfg2"]["parity"] = parity_record(o2[rows], gold)
+                del o2, a2h, b2h, gold
+            del a2, b2
+        if only_cfg in (None, "cfg3"):
+            # config 3: MXFP8 dense
+            m3, k3, n3 = 4096, 2048, 7168
+            a3, sa3 = cc.mx_quant(torch.randn(m3, k3, device=dev).to(torch.bfloat16), "e4m3")
+            b3, sb3 = cc.mx_quant_b(torch.randn(k3, n3, device=dev).to(torch.bfloat16), "e4m3", trans_b=TRANS_B)
+            t3 = [queue_time_ms(lambda: cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", TRANS_B), 30, 60.0)]
+            extra["mxfp8_dense_cfg3"] = {"tflops": round(2.0 * m3 * n3 * k3 / (np.mean(t3) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t3)) * 1e3, 1)}
+            extra["mxfp8_dense_cfg3"]["frac_of_fp8_peak"] = round(extra["mxfp8_dense_cfg3"]["tflops"] / FP8_PEAK_TFLOPS, 4)
+            if cpu:
+                o3 = cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", TRANS_B).float().cpu().numpy()
+                h3 = [t.cpu().numpy() for t in (a3, sa3, b3, sb3)]
+                rows, gold, rec = cpu_leg(lambda r: orc.mx_gmm(h3[0], h3[1], h3[2], h3[3], n3, k3, orc.E4M3, TRANS_B, rows=r, blocked=True), 2.0 * m3 * n3 * k3, m3,
+                                          lambda n: np.sort(rng_s.choice(m3, n, replace=False)).astype(np.int64), 6.0, "TFLOP/s")
+                extra["mxfp8_dense_cfg3"]["cpu_baseline"] = rec
+                extra["mxfp8_dense_cfg3"]["parity"] = parity_record(o3[rows], gold)
+                del o3, h3, gold
+        if only_cfg in (None, "cfg4"):
+            # config 4: MoE W8A8 grouped + dequant + SwiGLU
+            e4, t4, k4, n4 = 16, 8192, 7168, 4096
+            gs4 = torch.from_numpy(zipf_groups(rng, t4, e4)).to(dev)
+            x4 = torch.randint(-127, 128, (t4, k4), dtype=torch.int8, device=dev)
+            w4 = torch.randint(-127, 128, (e4, k4, n4), dtype=torch.int8, device=dev)
+            pt4 = torch.rand(t4, device=dev) * 0.019 + 0.001
+            pc4 = torch.rand(e4, n4, device=dev) * 0.019 + 0.001
+            tt4 = [queue_time_ms(lambda: cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), 30, 60.0)]
+            extra["moe_w8a8_swiglu_cfg4"] = {"tops": round(2.0 * t4 * n4 * k4 / (np.mean(tt4) * 1e-3) / 1e12, 1), "us": round(float(np.mean(tt4)) * 1e3, 1)}
+            extra["moe_w8a8_swiglu_cfg4"]["frac_of_int8_peak"] = round(extra["moe_w8a8_swiglu_cfg4"]["tops"] / FP8_PEAK_TFLOPS, 4)
+            # the same with the activation leaving as MXFP8 from the epilogue, against the two-kernel chain it replaces
+            tf4 = queue_time_ms(lambda: cc.gmm_dequant_swiglu_mx(x4, w4, gs4, pt4, pc4, TRANS_B, "e4m3"), 30, 60.0)
+            tc4 = queue_time_ms(lambda: cc.mx_quant(cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), "e4m3"), 30, 60.0)
+            pf4, sf4 = cc.gmm_dequant_swiglu_mx(x4, w4, gs4, pt4, pc4, TRANS_B, "e4m3")
+            pq4, sq4 = cc.mx_quant(cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), "e4m3")
+            extra["moe_w8a8_swiglu_mxfp8_out_cfg4"] = {"us": round(tf4 * 1e3, 1), "two_kernel_chain_us": round(tc4 * 1e3, 1),
+                                                       "tops": round(2.0 * t4 * n4 * k4 / (tf4 * 1e-3) / 1e12, 1),
+                                                       "parity": {"bit_exact_vs_quantised_bf16_output": bool(torch.equal(pf4, pq4) and torch.equal(sf4, sq4))}}
+            del pf4, sf4, pq4, sq4
+            if cpu:
+                o4 = cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B).float().cpu().numpy()
+                h4 = [t.cpu().numpy() for t in (x4, w4, gs4, pt4, pc4)]
+                used4 = int(h4[2].sum())
+                rows, gold, rec = cpu_leg(lambda r: orc.gmm_i8_dequant_swiglu(h4[0], h4[1], h4[2], h4[3], h4[4], rows=r, blocked=True), 2.0 * used4 * n4 * k4,
+                                          used4, lambda n: sample_rows(rng_s, h4[2], n), 8.0, "TOP/s")
+                extra["moe_w8a8_swiglu_cfg4"]["cpu_baseline"] = rec
+                extra["moe_w8a8_swiglu_cfg4"]["parity"] = parity_record(o4[rows], gold)
+                extra["moe_w8a8_swiglu_cfg4"]["parity"]["rows_past_the_groups_are_zero"] = bool(np.all(o4[used4:] == 0))
+                del o4, h4, gold
+            del x4, w4
+        if only_cfg is None:
+            # input side of config 4: per-token dynamic int8 quantisation of the bf16 tokens (queued launches through the C ABI)
+            from catccos_amd import _abi
+            xs4 = [torch.randn(t4, k4, device=dev).to(torch.bfloat16) for _ in range(4)]
+            q4 = torch.empty((t4, k4), dtype=torch.int8, device=dev)
+            s4 = torch.empty((t4,), dtype=torch.float32, device=dev)
+            st4 = torch.cuda.current_stream().cuda_stream
+
+            def dq_launch(i):
+                _abi.check(_abi.lib().cch_dyn_quant_i8_rows(xs4[i % 4].data_ptr(), None, q4.data_ptr(), s4.data_ptr(), t4, t4, k4, 1, 0, st4))
+
+            for i in range(800):
+                dq_launch(i)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(60):
+                dq_launch(i)
+            e1.record()
+            torch.cuda.synchronize()
+            dq_us = e0.elapsed_time(e1) * 1e3 / 60
+            dq_bytes = t4 * k4 * 3 + t4 * 4
+            extra["dyn_quant_i8_cfg4_tokens"] = {"gb_per_s": round(dq_bytes / dq_us / 1e3, 1), "frac_of_hbm_peak": round(dq_bytes / dq_us / 1e3 / HBM_PEAK_GBS, 4),
+                                                 "us": round(dq_us, 2), "bytes": dq_bytes}
+            if cpu:
+                dq_launch(0)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                qh, sh = orc.dyn_quant_i8_rows(xs4[0].view(torch.int16).cpu().numpy().view(np.uint16))
+                dt = time.perf_counter() - t0
+                extra["dyn_quant_i8_cfg4_tokens"]["cpu_baseline"] = {"value": round(dq_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": orc.num_threads(),
+                                                                     "kind": "port", "sample": "all 8192 tokens, %.2f s" % dt}
+                extra["dyn_quant_i8_cfg4_tokens"]["parity"] = {"bit_exact_whole_tensor": bool(np.array_equal(q4.cpu().numpy(), qh) and
+                                                                                            np.array_equal(s4.cpu().numpy(), sh))}
+            del xs4, q4
+            # combine side: top-2 weighted un-permute of 8192 expert-output rows back to 4096 tokens
+            tok_u, hid_u, topk_u = 4096, 7168, 2
+            ys = [torch.randn(tok_u * topk_u, hid_u, device=dev).to(torch.bfloat16) for _ in range(3)]
+            idx_u = torch.randperm(tok_u * topk_u, device=dev).to(torch.int32)
+            pr_u = torch.rand(tok_u * topk_u, device=dev)
+            out_u = torch.empty((tok_u, hid_u), dtype=torch.bfloat16, device=dev)
+
+            def un_launch(i):
+                _abi.check(_abi.lib().cch_moe_token_unpermute(ys[i % 3].data_ptr(), idx_u.data_ptr(), pr_u.data_ptr(), out_u.data_ptr(),
+                                                              tok_u * topk_u, tok_u, hid_u, topk_u, st4))
+
+            for i in range(600):
+                un_launch(i)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(60):
+                un_launch(i)
+            e1.record()
+            torch.cuda.synchronize()
+            un_us = e0.elapsed_time(e1) * 1e3 / 60
+            un_bytes = tok_u * topk_u * hid_u * 2 + tok_u * hid_u * 2 + tok_u * topk_u * 8
+            extra["moe_token_unpermute_top2"] = {"gb_per_s": round(un_bytes / un_us / 1e3, 1), "frac_of_hbm_peak": round(un_bytes / un_us / 1e3 / HBM_PEAK_GBS, 4),
+                                                 "us": round(un_us, 2), "bytes": un_bytes}
+            if cpu:
+                un_launch(0)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                uh = orc.moe_token_unpermute(ys[0].view(torch.int16).cpu().numpy().view(np.uint16), idx_u.cpu().numpy(), pr_u.cpu().numpy(), topk_u)
+                dt = time.perf_counter() - t0
+                extra["moe_token_unpermute_top2"]["cpu_baseline"] = {"value": round(un_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": orc.num_threads(),
+                                                                     "kind": "port", "sample": "all 4096 tokens, %.2f s" % dt}
+                extra["moe_token_unpermute_top2"]["parity"] = {"bit_exact_whole_tensor": bool(np.array_equal(
+                    out_u.view(torch.int16).cpu().numpy().view(np.uint16), uh))}
+            del ys, out_u
+            # routing sort of config 4's routes (8192 tokens, top-2, 16 experts): three short launches through the C ABI
+            rt_rows, rt_e = 8192 * 2, 16
+            rt_idx = torch.randint(0, rt_e, (rt_rows,), dtype=torch.int32, device=dev)
+            rt_d2s = torch.empty(rt_rows, dtype=torch.int32, device=dev)
+            rt_s2d = torch.empty_like(rt_d2s)
+            rt_cnt = torch.empty(rt_e, dtype=torch.int32, device=dev)
+            rt_wsb = int(_abi.lib().cch_moe_init_routing_workspace_bytes(rt_rows, rt_e))
+            rt_ws = torch.empty(max(rt_wsb, 4), dtype=torch.uint8, device=dev)
+
+            def rt_launch():
+                _abi.check(_abi.lib().cch_moe_init_routing(rt_idx.data_ptr(), rt_rows, rt_e, rt_d2s.data_ptr(), rt_s2d.data_ptr(),
+                                                           rt_cnt.data_ptr(), 0, rt_ws.data_ptr(), rt_wsb, st4))
+
+            for _ in range(200):
+                rt_launch()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(100):
+                rt_launch()
+            e1.record()
+            torch.cuda.synchronize()
+            extra["moe_init_routing_cfg4_routes"] = {"us": round(e0.elapsed_time(e1) * 1e3 / 100, 2), "routes": rt_rows, "experts": rt_e,
+                                                     "launches_per_call": 3}
+            if cpu:
+                t0 = time.perf_counter()
+                d2s_h, s2d_h, cnt_h = orc.moe_init_routing(rt_idx.cpu().numpy(), rt_e)
+                dt = time.perf_counter() - t0
+                extra["moe_init_routing_cfg4_routes"]["cpu_baseline"] = {"value": round(dt * 1e6, 1), "unit": "us", "cores": 1, "kind": "port",
+                                                                         "sample": "all 16384 routes (numpy stable argsort and bincount)"}
+                extra["moe_init_routing_cfg4_routes"]["parity"] = {"bit_exact_whole_tensor": bool(
+                    np.array_equal(rt_d2s.cpu().numpy(), d2s_h) and np.array_equal(rt_s2d.cpu().numpy(), s2d_h) and np.array_equal(rt_cnt.cpu().numpy(), cnt_h))}
+        if only_cfg in (None, "cfg5"):
+            # config 5: MXFP4 grouped (same groups as the headline)
+            a5, sa5 = cc.mx_quant((torch.randn(T, K, device=dev) * 0.02).to(torch.bfloat16), "e2m1")
+            b5 = torch.empty((E, K, N // 2), dtype=torch.uint8, device=dev)
+            sb5 = torch.empty((E, K // 64, N, 2), dtype=torch.uint8, device=dev)
+            for e in range(E):
+                b5[e], sb5[e] = cc.mx_quant_b((torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16), "e2m1", trans_b=TRANS_B)
+            t5 = [queue_time_ms(lambda: cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", TRANS_B), 30, 60.0)]
+            extra["mxfp4_grouped_cfg5"] = {"tflops": round(flop / (np.mean(t5) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t5)) * 1e3, 1)}
+            extra["mxfp4_grouped_cfg5"]["frac_of_fp4_peak"] = round(extra["mxfp4_grouped_cfg5"]["tflops"] / FP4_PEAK_TFLOPS, 4)
+            if cpu:
+                o5 = cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", TRANS_B).float().cpu().numpy()
+                h5 = [t.cpu().numpy() for t in (a5, sa5, b5, sb5)]
+                used5 = int(gs_host.sum())
+                rows, gold, rec = cpu_leg(lambda r: orc.mx_gmm(h5[0], h5[1], h5[2], h5[3], N, K, orc.E2M1, TRANS_B, group_sizes=gs_host, rows=r, blocked=True),
+                                          2.0 * used5 * N * K, used5, lambda n: sample_rows(rng_s, gs_host, n), 10.0, "TFLOP/s")
+                extra["mxfp4_grouped_cfg5"]["cpu_baseline"] = rec
+                extra["mxfp4_grouped_cfg5"]["parity"] = parity_record(o5[rows], gold)
+                del o5, h5, gold
+            del a5, sa5, b5, sb5
+        if only_cfg is None:
+            # Yardstick, not part of this build: the vendor library's dense FP8 GEMM (per-tensor scales, E4M3,
+            # bf16 out) on the headline's shape as one group, and this kernel on the same bytes with unit scales.
+            try:
+                ya = (torch.randn(T, K, device=dev) * 0.5).to(torch.float8_e4m3fn)
+                yb = (torch.randn(N, K, device=dev) * 0.5).to(torch.float8_e4m3fn)
+                one = torch.tensor(1.0, device=dev)
+                t_lib = queue_time_ms(lambda: torch._scaled_mm(ya, yb.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16), 100, 150.0)
+                ysa = torch.full((T, K // 32), 127, dtype=torch.uint8, device=dev)
+                ysb = torch.full((N, K // 32), 127, dtype=torch.uint8, device=dev)
+                t_own = queue_time_ms(lambda: cc.mx_matmul(ya.view(torch.uint8), ysa, yb.view(torch.uint8), ysb, "e4m3", 1), 100, 150.0)
+                extra["yardstick_dense_fp8_16384x4096x7168"] = {
+                    "library_scaled_mm_tflops": round(flop / (t_lib * 1e-3) / 1e12, 1), "this_kernel_same_data_tflops": round(flop / (t_own * 1e-3) / 1e12, 1),
+                    "note": "library = torch._scaled_mm (per-tensor scales); both with B as [N,K]"}
+            except Exception as exc:   # the library call is optional: a box without it still reports everything else
+                extra["yardstick_dense_fp8_16384x4096x7168"] = {"error": repr(exc)[:200]}
         result["extra"] = extra
 
     print(json.dumps(result), flush=True)

@@ -2,6 +2,7 @@
 
     python -m catccos_amd.build            # everything
     python -m catccos_amd.build --only lib
+    python -m catccos_amd.build --only lib --define CCH_V_NOLOAD --out /tmp/noload   # a measurement build of the GEMM kernels
 
 Outputs (git-ignored, shipped as built files):
     catccos_amd/libcatccos_hip.so      C ABI + HIP kernels   (include/catccos_hip.h)
@@ -43,19 +44,25 @@ def _run(cmd):
         print(out, file=sys.stderr)
 
 
-def _compile(src):
-    os.makedirs(OBJ, exist_ok=True)
-    obj = os.path.join(OBJ, os.path.basename(src) + ".o")
-    _run([HIPCC] + HIP_FLAGS + ["-c", src, "-o", obj])
+def _compile(src, defines=(), obj_dir=None):
+    obj_dir = obj_dir or OBJ
+    os.makedirs(obj_dir, exist_ok=True)
+    obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
+    _run([HIPCC] + HIP_FLAGS + ["-D" + d for d in defines] + ["-c", src, "-o", obj])
     return obj
 
 
-def build_lib(jobs=8):
+def build_lib(jobs=8, defines=(), out_dir=None):
+    """The shipped library, or (with `defines` and `out_dir`) a measurement build of it in a directory of its own."""
+    if defines and not out_dir:
+        raise ValueError("a build with extra defines needs --out: it must not replace the shipped library")
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    obj_dir = os.path.join(out_dir, "obj") if out_dir else None
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(_compile, srcs))
-    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
-    return LIB
+        objs = list(ex.map(lambda src: _compile(src, defines, obj_dir), srcs))
+    lib = os.path.join(out_dir, "libcatccos_hip.so") if out_dir else LIB
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs)
+    return lib
 
 
 def build_host():
@@ -83,8 +90,10 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--only", choices=["lib", "host"])
     ap.add_argument("-j", type=int, default=8)
+    ap.add_argument("--define", action="append", default=[], metavar="NAME", help="extra -D for the HIP sources (needs --out)")
+    ap.add_argument("--out", metavar="DIR", help="directory for a library built with --define")
     a = ap.parse_args()
     if a.only in (None, "lib"):
-        print(build_lib(a.j))
+        print(build_lib(a.j, a.define, a.out))
     if a.only in (None, "host"):
         print(build_host())

@@ -119,15 +119,6 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 
 // Workgroup barrier that the compiler moves no memory access across (the intrinsic alone is not a
 // memory barrier to the optimiser) and that the instruction scheduler leaves where it is.
-#ifndef CCH_PRIO_C
-#define CCH_PRIO_C 1
-#define CCH_PRIO_L 0
-#endif
-#ifdef CCH_V_NOPRIO
-#define CCH_SETPRIO(n)
-#else
-#define CCH_SETPRIO(n) __builtin_amdgcn_s_setprio(n)
-#endif
 #define CCH_BARRIER()                                  \
     do {                                               \
         __builtin_amdgcn_sched_barrier(0);             \
@@ -213,8 +204,15 @@ __device__ __forceinline__ uint32_t lds_read4_abs(uint32_t addr)
 // c ^ ((row >> 1) & 7), which spreads 16 consecutive rows over all 64 banks for 16-byte reads.
 __device__ __forceinline__ uint32_t swizzle_of_row(int row) { return (uint32_t)((row >> 1) & 7); }
 
+// Measurement builds of this file (never the shipped library; results are wrong or slower):
+//   -DCCH_PROF       every wave counts the shader cycles it spends in each wait and barrier of the
+//                    K loop; cch_prof_read() copies the counters out (per workgroup and wave: total,
+//                    then the seven waits in program order);
+//   -DCCH_V_NOLOAD   no panel requests: matrix instructions and LDS reads alone (the MFMA-side ceiling);
+//   -DCCH_V_NOMFMA   no matrix instructions after a tile's first step: requests, LDS reads, waits and
+//                    barriers alone (the memory-side ceiling).
+// `python -m catccos_amd.build --only lib --define NAME --out DIR` builds one.
 #ifdef CCH_PROF
-// Instrumented build: cycles per wave spent in the waits and barriers of the K loop.
 __device__ uint64_t cch_prof[256 * 8 * 8];
 #define PROF_BEGIN(t) const uint64_t t = __builtin_readcyclecounter()
 #define PROF_END(t, acc) acc += __builtin_readcyclecounter() - t
@@ -641,18 +639,12 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 
         auto frag_a = [&](auto stg_c, int ks, int i) {
             constexpr int STG = decltype(stg_c)::value;
-#ifdef CCH_V_NOLDS
-            return (v8i){ks, i, 0, 0, 0, 0, 0, 0};
-#endif
             const v4i lo = lds_read16_abs(fr_a[ks * 2] + (uint32_t)(STG * PANEL_BYTES + i * 32 * BKB));
             const v4i hi = lds_read16_abs(fr_a[ks * 2 + 1] + (uint32_t)(STG * PANEL_BYTES + i * 32 * BKB));
             return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         };
         auto frag_b = [&](auto stg_c, int ks, int j) {
             constexpr int STG = decltype(stg_c)::value;
-#ifdef CCH_V_NOLDS
-            return (v8i){ks, j, 0, 0, 0, 0, 0, 0};
-#endif
             if constexpr (TB) {
                 const v4i lo = lds_read16_abs(fr_b[ks * 2] + (uint32_t)(STG * PANEL_BYTES + j * 32 * BKB));
                 const v4i hi = lds_read16_abs(fr_b[ks * 2 + 1] + (uint32_t)(STG * PANEL_BYTES + j * 32 * BKB));
@@ -687,9 +679,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // bytes 0 and 2, where the matrix instruction's byte selector finds them.
         uint32_t raw_lo[NSC][MT + NT], raw_hi[NSC][MT + NT];
         auto read_scales_raw = [&]() {
-#ifdef CCH_V_NOSCALE
-            return;
-#endif
             if constexpr (MX) {
 #pragma unroll
                 for (int d = 0; d < SCALE_DW; d++) {
@@ -714,10 +703,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             }
         };
         auto finish_scales = [&](auto last_c, int kt) {
-#ifdef CCH_V_NOSCALE
-            for (int d = 0; d < NSC; d++) for (int s = 0; s < MT + NT; s++) sc[d][s] = 0x7f7f7f7fu;
-            return;
-#endif
             if constexpr (MX) {
                 constexpr bool LAST = decltype(last_c)::value != 0;
                 const int nblk = (p.K + 31) >> 5;
@@ -846,7 +831,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             Tail rq_tl;
             uint32_t rq_boff = 0;
             if constexpr (MTH > 0) {
-                CCH_SETPRIO(CCH_PRIO_C);
                 mfma_block(IC<FIRST>{}, IC<0>{}, IC<0>{}, fa[0][0]);
                 __builtin_amdgcn_sched_barrier(0);
                 rq_tl = tail_of(rq_kt);
@@ -859,7 +843,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 __builtin_amdgcn_sched_barrier(0);
                 mfma_block(IC<0>{}, IC<1>{}, IC<0>{}, fa[0][1]);
                 mfma_block(IC<0>{}, IC<1>{}, IC<1>{}, fa[1][1]);
-                CCH_SETPRIO(CCH_PRIO_L);
             } else {
                 rq_tl = tail_of(rq_kt);
                 if constexpr (!TB) rq_boff = boff_of(rq_kt);
@@ -905,7 +888,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b2); }
             // ------------------------------------------------------------------ C1
             if constexpr (MTH > 1) {
-                CCH_SETPRIO(CCH_PRIO_C);
                 mfma_block(IC<FIRST>{}, IC<0>{}, IC<2>{}, fa[0][0]);
                 __builtin_amdgcn_sched_barrier(0);
                 issue_b(rq, rq_tl, rq_boff, stg_c, IC<2>{});
@@ -916,7 +898,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 __builtin_amdgcn_sched_barrier(0);
                 mfma_block(IC<0>{}, IC<1>{}, IC<2>{}, fa[0][1]);
                 mfma_block(IC<0>{}, IC<1>{}, IC<3>{}, fa[1][1]);
-                CCH_SETPRIO(CCH_PRIO_L);
             } else {
                 issue_b(rq, rq_tl, rq_boff, stg_c, IC<2>{});
                 issue_b(rq, rq_tl, rq_boff, stg_c, IC<3>{});
