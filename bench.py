@@ -27,10 +27,10 @@ sys.path.insert(0, ROOT)
 FP8_PEAK_TFLOPS = 5000.0   # MI355X dense FP8 / INT8 MFMA, published
 FP4_PEAK_TFLOPS = 10100.0  # MI355X dense FP4 MFMA, published
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
-# Bytes per launch of the headline kernel at the L2 <-> memory interface, from two rocprofv3 --pmc runs
-# of this script (FETCH_SIZE 1 018 123 KiB x 2.000, WRITE_SIZE 131 072 KiB x 1.000; the factors are what
-# the same counters read for a 512 MiB device copy, `--only copy`).  Algorithmic bytes: 1 224 212 480.
-GMM_TRAFFIC_BYTES = 2219333632
+# Bytes per launch of the headline kernel between the L2s and the fabric (Infinity Cache and HBM behind it), from two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE 1 071 743 KiB x 2.000, WRITE_SIZE 131 072 KiB x 1.000; the factors are
+# what the same counters read for a 512 MiB device copy, `--only copy`).  Algorithmic bytes: 1 224 212 480.
+GMM_TRAFFIC_BYTES = 2329147392
 
 
 def zipf_groups(rng, t, e):
@@ -328,7 +328,7 @@ def main():
                        "n": N, "trans_b": TRANS_B, "group_sizes": gs_host.tolist()},
             "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(achieved / FP8_PEAK_TFLOPS, 4), "traffic": GMM_TRAFFIC_BYTES,
-                         "kernel": "gemm_tile_kernel<KIND_F8, EPI_PLAIN, E4M3, TB=0>", "algorithmic_flop_per_launch": flop,
+                         "kernel": "gemm_tile_kernel<KIND_F8, EPI_PLAIN, E4M3, TB=0, UA=0>", "algorithmic_flop_per_launch": flop,
                          "kernel_ms_min": round(float(np.min(per_ms)), 4), "kernel_ms_median": round(float(np.median(per_ms)), 4),
                          "kernel_ms_mean": round(kernel_ms, 4), **clk},
         }
