@@ -47,5 +47,10 @@ def test_ops_need_init_then_match_the_oracle():
         pc = rng.uniform(0.001, 0.02, (e, n)).astype(np.float32)
         close(OPS.gmm_dequant_swiglu(dev(xi), dev(wi), dev(gs), dev(pt), dev(pc), 0), orc.gmm_i8_dequant_swiglu(xi, wi, gs, pt, pc))
         close(OPS.w8a8_matmul_dequant(dev(xi), dev(wi[0]), dev(pt), dev(pc[0]), 0), orc.gemm_i8_dequant(xi, wi[0], pt, pc[0]))
+        act = OPS.gmm_dequant_swiglu(dev(xi), dev(wi), dev(gs), dev(pt), dev(pc), 0)
+        pq, sq = OPS.gmm_dequant_swiglu_mx(dev(xi), dev(wi), dev(gs), dev(pt), dev(pc), 0, "e4m3")
+        torch.cuda.synchronize()
+        want_p, want_s = orc.mx_quant_rows(act.view(torch.int16).cpu().numpy().view(np.uint16), orc.E4M3)
+        assert np.array_equal(pq.cpu().numpy(), want_p) and np.array_equal(sq.cpu().numpy(), want_s)
     finally:
         assert OPS.finalize() == 0

@@ -17,7 +17,7 @@ def initialised():
 
 
 def test_schemas_are_registered():
-    for name in ("init", "finalize", "mx_quant", "w8a8_matmul_dequant", "mx_matmul", "gmm_dequant_swiglu", "mx_grouped_matmul"):
+    for name in ("init", "finalize", "mx_quant", "w8a8_matmul_dequant", "mx_matmul", "gmm_dequant_swiglu", "mx_grouped_matmul", "gmm_dequant_swiglu_mx"):
         assert hasattr(OPS, name), name
     assert str(OPS.init.default._schema) == "catccos::init(int rank_id, int rank_size, int local_mem_size, str ip_port) -> int"
     assert str(OPS.finalize.default._schema) == "catccos::finalize() -> int"
@@ -52,6 +52,9 @@ def test_meta_shapes(initialised):
         out = OPS.gmm_dequant_swiglu(a, w, torch.empty(e, dtype=torch.int32, device="meta"), torch.empty(m, device="meta"),
                                      torch.empty((e, n), device="meta"), tb)
         assert out.shape == (m, n // 2) and out.dtype == torch.bfloat16
+        pq, sq = OPS.gmm_dequant_swiglu_mx(a, w, torch.empty(e, dtype=torch.int32, device="meta"), torch.empty(m, device="meta"),
+                                           torch.empty((e, n), device="meta"), tb, "e2m1")
+        assert pq.shape == (m, n // 4) and sq.shape == (m, 2 * ((n // 2 + 63) // 64)) and pq.dtype == sq.dtype == torch.uint8
     k = 1024
     u8 = lambda *shape: torch.empty(shape, dtype=torch.uint8, device="meta")   # noqa: E731
     assert OPS.mx_matmul(u8(m, k), u8(m, 32), u8(k, n), u8(16, n, 2), "e4m3", 0).shape == (m, n)
