@@ -372,7 +372,8 @@ def mx_grouped_matmul_mapped(a, sa, b, sb, group_sizes, out_row_map, out, fmt="e
         raise ValueError("out_row_map must hold one int32 entry per row of a")
     if out.dim() != 2 or out.dtype not in (torch.bfloat16, torch.float16) or out.shape[1] != n or not out.is_contiguous():
         raise ValueError("out must be a contiguous bfloat16 or float16 [rows, %d] tensor" % n)
-    check(_abi.lib().cch_mx_gmm_mapped(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(group_sizes), _ptr(out_row_map.contiguous()),
+    row_map = out_row_map.contiguous()   # held until the launch is queued (a strided map becomes a copy)
+    check(_abi.lib().cch_mx_gmm_mapped(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(group_sizes), _ptr(row_map),
                                        _ptr(out), out.shape[0], 1 if out.dtype == torch.float16 else 0, e, t, n, k, fmt,
                                        int(trans_b), _stream()))
     return out

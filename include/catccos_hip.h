@@ -316,6 +316,10 @@ int cch_dyn_quant_i8_rows_smooth(const void *x, const int32_t *src_rows, const f
  * 3-4 % faster (no difference for the others); "quant_integer_encoder" = 1 runs the E4M3
  * round-to-nearest-even quantiser through the integer encoder instead of the hardware conversion (an
  * on-device cross-check; same bytes).  Results do not depend on any of them.
+ * The tiled MFMA kernels take every problem whose rows of K are a multiple of 16 bytes, with
+ * n % 8 == 0 (and, for [K,N] operands, rows of B a multiple of 4 bytes), 16-byte aligned operands
+ * below 2 GiB each and MX scale arrays back to back.  The generic kernels take everything else up to
+ * 65535 rows per call (more is CCH_ENOSUP).
  * When a GEMM entry point falls back from the tiled MFMA kernels to the one-thread-per-element
  * kernels (orders of magnitude slower), the call still returns CCH_OK, cch_last_error() names the
  * precondition that failed, and the first such call of the process prints one line to stderr. */

@@ -121,7 +121,7 @@ def test_mx_gemm(fmt, shape, trans_b, path):
     (examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/test_shapes.csv)."""
     m, n, k = shape
     if path == 1 and m * n * k > 3e8:
-        pytest.skip("generic path: keep the run short")
+        m = max(8, int(3e8 / (n * k)))   # generic path (one thread per output): fewer rows of the same N and K keep the run short
     rng = np.random.default_rng(m * 7 + n * 3 + k)
     pa, sa, pb, sb = mx_operands(rng, m, n, k, fmt, trans_b)
     want = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], trans_b)
@@ -190,7 +190,8 @@ def test_mx_gemm_scale_extremes():
 def test_mx_gmm(fmt, cfg, trans_b, path):
     e, t, n, k, gs = cfg
     if path == 1 and t * n * k > 3e8:
-        pytest.skip("generic path: keep the run short")
+        assert gs is None
+        t = max(4 * e, int(3e8 / (n * k)))   # generic path: fewer tokens over the same experts keep the run short
     rng = np.random.default_rng(e + t + n + k)
     gs = zipf_groups(rng, t - 5, e) if gs is None else np.array(gs, np.int32)
     sigma = 0.02 if fmt == "e2m1" else 1.0
