@@ -93,7 +93,8 @@ def parity_record(got, gold):
 
 
 def event_time_ms(fn, steps, warmup, warm_ms=0.0):
-    """Mean and per-launch durations of fn() on the current stream, by HIP events.
+    """Wall time per step, average launch duration over the timed region and per-launch durations of fn()
+    on the current stream, the latter two by HIP events.
 
     The shader clock needs some tens of milliseconds of load to reach its steady state (launch
     durations fall by 15-20 % over the first 50 ms after an idle period), so the untimed part must
@@ -108,17 +109,27 @@ def event_time_ms(fn, steps, warmup, warm_ms=0.0):
         for _ in range(10):
             fn()
         torch.cuda.synchronize()
+    # the timed region: exactly `steps` launches queued back to back between one pair of events
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    region = e0.elapsed_time(e1) / steps
+    # the same launches again, each between its own events: the spread (an event pair adds about 1 %)
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    t0 = time.perf_counter()
     for i in range(steps):
         starts[i].record()
         fn()
         ends[i].record()
     torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) * 1e3 / steps
     per = [s.elapsed_time(e) for s, e in zip(starts, ends)]
-    return wall, per
+    return wall, region, per
 
 
 def clock_under_load(fn, seconds=1.5):
@@ -246,7 +257,7 @@ def main():
     if args.only == "copy":
         src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).fill_(7)
         dst = torch.empty_like(src)
-        _, ms = event_time_ms(lambda: dst.copy_(src), args.steps, args.warmup)
+        _, _, ms = event_time_ms(lambda: dst.copy_(src), args.steps, args.warmup)
         print(json.dumps({"only": "copy", "bytes_read": src.numel(), "bytes_written": src.numel(), "ms": float(np.mean(ms))}))
         return
     if args.only == "quant":
@@ -286,8 +297,7 @@ def main():
             out[0] = cc.mx_grouped_matmul(a, sa, b, sb, gs, "e4m3", TRANS_B)
 
         # `warmup` launches as asked for, then more of the same until the shader clock has settled (see event_time_ms)
-        wall_ms, per_ms = event_time_ms(step, args.steps, args.warmup, warm_ms=100.0)
-        kernel_ms = float(np.mean(per_ms))
+        wall_ms, kernel_ms, per_ms = event_time_ms(step, args.steps, args.warmup, warm_ms=100.0)
         flop = 2.0 * T * N * K
         value = flop / (wall_ms * 1e-3) / 1e12
         achieved = flop / (kernel_ms * 1e-3) / 1e12
@@ -330,7 +340,7 @@ def main():
                          "frac": round(achieved / FP8_PEAK_TFLOPS, 4), "traffic": GMM_TRAFFIC_BYTES,
                          "kernel": "gemm_tile_kernel<KIND_F8, EPI_PLAIN, E4M3, TB=0, UA=0>", "algorithmic_flop_per_launch": flop,
                          "kernel_ms_min": round(float(np.min(per_ms)), 4), "kernel_ms_median": round(float(np.median(per_ms)), 4),
-                         "kernel_ms_mean": round(kernel_ms, 4), **clk},
+                         "kernel_ms_mean": round(kernel_ms, 4), "kernel_ms_mean_single_launches": round(float(np.mean(per_ms)), 4), **clk},
         }
 
         # ------------------------------------------------------------ CPU baseline on a bounded sample of rows
