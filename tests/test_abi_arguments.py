@@ -28,6 +28,9 @@ def test_quantiser_arguments():
     rejected(L.cch_mx_quant_scatter_packed(P, P, P, 4, 64, -1, 0, 0, None), "top_k")
     assert L.cch_mx_quant_scatter_packed(P, P, P, 4, 64, 0, 0, 0, None) == _abi.OK   # no routes: nothing to do
     rejected(L.cch_mx_quant_scatter_packed(P, P, P, 4, 64, 9, 0, 0, None), "top_k")
+    rejected(L.cch_mx_quant_scatter_packed_rows(P, P, P, -1, 4, 64, 2, 0, 0, None), "out_rows")
+    rejected(L.cch_mx_quant_scatter_packed_rows(P, P, P, 8, 4, 64, 2, 9, 0, None), "format")
+    assert L.cch_mx_quant_scatter_packed_rows(P, P, P, 8, 0, 64, 2, 0, 0, None) == _abi.OK   # no tokens
 
 
 def test_dynamic_quantiser_arguments():
@@ -55,6 +58,13 @@ def test_gemm_arguments():
     rejected(L.cch_gmm_i8_dequant(P, P, P, P, P, P, 257, 8, 8, 8, 0, None), "num_experts", "256")
     rejected(L.cch_gmm_i8_dequant_swiglu(P, P, P, P, P, P, 257, 8, 8, 8, 0, None), "num_experts", "256")
     rejected(L.cch_mx_gmm(P, P, P, P, P, P, 257, 8, 8, 64, 0, 0, None), "num_experts", "256")
+    # SwiGLU with MX-quantised output: payload formats E4M3, E5M2, E2M1; n even (FP4: a multiple of 4)
+    rejected(L.cch_gmm_i8_dequant_swiglu_mx(P, P, P, P, P, P, P, 2, 8, 8, 8, 0, 3, None), "fmt")
+    rejected(L.cch_gmm_i8_dequant_swiglu_mx(P, P, P, P, P, P, P, 2, 8, 7, 8, 0, 0, None), "even")
+    rejected(L.cch_gmm_i8_dequant_swiglu_mx(P, P, P, P, P, P, P, 2, 8, 6, 8, 0, 2, None), "FP4")
+    rejected(L.cch_gmm_i8_dequant_swiglu_mx(P, P, P, P, P, P, P, 257, 8, 8, 8, 0, 0, None), "num_experts", "256")
+    rejected(L.cch_gmm_i8_dequant_swiglu_mx(P, P, P, P, P, P, None, 2, 8, 8, 8, 0, 0, None), "null")
+    assert L.cch_gmm_i8_dequant_swiglu_mx(None, None, None, None, None, None, None, 2, 0, 8, 8, 0, 0, None) == _abi.OK   # no rows
     rejected(L.cch_mx_gmm_mapped(P, P, P, P, P, P, P, 8, 0, 257, 8, 8, 64, 0, 0, None), "num_experts", "256")
     rejected(L.cch_mx_gemm(P, P, P, P, P, 8, 8, 64, 7, 0, None))           # format
     rejected(L.cch_mx_gemm(P, P, P, P, P, 8, 7, 64, 2, 0, None), "FP4")   # FP4 packs two columns per byte
