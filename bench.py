@@ -624,6 +624,18 @@ def main():
                 del o5, h5, gold
             del a5, sa5, b5, sb5
         if only_cfg is None:
+            # the headline's operands as the up projection of the MX FFN chain: SwiGLU on the bf16 tile in the epilogue, and the
+            # same with the activation leaving as MXFP8 (what the down projection reads), against the kernel chain it replaces
+            tu = queue_time_ms(lambda: cc.mx_grouped_matmul_swiglu(a, sa, b, sb, gs, "e4m3", TRANS_B), 30, 60.0)
+            tq = queue_time_ms(lambda: cc.mx_grouped_matmul_swiglu(a, sa, b, sb, gs, "e4m3", TRANS_B, out_fmt="e4m3"), 30, 60.0)
+            tch = queue_time_ms(lambda: cc.mx_quant(cc.mx_grouped_matmul_swiglu(a, sa, b, sb, gs, "e4m3", TRANS_B), "e4m3"), 30, 60.0)
+            pu, su = cc.mx_grouped_matmul_swiglu(a, sa, b, sb, gs, "e4m3", TRANS_B, out_fmt="e4m3")
+            pv, sv = cc.mx_quant(cc.mx_grouped_matmul_swiglu(a, sa, b, sb, gs, "e4m3", TRANS_B), "e4m3")
+            extra["mxfp8_up_projection_swiglu_headline_shapes"] = {
+                "bf16_out_us": round(tu * 1e3, 1), "mxfp8_out_us": round(tq * 1e3, 1), "two_kernel_chain_us": round(tch * 1e3, 1),
+                "tflops_mxfp8_out": round(flop / (tq * 1e-3) / 1e12, 1),
+                "parity": {"bit_exact_vs_quantised_bf16_output": bool(torch.equal(pu, pv) and torch.equal(su, sv))}}
+            del pu, su, pv, sv
             # Yardstick, not part of this build: the vendor library's dense FP8 GEMM (per-tensor scales, E4M3,
             # bf16 out) on the headline's shape as one group, and this kernel on the same bytes with unit scales.
             try:

@@ -9,7 +9,10 @@
 namespace cch {
 
 enum GemmKind { KIND_I8 = 0, KIND_F8 = 1, KIND_F4 = 2 };
-enum GemmEpilogue { EPI_PLAIN = 0, EPI_DEQUANT = 1, EPI_DEQUANT_SWIGLU = 2 };
+// EPI_SWIGLU (MX kinds): the accumulators are rounded to bf16, then out = silu(gate) * up on those values,
+// as the reference's up projection hands its bf16 tile to the SwiGLU stage
+// (include/catccos/epilogue/block/block_epilogue_regbase_swiglu.hpp:38-80)
+enum GemmEpilogue { EPI_PLAIN = 0, EPI_DEQUANT = 1, EPI_DEQUANT_SWIGLU = 2, EPI_SWIGLU = 3 };
 
 constexpr int MAX_GROUPS = 256;
 

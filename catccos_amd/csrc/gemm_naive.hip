@@ -83,7 +83,12 @@ __global__ __launch_bounds__(256) void gemm_naive_kernel(GemmProblem p)
     }
     float v = 0.0f;
     if (e < p.num_groups) {
-        if (EPI == EPI_DEQUANT_SWIGLU) {
+        if (EPI == EPI_SWIGLU) {
+            // gate and up as the bf16 tile of the up projection, then the activation in fp32
+            const float g = bf16_bits_to_f32(f32_to_bf16_bits(dot_column<KIND>(p, row, e, col)));
+            const float u = bf16_bits_to_f32(f32_to_bf16_bits(dot_column<KIND>(p, row, e, col + p.n_out)));
+            v = g / (1.0f + expf(-g)) * u;
+        } else if (EPI == EPI_DEQUANT_SWIGLU) {
             float g = dot_column<KIND>(p, row, e, col) * p.per_ch[(size_t)e * p.N + col];
             float u = dot_column<KIND>(p, row, e, col + p.n_out) * p.per_ch[(size_t)e * p.N + col + p.n_out];
             g *= p.per_tok[row];
@@ -98,10 +103,10 @@ __global__ __launch_bounds__(256) void gemm_naive_kernel(GemmProblem p)
     p.out[out_row * p.n_out + col] = p.out_fp16 ? __builtin_bit_cast(uint16_t, (_Float16)v) : (uint16_t)f32_to_bf16_bits(v);
 }
 
-// The grouped int8 GEMM with dequantisation and SwiGLU whose activation leaves MX-quantised: what the
-// row quantiser makes of the bf16 output of the kernel above, without the bf16 tensor in between.
-// 32 neighbouring lanes hold one block of a row (the last block of a row may be shorter).
-template <int FMT>
+// The grouped GEMMs with SwiGLU (int8 with dequantisation, or MX) whose activation leaves MX-quantised:
+// what the row quantiser makes of the bf16 output of the kernel above, without the bf16 tensor in
+// between.  32 neighbouring lanes hold one block of a row (the last block of a row may be shorter).
+template <int KIND, int FMT>
 __global__ __launch_bounds__(256) void gemm_naive_swiglu_mx_kernel(GemmProblem p)
 {
     using T = FmtTraits<FMT>;
@@ -114,11 +119,17 @@ __global__ __launch_bounds__(256) void gemm_naive_swiglu_mx_kernel(GemmProblem p
     const int e = find_group(tab, p.num_groups, row);
     float v = 0.0f;
     if (live && e < p.num_groups) {
-        float g = dot_column<KIND_I8>(p, row, e, col) * p.per_ch[(size_t)e * p.N + col];
-        float u = dot_column<KIND_I8>(p, row, e, col + p.n_out) * p.per_ch[(size_t)e * p.N + col + p.n_out];
-        g *= p.per_tok[row];
-        u *= p.per_tok[row];
-        v = g * (1.0f / (1.0f + expf(-g))) * u;
+        if (KIND == KIND_I8) {
+            float g = dot_column<KIND>(p, row, e, col) * p.per_ch[(size_t)e * p.N + col];
+            float u = dot_column<KIND>(p, row, e, col + p.n_out) * p.per_ch[(size_t)e * p.N + col + p.n_out];
+            g *= p.per_tok[row];
+            u *= p.per_tok[row];
+            v = g * (1.0f / (1.0f + expf(-g))) * u;
+        } else {
+            const float g = bf16_bits_to_f32(f32_to_bf16_bits(dot_column<KIND>(p, row, e, col)));
+            const float u = bf16_bits_to_f32(f32_to_bf16_bits(dot_column<KIND>(p, row, e, col + p.n_out)));
+            v = g / (1.0f + expf(-g)) * u;
+        }
     }
     const uint32_t h = live ? f32_to_bf16_bits(v) : 0u;
     uint32_t amax = h & 0x7FFFu;
@@ -157,19 +168,28 @@ static int launch_naive_t(const GemmProblem &p, hipStream_t stream)
 int launch_gemm_naive(const GemmProblem &p, int kind, int epi, hipStream_t stream)
 {
     if (p.mx_out) {
-        if (kind != KIND_I8 || epi != EPI_DEQUANT_SWIGLU) return fail(CCH_ENOSUP, "MX-quantised output exists for the int8 SwiGLU epilogue only");
+        if (epi != EPI_DEQUANT_SWIGLU && epi != EPI_SWIGLU) return fail(CCH_ENOSUP, "MX-quantised output exists for the SwiGLU epilogues only");
         if (p.T == 0 || p.n_out == 0) return CCH_OK;
         if (p.T > 65535) return fail(CCH_ENOSUP, "generic GEMM path takes at most 65535 rows per call (got %d)", p.T);
         dim3 grid((unsigned)((p.n_out + 255) / 256), (unsigned)p.T);
-        if (p.mx_out_fmt == CCH_FMT_E4M3) hipLaunchKernelGGL((gemm_naive_swiglu_mx_kernel<CCH_FMT_E4M3>), grid, dim3(256), 0, stream, p);
-        else if (p.mx_out_fmt == CCH_FMT_E5M2) hipLaunchKernelGGL((gemm_naive_swiglu_mx_kernel<CCH_FMT_E5M2>), grid, dim3(256), 0, stream, p);
-        else hipLaunchKernelGGL((gemm_naive_swiglu_mx_kernel<CCH_FMT_E2M1>), grid, dim3(256), 0, stream, p);
+#define CCH_NAIVE_MX_OUT(K)                                                                                                                        \
+    do {                                                                                                                                           \
+        if (p.mx_out_fmt == CCH_FMT_E4M3) hipLaunchKernelGGL((gemm_naive_swiglu_mx_kernel<K, CCH_FMT_E4M3>), grid, dim3(256), 0, stream, p);      \
+        else if (p.mx_out_fmt == CCH_FMT_E5M2) hipLaunchKernelGGL((gemm_naive_swiglu_mx_kernel<K, CCH_FMT_E5M2>), grid, dim3(256), 0, stream, p); \
+        else hipLaunchKernelGGL((gemm_naive_swiglu_mx_kernel<K, CCH_FMT_E2M1>), grid, dim3(256), 0, stream, p);                                   \
+    } while (0)
+        if (kind == KIND_I8) CCH_NAIVE_MX_OUT(KIND_I8);
+        else if (kind == KIND_F8) CCH_NAIVE_MX_OUT(KIND_F8);
+        else CCH_NAIVE_MX_OUT(KIND_F4);
+#undef CCH_NAIVE_MX_OUT
         return launch_status("gemm_naive_swiglu_mx_kernel");
     }
     if (kind == KIND_I8 && epi == EPI_DEQUANT) return launch_naive_t<KIND_I8, EPI_DEQUANT>(p, stream);
     if (kind == KIND_I8 && epi == EPI_DEQUANT_SWIGLU) return launch_naive_t<KIND_I8, EPI_DEQUANT_SWIGLU>(p, stream);
     if (kind == KIND_F8 && epi == EPI_PLAIN) return launch_naive_t<KIND_F8, EPI_PLAIN>(p, stream);
     if (kind == KIND_F4 && epi == EPI_PLAIN) return launch_naive_t<KIND_F4, EPI_PLAIN>(p, stream);
+    if (kind == KIND_F8 && epi == EPI_SWIGLU) return launch_naive_t<KIND_F8, EPI_SWIGLU>(p, stream);
+    if (kind == KIND_F4 && epi == EPI_SWIGLU) return launch_naive_t<KIND_F4, EPI_SWIGLU>(p, stream);
     return fail(CCH_ENOSUP, "no generic GEMM kernel for kind %d with epilogue %d", kind, epi);
 }
 

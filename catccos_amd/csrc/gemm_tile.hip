@@ -245,7 +245,8 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     using KT = KindTraits<KIND>;
     using Acc = typename KT::Acc;
     constexpr bool MX = KIND != KIND_I8;
-    constexpr bool SWIGLU = EPI == EPI_DEQUANT_SWIGLU;
+    constexpr bool SWIGLU = EPI == EPI_DEQUANT_SWIGLU || EPI == EPI_SWIGLU;
+    constexpr bool DEQ = EPI == EPI_DEQUANT || EPI == EPI_DEQUANT_SWIGLU;   // per-token x per-channel scales in the epilogue
     constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;   // output columns per tile
     constexpr int WN_OUT = SWIGLU ? WN / 2 : WN;   // output columns per wave
     constexpr int SCALE_DW = KT::SCALE_DW;         // scale dwords per row per step
@@ -257,7 +258,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     constexpr int PASS_ROWS = 64 / CPR;            // rows staged per pass: 1 KiB, one read-back instruction
     constexpr int NPASS = 32 / PASS_ROWS;          // passes per 32-row MFMA tile
     constexpr int NSTORES = MT * NPASS;            // output stores per wave and tile (always issued; out-of-range lanes dropped)
-    constexpr int NPARAM = EPI != EPI_PLAIN ? 2 : 1;   // epilogue parameter requests per wave and tile
+    constexpr int NPARAM = DEQ ? 2 : 1;   // epilogue parameter requests per wave and tile
     // requests per wave in the four slots of a step
     constexpr int NL0 = 2;                          // A rows of row blocks 2-3 of the next step
     constexpr int NC0 = 2;                          // A rows of row blocks 0-1 of the step after the next
@@ -384,7 +385,8 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         } else {
             const int kr = (wave * NJ + q) * BRPI + lane / BCPR;
             const int tc = (lane % BCPR) ^ (FP4K ? (kr >> 1) & 7 : (kr & 7) << 1);
-            const int col = SWIGLU ? ((tc >> 1) & 1) * p.n_out + (tc >> 2) * 32 + (tc & 1) * 16 : tc * 16 * EPB;   // relative to j0
+            // relative to j0 (FP4: a chunk is 32 columns, one whole gate or up block)
+            const int col = !SWIGLU ? tc * 16 * EPB : FP4K ? (tc & 1) * p.n_out + (tc >> 1) * 32 : ((tc >> 1) & 1) * p.n_out + (tc >> 2) * 32 + (tc & 1) * 16;
             off_b[q] = (uint32_t)kr * (uint32_t)ldb + (uint32_t)(col / EPB);
         }
     }
@@ -443,12 +445,17 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 c.off_sc = ((uint32_t)(c.m0 + min(idx, c.m_end - 1 - c.m0)) * (uint32_t)p.sld) & ~3u;
             } else if (TB) {
                 c.rs_sc = make_rsrc(p.sb, (uint32_t)min((int64_t)p.num_groups * p.N * p.sld, (int64_t)lim));
-                c.off_sc = ((uint32_t)(c.e * p.N + min(c.j0 + idx, p.N - 1)) * (uint32_t)p.sld) & ~3u;
+                // (SwiGLU: tile column w*64 + h*32 + c is gate (h = 0) or up (h = 1) column j0 + w*32 + c)
+                const int col = SWIGLU ? ((idx >> 5) & 1) * p.n_out + min(c.j0 + (idx >> 6) * 32 + (idx & 31), p.n_out - 1) : min(c.j0 + idx, p.N - 1);
+                c.off_sc = ((uint32_t)(c.e * p.N + col) * (uint32_t)p.sld) & ~3u;
             } else {
                 // [K/64][N][2]: a scale group is 8 rows of K64 blocks (4 MXFP8 steps, 2 MXFP4 steps)
                 // x 256 columns x 2 bytes; wave 4+i fetches rows 2i, 2i+1, lane l 16 bytes of row l/32
                 c.rs_sc = make_rsrc(p.sb + (size_t)c.e * p.sb_stride, (uint32_t)min((int64_t)p.N * p.sld, (int64_t)lim));
-                c.off_sc = (uint32_t)((lane >> 5) + 2 * (wave - 4)) * (uint32_t)p.N * 2u + (uint32_t)c.j0 * 2u + (uint32_t)(lane & 31) * 16u;
+                // (SwiGLU: the lane's 8 tile columns lie inside one gate or up block of 32)
+                const int tcol = (lane & 31) * 8;
+                const int col = SWIGLU ? ((tcol >> 5) & 1) * p.n_out + c.j0 + (tcol >> 6) * 32 + (tcol & 31) : c.j0 + tcol;
+                c.off_sc = (uint32_t)((lane >> 5) + 2 * (wave - 4)) * (uint32_t)p.N * 2u + (uint32_t)col * 2u;
             }
             // Rows wm*128 + s*32 + r of A and columns j0 + wn*64 + s*32 + r of B: only r, m0, j0 and the
             // expert decide by how many bytes (0 or 2) a scale row starts past a 4-byte boundary (the
@@ -542,7 +549,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         const int idx = (wave & 3) * 64 + lane;
         // destination of lane 0 of this wave; lane l lands 4*l bytes further
         const uint32_t dst = lds_base + (uint32_t)(PARAM_OFF + parity * PARAM_SET) + (uint32_t)(wave & 3) * 256u;
-        if (EPI != EPI_PLAIN) {
+        if (DEQ) {
             load4_to_lds(make_rsrc(p.per_tok + c.m0, min((uint32_t)(p.T - c.m0) * 4u, lim)), (uint32_t)min(idx, c.m_end - 1 - c.m0) * 4u, 0u, dst);
             int col;
             if (SWIGLU) col = ((idx >> 5) & 1) * p.n_out + min(c.j0 + (idx >> 6) * 32 + (idx & 31), p.n_out - 1);
@@ -978,7 +985,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             const __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(
                 reinterpret_cast<uint8_t *>(p.out) + (has_map ? (size_t)0 : (size_t)cur.m0 * out_row_bytes), 0, 0x7FFFFFFF, 0x00020000);
             float chs[NT];
-            if (EPI != EPI_PLAIN) {
+            if (DEQ) {
 #pragma unroll
                 for (int j = 0; j < NT; j++) chs[j] = __uint_as_float(lds_read4(prm + 1024u + (uint32_t)(wn * WN + j * 32 + r) * 4u));
             }
@@ -990,7 +997,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                     for (int qq = 0; qq < PASS_ROWS / 8; qq++) {
                         const int q = ps * (PASS_ROWS / 8) + qq;
                         float tok[4];
-                        if (EPI != EPI_PLAIN) {
+                        if (DEQ) {
                             const v4i tv = lds_read16(prm + (uint32_t)(wm * WM + i * 32 + q * 8 + g * 4) * 4u);
 #pragma unroll
                             for (int xr = 0; xr < 4; xr++) tok[xr] = __int_as_float(tv[xr]);
@@ -1003,7 +1010,12 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                                 float v[2];
 #pragma unroll
                                 for (int d = 0; d < 2; d++) {
-                                    if (SWIGLU) {
+                                    if (EPI == EPI_SWIGLU) {
+                                        // the up projection's result is a bf16 tile before the activation sees it
+                                        const float gate = (float)(__bf16)(float)acc[i][0][x + d];
+                                        const float up = (float)(__bf16)(float)acc[i][1][x + d];
+                                        v[d] = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;
+                                    } else if (SWIGLU) {
                                         const float gate = (float)acc[i][0][x + d] * chs[0] * tok[xr + d];
                                         const float up = (float)acc[i][1][x + d] * chs[1] * tok[xr + d];
                                         // hardware exp2 and reciprocal: relative error ~1e-6, far inside the bf16 result
@@ -1120,7 +1132,7 @@ static int launch_tile_ua(const GemmProblem &p, hipStream_t stream)
         attr_set.fetch_or(dev_bit, std::memory_order_release);
     }
     CCH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    constexpr int bn_out = EPI == EPI_DEQUANT_SWIGLU ? BN / 2 : BN;
+    constexpr int bn_out = (EPI == EPI_DEQUANT_SWIGLU || EPI == EPI_SWIGLU) ? BN / 2 : BN;
     const int64_t row_tiles = (p.T + BM - 1) / BM + (p.group_sizes ? p.num_groups : 0);  // upper bound
     const int64_t tiles = row_tiles * ((p.n_out + bn_out - 1) / bn_out);
     const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>(tiles, cus));
@@ -1146,7 +1158,7 @@ const char *gemm_tile_unsupported(const GemmProblem &p, int kind, int epi)
     // rows are fetched in 16-byte pieces
     if (p.K < 1 || p.K % (16 * epb) != 0) return "K must be a multiple of 16 bytes per row";
     if (p.n_out % 8 != 0 || !aligned(p.out, 16)) return "output rows must take 16-byte stores (n_out % 8 == 0, out 16-byte aligned)";
-    if (p.mx_out && (epi != EPI_DEQUANT_SWIGLU || p.n_out % 32 != 0 || p.out_fp16)) return "MX-quantised output needs whole 32-column blocks";
+    if (p.mx_out && ((epi != EPI_DEQUANT_SWIGLU && epi != EPI_SWIGLU) || p.n_out % 32 != 0 || p.out_fp16)) return "MX-quantised output needs whole 32-column blocks";
     if ((int64_t)BM * p.n_out * 2 >= ((int64_t)1 << 31)) return "output row tile beyond 2 GiB";
     // mapped output rows are addressed from the start of `out` with 32-bit offsets
     if (p.out_row_map && (epi != EPI_PLAIN || p.out_rows * p.n_out * 2 >= ((int64_t)1 << 31) || !aligned(p.out_row_map, 4)))
@@ -1159,11 +1171,11 @@ const char *gemm_tile_unsupported(const GemmProblem &p, int kind, int epi)
     if (kind != KIND_I8 && ((int64_t)p.num_groups * p.N * p.sld >= ((int64_t)1 << 31) || (int64_t)p.T * p.sld >= ((int64_t)1 << 31)))
         return "scale arrays beyond 2 GiB";
     if (kind != KIND_I8 && p.sb_stride != (int64_t)p.N * p.sld) return "scale arrays of the right-hand operands must be back to back";
-    if (epi != EPI_PLAIN && (!aligned(p.per_tok, 4) || !aligned(p.per_ch, 4))) return "dequantisation scales must be 4-byte aligned";
+    if ((epi == EPI_DEQUANT || epi == EPI_DEQUANT_SWIGLU) && (!aligned(p.per_tok, 4) || !aligned(p.per_ch, 4))) return "dequantisation scales must be 4-byte aligned";
     if (!p.trans_b) {
         // [K, N] operands: rows of B are fetched in 16-byte pieces that start on 4-byte boundaries
         if ((p.N / epb) % 4 != 0) return "[K,N] operands need rows of a multiple of 4 bytes";
-        if (epi == EPI_DEQUANT_SWIGLU && p.n_out % 4 != 0) return "[K,N] SwiGLU operands need n/2 to be a multiple of 4";
+        if ((epi == EPI_DEQUANT_SWIGLU || epi == EPI_SWIGLU) && (p.n_out / epb) % 4 != 0) return "[K,N] SwiGLU operands need n/2 to be a multiple of 4";
     }
     return nullptr;
 }
@@ -1181,6 +1193,12 @@ int launch_gemm_tile(const GemmProblem &p, int kind, int epi, hipStream_t stream
         return tb ? launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E5M2, 1>(p, stream) : launch_tile_t<KIND_F8, EPI_PLAIN, CCH_FMT_E5M2, 0>(p, stream);
     if (kind == KIND_F4 && epi == EPI_PLAIN)
         return tb ? launch_tile_t<KIND_F4, EPI_PLAIN, CCH_FMT_E2M1, 1>(p, stream) : launch_tile_t<KIND_F4, EPI_PLAIN, CCH_FMT_E2M1, 0>(p, stream);
+    if (kind == KIND_F8 && epi == EPI_SWIGLU && p.fmt == CCH_FMT_E4M3)
+        return tb ? launch_tile_t<KIND_F8, EPI_SWIGLU, CCH_FMT_E4M3, 1>(p, stream) : launch_tile_t<KIND_F8, EPI_SWIGLU, CCH_FMT_E4M3, 0>(p, stream);
+    if (kind == KIND_F8 && epi == EPI_SWIGLU && p.fmt == CCH_FMT_E5M2)
+        return tb ? launch_tile_t<KIND_F8, EPI_SWIGLU, CCH_FMT_E5M2, 1>(p, stream) : launch_tile_t<KIND_F8, EPI_SWIGLU, CCH_FMT_E5M2, 0>(p, stream);
+    if (kind == KIND_F4 && epi == EPI_SWIGLU)
+        return tb ? launch_tile_t<KIND_F4, EPI_SWIGLU, CCH_FMT_E2M1, 1>(p, stream) : launch_tile_t<KIND_F4, EPI_SWIGLU, CCH_FMT_E2M1, 0>(p, stream);
     return fail(CCH_ENOSUP, "no tiled GEMM kernel for kind %d with epilogue %d, trans_b %d", kind, epi, p.trans_b);
 }
 

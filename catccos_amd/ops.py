@@ -357,6 +357,36 @@ def mx_grouped_matmul(a, sa, b, sb, group_sizes, fmt="e4m3", trans_b=0, out_dtyp
     return out
 
 
+def mx_grouped_matmul_swiglu(a, sa, b, sb, group_sizes, fmt="e4m3", trans_b=0, out_dtype=torch.bfloat16, out_fmt=None):
+    """MX grouped GEMM + SwiGLU, the up projection of the MX FFN chain: the [T, N] product is rounded to
+    bf16, columns [0, N/2) are the gate and [N/2, N) the up half, out = silu(gate) * up [T, N/2] in
+    bf16 (or half).  With out_fmt ("e4m3", "e5m2", "e2m1") the activation leaves MX-quantised from the
+    epilogue instead: returns (payload, scales), the bytes mx_quant makes of the bf16 result."""
+    _require_gpu(a, sa, b, sb, group_sizes)
+    if group_sizes.dtype != torch.int32 or group_sizes.dim() != 1:
+        raise ValueError("group_sizes must be a 1-D int32 tensor")
+    a, sa, b, sb, group_sizes = a.contiguous(), sa.contiguous(), b.contiguous(), sb.contiguous(), group_sizes.contiguous()
+    fmt, t, n, k, e = _mx_shapes(a, sa, b, sb, fmt, trans_b, True)
+    if group_sizes.numel() != e:
+        raise ValueError("group_sizes must have one entry per expert")
+    if n % 2:
+        raise ValueError("n must be even (gate | up halves)")
+    h = n // 2
+    if out_fmt is not None:
+        ofmt = _fmt(out_fmt)
+        if ofmt == FMT_E2M1 and h % 2:
+            raise ValueError("n must be a multiple of 4 for FP4 output")
+        payload = torch.empty((t, h // 2 if ofmt == FMT_E2M1 else h), dtype=torch.uint8, device=a.device)
+        scales = torch.empty((t, scale_cols(h)), dtype=torch.uint8, device=a.device)
+        check(_abi.lib().cch_mx_gmm_swiglu_mx(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(group_sizes), _ptr(payload), _ptr(scales), e, t, n, k,
+                                              fmt, int(trans_b), ofmt, _stream()))
+        return payload, scales
+    out = torch.empty((t, h), dtype=out_dtype, device=a.device)
+    check(_abi.lib().cch_mx_gmm_swiglu(_ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(group_sizes), _ptr(out), e, t, n, k, fmt, int(trans_b),
+                                       _out_code(out_dtype), _stream()))
+    return out
+
+
 def mx_grouped_matmul_mapped(a, sa, b, sb, group_sizes, out_row_map, out, fmt="e4m3", trans_b=0):
     """MX grouped GEMM whose result row i is written to out[out_row_map[i]] (entries that are negative
     or past the end of `out` are dropped; rows of `out` that the map does not name keep their contents).  `out` is a contiguous

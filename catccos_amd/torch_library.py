@@ -39,6 +39,7 @@ _lib.define("w8a8_matmul_dequant(Tensor a, Tensor b, Tensor per_tok, Tensor per_
 _lib.define("mx_matmul(Tensor a, Tensor sa, Tensor b, Tensor sb, str fmt, int trans_b) -> Tensor")
 _lib.define("gmm_dequant_swiglu(Tensor x, Tensor w, Tensor group_sizes, Tensor per_tok, Tensor per_ch, int trans_b) -> Tensor")
 _lib.define("mx_grouped_matmul(Tensor a, Tensor sa, Tensor b, Tensor sb, Tensor group_sizes, str fmt, int trans_b) -> Tensor")
+_lib.define("mx_grouped_matmul_swiglu_mx(Tensor a, Tensor sa, Tensor b, Tensor sb, Tensor group_sizes, str fmt, int trans_b, str out_fmt) -> (Tensor, Tensor)")
 _lib.define("gmm_dequant_swiglu_mx(Tensor x, Tensor w, Tensor group_sizes, Tensor per_tok, Tensor per_ch, int trans_b, str fmt) -> (Tensor, Tensor)")
 
 
@@ -86,6 +87,8 @@ _lib.impl("mx_matmul", _guarded(ops.mx_matmul), "CUDA")
 _lib.impl("gmm_dequant_swiglu", _guarded(ops.gmm_dequant_swiglu), "CUDA")
 _lib.impl("mx_grouped_matmul", _guarded(ops.mx_grouped_matmul), "CUDA")
 _lib.impl("gmm_dequant_swiglu_mx", _guarded(ops.gmm_dequant_swiglu_mx), "CUDA")
+_lib.impl("mx_grouped_matmul_swiglu_mx", _guarded(lambda a, sa, b, sb, gs, fmt, tb, ofmt: ops.mx_grouped_matmul_swiglu(a, sa, b, sb, gs, fmt, tb, out_fmt=ofmt)),
+          "CUDA")
 
 
 # ---- Meta kernels: output shapes only (symbolic sizes pass through the arithmetic untouched)
@@ -123,6 +126,12 @@ def _gmm_swiglu_mx_meta(x, w, group_sizes, per_tok, per_ch, trans_b, fmt):
     return payload, x.new_empty((x.shape[0], 2 * ((h + 63) // 64)), dtype=torch.uint8)
 
 
+def _mx_gmm_swiglu_mx_meta(a, sa, b, sb, group_sizes, fmt, trans_b, out_fmt):
+    h = _mx_n(b.shape[1:], fmt, trans_b) // 2
+    payload = a.new_empty((a.shape[0], h // 2 if _fp4(out_fmt) else h), dtype=torch.uint8)
+    return payload, a.new_empty((a.shape[0], 2 * ((h + 63) // 64)), dtype=torch.uint8)
+
+
 def _mx_gmm_meta(a, sa, b, sb, group_sizes, fmt, trans_b):
     return a.new_empty((a.shape[0], _mx_n(b.shape[1:], fmt, trans_b)), dtype=torch.bfloat16)
 
@@ -133,3 +142,4 @@ _lib.impl("mx_matmul", _mx_matmul_meta, "Meta")
 _lib.impl("gmm_dequant_swiglu", _gmm_swiglu_meta, "Meta")
 _lib.impl("mx_grouped_matmul", _mx_gmm_meta, "Meta")
 _lib.impl("gmm_dequant_swiglu_mx", _gmm_swiglu_mx_meta, "Meta")
+_lib.impl("mx_grouped_matmul_swiglu_mx", _mx_gmm_swiglu_mx_meta, "Meta")

@@ -184,6 +184,25 @@ int cch_mx_gemm_out(const void *a, const void *sa, const void *b, const void *sb
 int cch_mx_gmm(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes, void *out,
                int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, void *stream);
 
+/* ---- MX grouped matmul + SwiGLU: the up projection of the MX FFN chain ------
+ * Replaces GMM1 and the SwiGLU stage of the Ascend950 dispatch-FFN-combine kernel
+ * (examples/ascend950_dispatch_ffn_combine/ascend950_dispatch_ffn_combine_device.h:124-176: the up
+ * projection writes a bf16 tile, Ascend950SwigluFromUbKernel turns its gate and up planes into the
+ * activation, examples/aux_ops/ascend950_swiglu_from_ub.h:92-213; arithmetic of
+ * include/catccos/epilogue/block/block_epilogue_regbase_swiglu.hpp:38-80):
+ *   c = bf16(A_e x B_e) [t, n] per expert as cch_mx_gmm (columns [0, n/2) gate, [n/2, n) up);
+ *   out[r, j] = bf16( g / (1 + exp(-g)) * u ) with g = c[r, j], u = c[r, j + n/2], in fp32
+ * out [t, n/2] of out_dtype (CCH_OUT_BF16 / CCH_OUT_FP16); rows past sum(group_sizes) are zeros. */
+int cch_mx_gmm_swiglu(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes, void *out,
+                      int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, int out_dtype, void *stream);
+/* The same with the activation leaving MX-quantised along its rows (Ascend950SwigluMxQuantFromUbKernel,
+ * examples/aux_ops/ascend950_swiglu_from_ub.h:216-389): the bytes cch_mx_quant_rows (round to nearest
+ * even) makes of the bf16 output above, as the input of the down projection (cch_mx_gmm_mapped).
+ * payload / scales / out_fmt as cch_gmm_i8_dequant_swiglu_mx. */
+int cch_mx_gmm_swiglu_mx(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes, void *payload,
+                         void *scales, int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, int out_fmt,
+                         void *stream);
+
 /* ---- MXFP8 / MXFP4 grouped matmul with mapped output rows (down projection, config-5 twin) ----
  * Replaces the matmul half of GroupedMatmulAllToAllV for MX operands
  * (include/catccos/dgemm/kernel/grouped_matmul_alltoallv_mx.hpp:250 with the scheduler's RemapperC,

@@ -263,6 +263,16 @@ def gmm_i8_dequant_swiglu(x, w, group_sizes, per_tok, per_ch, fp16_step=False, r
     return (out, out16) if want_bf16 else out
 
 
+def swiglu_bf16(c_bf16):
+    """bf16 bits [T, N] (gate | up halves) -> bf16 bits [T, N/2] = silu(gate) * up, see oracle.c:orc_swiglu_bf16."""
+    c = np.ascontiguousarray(c_bf16, dtype=np.uint16)
+    t, n = c.shape
+    assert n % 2 == 0
+    out = np.empty((t, n // 2), dtype=np.uint16)
+    lib().orc_swiglu_bf16(_p(c), _i64(t), _i64(n), _p(out))
+    return out
+
+
 def mx_gmm(a, sa, b, sb, n, k, fmt=E4M3, trans_b=0, group_sizes=None, rows=None, want_bf16=False, want_f64=False, blocked=False):
     """Dense (group_sizes None, b one expert) or grouped MX GEMM golden; see oracle.c:orc_mx_gmm.
     `blocked` picks the cache-blocked routine (the CPU baseline; same values, no fp64 copy)."""

@@ -750,6 +750,29 @@ void orc_mx_gmm(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uin
     free(row_expert);
 }
 
+/*
+ * SwiGLU of a bf16 [T, N] tile, gate = columns [0, N/2), up = [N/2, N), as the reference's
+ * register-level routine computes it from the up projection's bf16 planes
+ * (include/catccos/epilogue/block/block_epilogue_regbase_swiglu.hpp:38-80): widen both to fp32,
+ *   d = exp(gate * -1) + 1;  r = gate / d;  r = r * up;  out = bf16(r), round to nearest even.
+ * pinned by: torch.nn.functional.silu(gate.float()) * up.float() rounded to bf16 (equal up to one
+ *            bf16 step where the two fp32 formulas round differently, equal exactly on most inputs),
+ *            the closed forms at gate = 0, large positive and large negative gate.
+ */
+void orc_swiglu_bf16(const uint16_t *c, int64_t T, int64_t N, uint16_t *out)
+{
+    const int64_t H = N / 2;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < T; r++)
+        for (int64_t j = 0; j < H; j++) {
+            float g = orc_bf16_to_f32(c[r * N + j]), u = orc_bf16_to_f32(c[r * N + j + H]);
+            float d = expf(g * -1.0f) + 1.0f;
+            float v = g / d;
+            v = v * u;
+            out[r * H + j] = orc_f32_to_bf16(v);
+        }
+}
+
 /* ------------------------------------------------ blocked CPU baselines */
 
 /*

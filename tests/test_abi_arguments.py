@@ -58,6 +58,13 @@ def test_gemm_arguments():
     rejected(L.cch_gmm_i8_dequant(P, P, P, P, P, P, 257, 8, 8, 8, 0, None), "num_experts", "256")
     rejected(L.cch_gmm_i8_dequant_swiglu(P, P, P, P, P, P, 257, 8, 8, 8, 0, None), "num_experts", "256")
     rejected(L.cch_mx_gmm(P, P, P, P, P, P, 257, 8, 8, 64, 0, 0, None), "num_experts", "256")
+    rejected(L.cch_mx_gmm_swiglu(P, P, P, P, P, P, 2, 8, 7, 64, 0, 0, 0, None), "even")
+    rejected(L.cch_mx_gmm_swiglu(P, P, P, P, P, P, 2, 8, 8, 64, 0, 0, 2, None), "out_dtype")
+    rejected(L.cch_mx_gmm_swiglu(P, P, P, P, None, P, 2, 8, 8, 64, 0, 0, 0, None), "group_sizes")
+    rejected(L.cch_mx_gmm_swiglu(P, P, P, P, P, P, 257, 8, 8, 64, 0, 0, 0, None), "num_experts", "256")
+    rejected(L.cch_mx_gmm_swiglu_mx(P, P, P, P, P, P, P, 2, 8, 8, 64, 0, 0, 3, None), "out_fmt")
+    rejected(L.cch_mx_gmm_swiglu_mx(P, P, P, P, P, P, P, 2, 8, 6, 64, 0, 0, 2, None), "FP4")
+    rejected(L.cch_mx_gmm_swiglu_mx(P, P, P, P, P, P, None, 2, 8, 8, 64, 0, 0, 0, None), "null")
     # SwiGLU with MX-quantised output: payload formats E4M3, E5M2, E2M1; n even (FP4: a multiple of 4)
     rejected(L.cch_gmm_i8_dequant_swiglu_mx(P, P, P, P, P, P, P, 2, 8, 8, 8, 0, 3, None), "fmt")
     rejected(L.cch_gmm_i8_dequant_swiglu_mx(P, P, P, P, P, P, P, 2, 8, 7, 8, 0, 0, None), "even")

@@ -92,3 +92,61 @@ def test_bad_arguments():
         cc.gmm_dequant_swiglu_mx(x, wd, gsd, pt, pc, 0, "e1m2x")
     with pytest.raises(cc.CatccosError):
         cc.gmm_dequant_swiglu_mx(x, wd, gsd, pt, pc, 0, "e1m2")
+
+
+# ---------------------------------------------------------------- MX up projection + SwiGLU
+
+def mx_case(e, t, k, n, gs, fmt, trans_b, seed):
+    rng = np.random.default_rng(seed)
+    sigma = 0.05 if fmt == "e2m1" else 0.5
+    pa, sa = orc.mx_quant_rows(orc.f32_to_bf16((rng.standard_normal((t, k)) * sigma).astype(np.float32)), FMT[fmt])
+    pbs, sbs = zip(*[orc.mx_quant_b(orc.f32_to_bf16((rng.standard_normal((k, n)) * sigma).astype(np.float32)), FMT[fmt], orc.RNE, trans_b)
+                     for _ in range(e)])
+    return pa, sa, np.stack(pbs), np.stack(sbs), np.array(gs, np.int32)
+
+
+def to_dev(x):
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
+@pytest.mark.parametrize("trans_b", [0, 1])
+@pytest.mark.parametrize("cfg", [(4, 700, 512, 1088, [300, 0, 143, 250]),     # n/2 = 544: ragged last column tile, odd block count
+                                 (3, 300, 1216, 512, [1, 0, 299]),            # K tail, scale rows off 4-byte boundaries
+                                 (5, 1500, 768, 2048, [700, 13, 0, 256, 531])])
+@pytest.mark.parametrize("tiled", [True, False], ids=["tiled", "generic"])
+def test_mx_gmm_swiglu_against_oracle_chain_and_fused_bytes(fmt, trans_b, cfg, tiled):
+    """bf16 result against the oracle chain (grouped MX GEMM -> bf16 -> SwiGLU of the bf16 tile), then the
+    fused MX-quantised activation byte for byte against the oracle's row quantiser of that bf16 result."""
+    e, t, k, n, gs = cfg
+    if not tiled:
+        t, gs = 120, [50, 0, 70][:e] + [0] * (e - 3)     # one thread per output: a few rows of the same N and K
+    pa, sa, pb, sb, gsh = mx_case(e, t, k, n, gs, fmt, trans_b, seed=t + k + n + trans_b)
+    cc.set_option("require_tiled_gemm" if tiled else "force_generic_gemm", 1)
+    try:
+        args = (to_dev(pa), to_dev(sa), to_dev(pb), to_dev(sb), to_dev(gsh), fmt, trans_b)
+        plain = cc.mx_grouped_matmul_swiglu(*args)
+        outs = {of: cc.mx_grouped_matmul_swiglu(*args, out_fmt=of) for of in ("e4m3", "e2m1")}
+        full = cc.mx_grouped_matmul(*args)
+    finally:
+        cc.set_option("require_tiled_gemm" if tiled else "force_generic_gemm", 0)
+    # (a) the activation, given the tile: the kernel rounds its accumulators to bf16 exactly as the plain grouped
+    # GEMM does (same accumulators), so the oracle's SwiGLU of that kernel's bf16 output must reproduce the result -
+    # to the bit, but for the hardware's exp and reciprocal: at most one bf16 step on at most one element in 10 000
+    want16 = orc.swiglu_bf16(bits(full))
+    got16 = bits(plain)
+    d16 = np.abs(got16.astype(np.int32) - want16.astype(np.int32))
+    assert d16.max() <= 1 and np.mean(d16 != 0) <= 1e-4, (int(d16.max()), float(np.mean(d16 != 0)))
+    # (b) end to end against the oracle chain (its own GEMM, bf16, SwiGLU): the two GEMMs agree to about 1e-6 of
+    # their terms, which flips the bf16 rounding of gate or up on one element in a hundred and swings sums that
+    # cancel to nearly zero; against the tensor's rms that stays inside the GEMM gate
+    _, c16 = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], trans_b, group_sizes=gsh, want_bf16=True)
+    want = orc.bf16_to_f32(orc.swiglu_bf16(c16))
+    got = plain.float().cpu().numpy()
+    m = orc.compare(got, want)
+    assert m["max_rel_floor_rms"] <= 3e-2 and m["frac_bad"] <= 1e-2 and abs(m["eb"]) <= 2.0 ** -7, m
+    assert np.all(got[int(gsh.sum()):] == 0)
+    for of, (pay, sc) in outs.items():
+        want_p, want_s = orc.mx_quant_rows(bits(plain), FMT[of])
+        assert np.array_equal(sc.cpu().numpy(), want_s), of
+        assert np.array_equal(pay.cpu().numpy(), want_p), of

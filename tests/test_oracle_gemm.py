@@ -165,3 +165,29 @@ def test_compare_metrics_vs_numpy():
     assert np.isclose(m["max_rel_floor_rms"], (diff / np.maximum(np.abs(g), rms)).max())
     assert np.isclose(m["eb"], ((d.astype(np.float64) - g) / f1).mean())
     assert np.isclose(m["rms_golden"], rms)
+
+
+def test_swiglu_bf16_against_torch_and_closed_forms():
+    """The SwiGLU of a bf16 tile (gate | up halves): torch's silu on the widened values, rounded to
+    bf16, is the independent check.  The oracle divides gate by 1 + exp(-gate) where torch multiplies by a
+    sigmoid: both are fp32 and may round one fp32 step apart, which moves the bf16 result by at most one
+    step and only on a small share of the inputs."""
+    import torch
+    rng = np.random.default_rng(8)
+    t, n = 300, 256
+    c = orc.f32_to_bf16((rng.standard_normal((t, n)) * 3.0).astype(np.float32))
+    got = orc.swiglu_bf16(c)
+    cf = torch.from_numpy(orc.bf16_to_f32(c))
+    want = (torch.nn.functional.silu(cf[:, : n // 2]) * cf[:, n // 2:]).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    assert diff.max() <= 1 and np.mean(diff == 0) > 0.99, (diff.max(), np.mean(diff == 0))
+    # closed forms: gate 0 -> 0; gate = 40 -> gate * up exactly (exp(-40) vanishes against 1); gate = -100 -> -0 * up
+    z = np.zeros((1, 4), np.float32)
+    z[0] = [0.0, 40.0, 3.0, -2.5]            # gates 0 and 40, ups 3 and -2.5
+    out = orc.bf16_to_f32(orc.swiglu_bf16(orc.f32_to_bf16(z)))
+    assert out[0, 0] == 0.0 and out[0, 1] == -100.0
+    z[0] = [-100.0, 1.0, 7.0, 2.0]
+    out = orc.bf16_to_f32(orc.swiglu_bf16(orc.f32_to_bf16(z)))
+    assert out[0, 0] == 0.0 and abs(out[0, 1] - 2.0 * 0.7310586) < 0.01
+    # a swapped gate and up would fail this one: silu(1) * 2 != silu(2) * 1
+    assert abs(out[0, 1] - 2.0 / (1.0 + np.exp(-1.0))) < 0.01 and abs(out[0, 1] - 2.0 / (1.0 + np.exp(-2.0))) > 0.1

@@ -17,7 +17,7 @@ def initialised():
 
 
 def test_schemas_are_registered():
-    for name in ("init", "finalize", "mx_quant", "w8a8_matmul_dequant", "mx_matmul", "gmm_dequant_swiglu", "mx_grouped_matmul", "gmm_dequant_swiglu_mx"):
+    for name in ("init", "finalize", "mx_quant", "w8a8_matmul_dequant", "mx_matmul", "gmm_dequant_swiglu", "mx_grouped_matmul", "gmm_dequant_swiglu_mx", "mx_grouped_matmul_swiglu_mx"):
         assert hasattr(OPS, name), name
     assert str(OPS.init.default._schema) == "catccos::init(int rank_id, int rank_size, int local_mem_size, str ip_port) -> int"
     assert str(OPS.finalize.default._schema) == "catccos::finalize() -> int"
@@ -63,6 +63,9 @@ def test_meta_shapes(initialised):
     out = OPS.mx_grouped_matmul(u8(m, k // 2), u8(m, 32), u8(e, k, n // 2), u8(e, 16, n, 2),
                                 torch.empty(e, dtype=torch.int32, device="meta"), "e2m1", 0)
     assert out.shape == (m, n) and out.dtype == torch.bfloat16
+    pq, sq = OPS.mx_grouped_matmul_swiglu_mx(u8(m, k), u8(m, 32), u8(e, k, n), u8(e, 16, n, 2), torch.empty(e, dtype=torch.int32, device="meta"),
+                                             "e4m3", 0, "e4m3")
+    assert pq.shape == (m, n // 2) and sq.shape == (m, 2 * ((n // 2 + 63) // 64))
 
 
 def test_cpu_tensors_have_no_kernel(initialised):
