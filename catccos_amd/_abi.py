@@ -48,6 +48,7 @@ PROTOTYPES = {
     "cch_gmm_i8_dequant_swiglu_out": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _I, _P],
     "cch_gmm_i8_dequant_swiglu_mx": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _I, _P],
     "cch_mx_gmm_swiglu": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _I, _I, _P],
+    "cch_mx_gmm_swiglu_mx_packed": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _I, _I, _P],
     "cch_mx_gmm_swiglu_mx": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _I, _I, _P],
     "cch_mx_gemm_out": [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I, _I, _I, _P],
     "cch_gmm_i8_dequant": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I, _P],

@@ -303,6 +303,34 @@ int cch_mx_gmm_swiglu_mx(const void *a, const void *sa, const void *b, const voi
     return run(p, kind, EPI_SWIGLU, static_cast<hipStream_t>(stream));
 }
 
+int cch_mx_gmm_swiglu_mx_packed(const void *packed_a, const void *b, const void *sb, const int32_t *group_sizes, void *payload,
+                                void *scales, int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, int out_fmt,
+                                void *stream)
+{
+    GemmProblem p{};
+    int kind = 0;
+    CCH_REQUIRE(out_fmt == CCH_FMT_E4M3 || out_fmt == CCH_FMT_E5M2 || out_fmt == CCH_FMT_E2M1,
+                "cch_mx_gmm_swiglu_mx_packed: out_fmt %d (E4M3, E5M2 or E2M1)", out_fmt);
+    CCH_REQUIRE(group_sizes != nullptr || t == 0, "cch_mx_gmm_swiglu_mx_packed: null group_sizes");
+    CCH_REQUIRE(n % 2 == 0, "cch_mx_gmm_swiglu_mx_packed: n=%lld must be even (gate | up halves)", (long long)n);
+    CCH_REQUIRE(out_fmt != CCH_FMT_E2M1 || n % 4 == 0, "cch_mx_gmm_swiglu_mx_packed: n=%lld: FP4 rows hold two codes per byte", (long long)n);
+    CCH_REQUIRE(t == 0 || n == 0 || scales != nullptr, "cch_mx_gmm_swiglu_mx_packed: null pointer");
+    // a packed row: payload bytes, then the padded E8M0 scales (what cch_mx_quant_scatter_packed writes)
+    const int64_t payload_bytes = fmt == CCH_FMT_E2M1 ? (k + 1) / 2 : k, row_bytes = payload_bytes + 2 * ((k + 63) / 64);
+    const uint8_t *rows = static_cast<const uint8_t *>(packed_a);
+    int rc = mx_problem("cch_mx_gmm_swiglu_mx_packed", p, rows, rows ? rows + payload_bytes : nullptr, b, sb, group_sizes, payload, num_experts, t, n,
+                        k, fmt, trans_b, &kind);
+    if (rc) return rc;
+    p.a_pitch = row_bytes;
+    p.sa_pitch = row_bytes;
+    p.n_out = (int)(n / 2);
+    p.out_scales = static_cast<uint8_t *>(scales);
+    p.mx_out = 1;
+    p.mx_out_fmt = out_fmt;
+    p.mx_out_sld = (int)(2 * ((p.n_out + 63) / 64));
+    return run(p, kind, EPI_SWIGLU, static_cast<hipStream_t>(stream));
+}
+
 int cch_mx_gmm_mapped(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes,
                       const int32_t *out_row_map, void *out, int64_t out_rows, int out_dtype, int64_t num_experts, int64_t t,
                       int64_t n, int64_t k, int fmt, int trans_b, void *stream)

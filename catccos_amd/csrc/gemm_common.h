@@ -21,6 +21,8 @@ struct GemmProblem {
     const uint8_t *a;        // [T, K] payload (FP4: K/2 bytes per row)
     const uint8_t *b;        // per expert: trans_b ? [N, K] : [K, N]   (FP4: last axis halved)
     const uint8_t *sa;       // MX: [T, sld] E8M0
+    int64_t a_pitch;         // bytes between rows of a (0: rows are back to back)
+    int64_t sa_pitch;        // bytes between rows of sa (0: sld); packed rows [payload | scales] have a_pitch == sa_pitch
     const uint8_t *sb;       // MX: per expert trans_b ? [N, sld] : [sld/2, N, 2]
     const float *per_tok;    // int8: [T]
     const float *per_ch;     // int8: [E, N]

@@ -45,7 +45,7 @@ __device__ __forceinline__ float dot_column(const GemmProblem &p, int row, int e
     const size_t ldb = p.trans_b ? lda : (fp4 ? (size_t)(p.N + 1) / 2 : (size_t)p.N);
     float acc = 0.0f;
     for (int k = 0; k < p.K; k++) {
-        uint32_t qa = p.a[(size_t)row * lda + (fp4 ? k >> 1 : k)];
+        uint32_t qa = p.a[(size_t)row * (p.a_pitch ? (size_t)p.a_pitch : lda) + (fp4 ? k >> 1 : k)];
         if (fp4) qa = (qa >> ((k & 1) * 4)) & 0xFu;
         uint32_t qb;
         if (p.trans_b) {
@@ -56,7 +56,7 @@ __device__ __forceinline__ float dot_column(const GemmProblem &p, int row, int e
             if (fp4) qb = (qb >> ((col & 1) * 4)) & 0xFu;
         }
         const int kb = k >> 5;
-        const uint32_t sa_b = p.sa[(size_t)row * p.sld + kb];
+        const uint32_t sa_b = p.sa[(size_t)row * (p.sa_pitch ? (size_t)p.sa_pitch : (size_t)p.sld) + kb];
         const uint32_t sb_b = p.trans_b ? sb[(size_t)col * p.sld + kb] : sb[((size_t)(kb >> 1) * p.N + col) * 2 + (kb & 1)];
         const float av = decode_small(qa, p.fmt) * e8m0_value(sa_b);
         const float bv = decode_small(qb, p.fmt) * e8m0_value(sb_b);

@@ -277,6 +277,8 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     const int r = lane & 31, g = lane >> 5;
 
     const int lda = p.K / KT::ELEMS_PER_BYTE;  // bytes per row of A and of B (K-contiguous)
+    const int pa = p.a_pitch ? (int)p.a_pitch : lda;     // bytes between rows of A (packed rows carry their scales behind the payload)
+    const int psa = p.sa_pitch ? (int)p.sa_pitch : p.sld;   // bytes between scale rows of A
     // an even number of steps per tile, so that a step's ring stage is its parity: an odd count runs one
     // more, empty step (its requests fetch nothing, its products are zero)
     const int ksteps = max(((lda + BKB - 1) / BKB + 1) & ~1, 2);
@@ -376,7 +378,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 #pragma unroll
     for (int q = 0; q < NJ; q++) {
         const int row = wm * WM + (q >> 1) * 64 + (wn * 2 + (q & 1)) * 8 + (lane >> 3);
-        off_a[q] = (uint32_t)row * (uint32_t)lda + ((uint32_t)(lane & 7) ^ swizzle_of_row(row)) * 16u;
+        off_a[q] = (uint32_t)row * (uint32_t)pa + ((uint32_t)(lane & 7) ^ swizzle_of_row(row)) * 16u;
         if (TB) {
             const int brow = (wave * NJ + q) * 8 + (lane >> 3);
             const uint32_t chunk = ((uint32_t)(lane & 7) ^ swizzle_of_row(brow)) * 16u;
@@ -431,7 +433,8 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // (TB = 1: row j0 of the expert's [N, K]; TB = 0: column j0 of its [K, N]) and ends with the
         // expert's operand: what a request finds past the tile's last valid column - other columns'
         // or the next expert's bytes, or nothing past the end - feeds columns that are never stored.
-        c.rs_a = make_rsrc(p.a + (size_t)c.m0 * lda, min((uint32_t)min(c.m_end - c.m0, BM) * (uint32_t)lda, lim));
+        // (with a pitch the last row ends lda bytes into its slot)
+        c.rs_a = make_rsrc(p.a + (size_t)c.m0 * pa, min((uint32_t)(min(c.m_end - c.m0, BM) - 1) * (uint32_t)pa + (uint32_t)lda, lim));
         const uint32_t b_first = TB ? (uint32_t)c.j0 * (uint32_t)lda : (uint32_t)(c.j0 / EPB);
         c.rs_b = make_rsrc(p.b + (size_t)c.e * p.b_stride + b_first, min(b_bytes - min(b_first, b_bytes), lim));
         if (MX) {
@@ -441,8 +444,8 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             // therefore start at the (aligned) beginning of the whole scale array.
             const int idx = (wave & 3) * 64 + lane;
             if (wave < 4) {
-                c.rs_sc = make_rsrc(p.sa, (uint32_t)min((int64_t)p.T * p.sld, (int64_t)lim));
-                c.off_sc = ((uint32_t)(c.m0 + min(idx, c.m_end - 1 - c.m0)) * (uint32_t)p.sld) & ~3u;
+                c.rs_sc = make_rsrc(p.sa, (uint32_t)min((int64_t)(p.T - 1) * psa + p.sld, (int64_t)lim));
+                c.off_sc = ((uint32_t)(c.m0 + min(idx, c.m_end - 1 - c.m0)) * (uint32_t)psa) & ~3u;
             } else if (TB) {
                 c.rs_sc = make_rsrc(p.sb, (uint32_t)min((int64_t)p.num_groups * p.N * p.sld, (int64_t)lim));
                 // (SwiGLU: tile column w*64 + h*32 + c is gate (h = 0) or up (h = 1) column j0 + w*32 + c)
@@ -462,7 +465,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             // other terms are multiples of 4 rows).  The reader holds the 8 bytes from the fetched
             // dword of a step on (lo, hi); lane group g wants the step's bytes g and 2 + g in bytes 0
             // and 2 of one register (the matrix instruction picks either with its byte selector).
-            const uint32_t ph_a = ((uint32_t)(c.m0 + r) * (uint32_t)p.sld) & 3u;
+            const uint32_t ph_a = ((uint32_t)(c.m0 + r) * (uint32_t)psa) & 3u;
             const uint32_t ph_b = ((uint32_t)(c.e * p.N + c.j0 + r) * (uint32_t)p.sld) & 3u;
             c.sel_a = 0x0c000c00u | (ph_a + g) | ((ph_a + g + 2) << 16);
             // TB = 0: lo / hi are the dwords of K64 rows 2x and 2x+1, two columns of two bytes each
@@ -1144,7 +1147,7 @@ template <int KIND, int EPI, int FMT, int TB>
 static int launch_tile_t(const GemmProblem &p, hipStream_t stream)
 {
     if constexpr (KIND != KIND_I8) {
-        if ((p.sld & 3) != 0) return launch_tile_ua<KIND, EPI, FMT, TB, 1>(p, stream);
+        if ((p.sld & 3) != 0 || (p.sa_pitch & 3) != 0) return launch_tile_ua<KIND, EPI, FMT, TB, 1>(p, stream);
     }
     return launch_tile_ua<KIND, EPI, FMT, TB, 0>(p, stream);
 }
@@ -1165,10 +1168,13 @@ const char *gemm_tile_unsupported(const GemmProblem &p, int kind, int epi)
         return "mapped output beyond 2 GiB or misaligned row map";
     if (p.num_groups > MAX_GROUPS) return "more than 256 groups";
     if ((int64_t)p.N * lda >= ((int64_t)1 << 31)) return "one right-hand operand beyond 2 GiB (32-bit source offsets)";
-    if ((int64_t)BM * lda >= ((int64_t)1 << 31)) return "a row tile of the left-hand operand beyond 2 GiB";
+    if ((int64_t)BM * std::max<int64_t>(lda, p.a_pitch) >= ((int64_t)1 << 31)) return "a row tile of the left-hand operand beyond 2 GiB";
+    // (the 16-byte requests need dword alignment only: packed rows of K = 256 are 264 bytes long)
+    if (p.a_pitch && (p.a_pitch % 4 != 0 || p.a_pitch < lda)) return "rows of the left-hand operand must start on 4-byte boundaries";
+    if (p.sa_pitch && (p.sa_pitch % 2 != 0 || p.sa_pitch < p.sld)) return "scale rows of the left-hand operand must start on even addresses";
     if (!aligned(p.a, 16) || !aligned(p.b, 16) || p.b_stride % 16 != 0) return "operands must be 16-byte aligned";
     if (kind != KIND_I8 && (!aligned(p.sa, 4) || !aligned(p.sb, 4) || p.sb_stride % 2 != 0)) return "scale arrays must be 4-byte aligned";
-    if (kind != KIND_I8 && ((int64_t)p.num_groups * p.N * p.sld >= ((int64_t)1 << 31) || (int64_t)p.T * p.sld >= ((int64_t)1 << 31)))
+    if (kind != KIND_I8 && ((int64_t)p.num_groups * p.N * p.sld >= ((int64_t)1 << 31) || (int64_t)p.T * std::max<int64_t>(p.sld, p.sa_pitch) >= ((int64_t)1 << 31)))
         return "scale arrays beyond 2 GiB";
     if (kind != KIND_I8 && p.sb_stride != (int64_t)p.N * p.sld) return "scale arrays of the right-hand operands must be back to back";
     if ((epi == EPI_DEQUANT || epi == EPI_DEQUANT_SWIGLU) && (!aligned(p.per_tok, 4) || !aligned(p.per_ch, 4))) return "dequantisation scales must be 4-byte aligned";

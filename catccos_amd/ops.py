@@ -387,6 +387,31 @@ def mx_grouped_matmul_swiglu(a, sa, b, sb, group_sizes, fmt="e4m3", trans_b=0, o
     return out
 
 
+def mx_grouped_matmul_swiglu_packed(packed_a, k, b, sb, group_sizes, fmt="e4m3", trans_b=0, out_fmt="e4m3"):
+    """mx_grouped_matmul_swiglu(..., out_fmt=...) whose left-hand operand is the packed buffer that
+    mx_quant_scatter_packed fills (uint8 [T, packed_row_bytes(k, fmt)]: payload then scales per row)."""
+    _require_gpu(packed_a, b, sb, group_sizes)
+    fmt, ofmt = _fmt(fmt), _fmt(out_fmt)
+    if packed_a.dim() != 2 or packed_a.dtype != torch.uint8 or packed_a.shape[1] != packed_row_bytes(k, fmt) or not packed_a.is_contiguous():
+        raise ValueError("packed_a must be a contiguous uint8 [T, %d] tensor" % packed_row_bytes(k, fmt))
+    if group_sizes.dtype != torch.int32 or group_sizes.dim() != 1:
+        raise ValueError("group_sizes must be a 1-D int32 tensor")
+    b, sb, group_sizes = b.contiguous(), sb.contiguous(), group_sizes.contiguous()
+    t, e = packed_a.shape[0], b.shape[0]
+    epb = 2 if fmt in _FP4 else 1
+    n = b.shape[1] if trans_b else b.shape[2] * epb
+    if b.dim() != 3 or (b.shape[2] * epb if trans_b else b.shape[1]) != k or group_sizes.numel() != e or sb.numel() != e * scale_cols(k) * n:
+        raise ValueError("shape mismatch between packed_a, b, sb and group_sizes")
+    if n % 2 or (ofmt == FMT_E2M1 and n % 4):
+        raise ValueError("n must be even (a multiple of 4 for FP4 output)")
+    h = n // 2
+    payload = torch.empty((t, h // 2 if ofmt == FMT_E2M1 else h), dtype=torch.uint8, device=packed_a.device)
+    scales = torch.empty((t, scale_cols(h)), dtype=torch.uint8, device=packed_a.device)
+    check(_abi.lib().cch_mx_gmm_swiglu_mx_packed(_ptr(packed_a), _ptr(b), _ptr(sb), _ptr(group_sizes), _ptr(payload), _ptr(scales), e, t, n, k,
+                                                 fmt, int(trans_b), ofmt, _stream()))
+    return payload, scales
+
+
 def mx_grouped_matmul_mapped(a, sa, b, sb, group_sizes, out_row_map, out, fmt="e4m3", trans_b=0):
     """MX grouped GEMM whose result row i is written to out[out_row_map[i]] (entries that are negative
     or past the end of `out` are dropped; rows of `out` that the map does not name keep their contents).  `out` is a contiguous

@@ -202,6 +202,15 @@ int cch_mx_gmm_swiglu(const void *a, const void *sa, const void *b, const void *
 int cch_mx_gmm_swiglu_mx(const void *a, const void *sa, const void *b, const void *sb, const int32_t *group_sizes, void *payload,
                          void *scales, int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, int out_fmt,
                          void *stream);
+/* The same reading its left-hand operand as the packed rows that cch_mx_quant_scatter_packed writes
+ * ([payload | scales] per row, t rows of k (FP8) or ceil(k/2) (FP4) + 2*ceil(k/64) bytes): the dispatch
+ * stage's buffer goes into the up projection as it is, as the reference's GMM1 reads its packed
+ * operand (PackedMxTileCopyTlaToUB, examples/ascend950_dispatch_ffn_combine/
+ * ascend950_dispatch_ffn_combine_device.h:118-122).  The tiled kernels take rows of a multiple of 4
+ * bytes (every K that is a multiple of 64). */
+int cch_mx_gmm_swiglu_mx_packed(const void *packed_a, const void *b, const void *sb, const int32_t *group_sizes, void *payload,
+                                void *scales, int64_t num_experts, int64_t t, int64_t n, int64_t k, int fmt, int trans_b, int out_fmt,
+                                void *stream);
 
 /* ---- MXFP8 / MXFP4 grouped matmul with mapped output rows (down projection, config-5 twin) ----
  * Replaces the matmul half of GroupedMatmulAllToAllV for MX operands
