@@ -144,7 +144,7 @@ def test_mx_gemm_reference_shape_list(shape):
     m, k, n = shape
     rng = np.random.default_rng(m + k + n)
     pa, sa, pb, sb = mx_operands(rng, m, n, k, "e4m3", 1)
-    want = orc.mx_gmm(pa, sa, pb, sb, n, k, orc.E4M3, 1)
+    want = orc.mx_gmm(pa, sa, pb, sb, n, k, orc.E4M3, 1, blocked=True)   # the cache-blocked routine: same bits, a fraction of the time
     got = out_f32(cc.mx_matmul(dev(pa), dev(sa), dev(pb), dev(sb), "e4m3", 1))
     assert_close(got, want, shape)
 
@@ -275,7 +275,7 @@ def test_mx_gemm_reference_shape_list_tiled(shape, trans_b, fmt, tiled_only):
     m, k, n = shape
     rng = np.random.default_rng(m + k + n + trans_b)
     pa, sa, pb, sb = mx_operands(rng, m, n, k, fmt, trans_b, 0.02 if fmt == "e2m1" else 1.0)
-    want = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], trans_b)
+    want = orc.mx_gmm(pa, sa, pb, sb, n, k, FMT[fmt], trans_b, blocked=True)
     got = out_f32(cc.mx_matmul(dev(pa), dev(sa), dev(pb), dev(sb), fmt, trans_b))
     assert_close(got, want, (shape, trans_b, fmt))
 
@@ -290,7 +290,7 @@ def test_i8_dequant_reference_mx_shapes_tiled(shape, trans_b, tiled_only):
     b = rng.integers(-127, 128, (k, n)).astype(np.int8)
     pt = rng.uniform(0.001, 0.02, m).astype(np.float32)
     pc = rng.uniform(0.001, 0.02, n).astype(np.float32)
-    want = orc.gemm_i8_dequant(a, b, pt, pc)
+    want = orc.gemm_i8_dequant(a, b, pt, pc, blocked=True)
     bb = np.ascontiguousarray(b.T) if trans_b else b
     got = out_f32(cc.w8a8_matmul_dequant(dev(a), dev(bb), dev(pt), dev(pc), trans_b))
     assert_close(got, want, ("i8 tiled", shape, trans_b))
