@@ -150,3 +150,37 @@ def test_mx_gmm_swiglu_against_oracle_chain_and_fused_bytes(fmt, trans_b, cfg, t
         want_p, want_s = orc.mx_quant_rows(bits(plain), FMT[of])
         assert np.array_equal(sc.cpu().numpy(), want_s), of
         assert np.array_equal(pay.cpu().numpy(), want_p), of
+
+
+@pytest.mark.parametrize("tiled", [True, False], ids=["tiled", "generic"])
+def test_edge_cases_of_the_fused_outputs(tiled):
+    """All groups empty (every row is a row of no group: zero codes, scale bytes 127), group sizes that run past
+    the rows (clipped, as the GEMMs do), one row, and no rows at all."""
+    e, k, n = 3, 256, 512
+    rng = np.random.default_rng(99)
+    cc.set_option("require_tiled_gemm" if tiled else "force_generic_gemm", 1)
+    try:
+        for t, gs in ((5, [0, 0, 0]), (70, [40, 0, 100]), (1, [0, 1, 0]), (0, [0, 0, 0])):
+            pa, sa, pb, sb, gsh = mx_case(e, max(t, 1), k, n, gs, "e4m3", 0, seed=t)
+            pa, sa = pa[:t], sa[:t]
+            args = (to_dev(pa), to_dev(sa), to_dev(pb), to_dev(sb), to_dev(gsh), "e4m3", 0)
+            plain = cc.mx_grouped_matmul_swiglu(*args)
+            pay, sc = cc.mx_grouped_matmul_swiglu(*args, out_fmt="e4m3")
+            torch.cuda.synchronize()
+            assert plain.shape == (t, n // 2) and pay.shape == (t, n // 2) and sc.shape == (t, 8)
+            if t == 0:
+                continue
+            want_p, want_s = orc.mx_quant_rows(bits(plain), orc.E4M3)
+            assert np.array_equal(pay.cpu().numpy(), want_p) and np.array_equal(sc.cpu().numpy(), want_s), (t, gs)
+            used = min(t, int(np.sum(gs)))
+            assert np.all(bits(plain)[used:] == 0) and np.all(pay.cpu().numpy()[used:] == 0) and np.all(sc.cpu().numpy()[used:] == 127)
+            # int8 twin on the same grouping
+            x = torch.from_numpy(rng.integers(-127, 128, (t, k)).astype(np.int8)).cuda()
+            w = torch.from_numpy(rng.integers(-127, 128, (e, k, n)).astype(np.int8)).cuda()
+            pt = torch.from_numpy(rng.uniform(0.001, 0.02, t).astype(np.float32)).cuda()
+            pc = torch.from_numpy(rng.uniform(0.001, 0.02, (e, n)).astype(np.float32)).cuda()
+            p8, s8 = cc.gmm_dequant_swiglu_mx(x, w, to_dev(gsh), pt, pc, 0, "e2m1")
+            w_p, w_s = orc.mx_quant_rows(bits(cc.gmm_dequant_swiglu(x, w, to_dev(gsh), pt, pc, 0)), orc.E2M1)
+            assert np.array_equal(p8.cpu().numpy(), w_p) and np.array_equal(s8.cpu().numpy(), w_s), (t, gs)
+    finally:
+        cc.set_option("require_tiled_gemm" if tiled else "force_generic_gemm", 0)
