@@ -11,7 +11,7 @@
 //                                 M,K,N reads and writes <data_dir>/<M>_<K>_<N>/
 //   catccos_run --list            registry names and dispatch keys, no device needed
 // <kernel> is a short name of CommTypeMap (mxqtag, agmmdq, a5mxfp8mmrs, dgds, a5fp4mxatavgmm,
-// a5fp8mxatavgmm); "-" as data_dir runs on constant inputs and writes nothing (perf mode).
+// a5fp8mxatavgmm, a5fp8gmmata, a5fp4gmmata, a5moe); "-" as data_dir runs on constant inputs and writes nothing (perf mode).
 #include <chrono>
 #include <cstdlib>
 #include <fstream>

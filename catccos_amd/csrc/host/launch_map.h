@@ -63,5 +63,7 @@ void LaunchAscend950Fp8MxGroupedMatmulAllToAllVFP16(void *, uint32_t, uint64_t, 
                                                     CocTilingParams &, uint32_t, uint32_t);
 void LaunchAscend950Fp4MxGroupedMatmulAllToAllVFP16(void *, uint32_t, uint64_t, KernelParams &, uint8_t *, uint8_t *,
                                                     CocTilingParams &, uint32_t, uint32_t);
+void LaunchAscend950DispatchFFNCombineBF16(void *, uint32_t, uint64_t, KernelParams &, uint8_t *, uint8_t *, CocTilingParams &,
+                                           uint32_t, uint32_t);
 
 #endif  // CATCCOS_HOST_LAUNCH_MAP_H

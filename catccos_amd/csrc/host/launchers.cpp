@@ -209,6 +209,37 @@ void LaunchAscend950Fp4MxGroupedMatmulAllToAllVFP16(void *stream, uint32_t, uint
     MxGroupedMatmulAllToAllV(stream, p, t, transB, CCH_FMT_E2M1, CCH_OUT_FP16, "Ascend950Fp4MxGroupedMatmulAllToAllV");
 }
 
+// The MXFP8 FFN of one rank, the stages of the reference's single kernel
+// (examples/ascend950_dispatch_ffn_combine/ascend950_dispatch_ffn_combine_device.h:124-176: routing sort, MX quantisation
+// into the dispatch rows, GMM1, SwiGLU + MX quantisation, GMM2, weighted un-permute) as five launches on one
+// stream with no host round trip: the packed rows feed GMM1 in place, GMM1 hands over MXFP8 payload and scales.
+// Pointer roles: see Ascend950DispatchFFNCombineOperator.  The weight files hold W transposed ([E,n,k]) whatever
+// the transB argument says (the reference passes weightNz = 1, transB = 0 for them, scripts/run.sh:92).
+void LaunchAscend950DispatchFFNCombineBF16(void *stream, uint32_t, uint64_t, KernelParams &p, uint8_t *, uint8_t *, CocTilingParams &t,
+                                           uint32_t, uint32_t)
+{
+    const int64_t topK = t.topK ? t.topK : 1, rows = (int64_t)t.m * topK, e = t.expertNum, k = t.k, n = t.n;
+    if (p.customCount < 13) {
+        Finish(CCH_EINVAL, stream, "Ascend950DispatchFFNCombine (buffers not allocated by its operator)");
+        return;
+    }
+    auto i32 = [&](int i) { return reinterpret_cast<int32_t *>(p.customPtrs[i]); };
+    int rc = cch_moe_init_routing(i32(1), rows, (int)e, i32(6), i32(5), i32(7), 0, p.customPtrs[12],
+                                  cch_moe_init_routing_workspace_bytes(rows, (int)e), stream);
+    if (rc == CCH_OK)
+        rc = cch_mx_quant_scatter_packed_rows(p.ptrA, i32(5), p.customPtrs[8], rows, t.m, k, (int)topK, CCH_FMT_E4M3, CCH_ROUND_RNE, stream);
+    if (rc == CCH_OK)
+        rc = cch_mx_gmm_swiglu_mx_packed(p.customPtrs[8], p.ptrB, p.customPtrs[3], i32(7), p.customPtrs[9], p.customPtrs[10], e, rows, n, k,
+                                         CCH_FMT_E4M3, 1, CCH_FMT_E4M3, stream);
+    if (rc == CCH_OK)
+        rc = cch_mx_gmm(p.customPtrs[9], p.customPtrs[10], p.customPtrs[0], p.customPtrs[4], i32(7), p.customPtrs[11], e, rows, k, n / 2,
+                        CCH_FMT_E4M3, 1, stream);
+    if (rc == CCH_OK)
+        rc = cch_moe_token_unpermute(p.customPtrs[11], i32(5), reinterpret_cast<const float *>(p.customPtrs[2]), p.ptrC, rows, t.m, k,
+                                     (int)topK, stream);
+    Finish(rc, stream, "Ascend950DispatchFFNCombine");
+}
+
 static AutoRegister s_reg0(MX_QUANT_ALLGATHER, FP8E4M3FN, &LaunchAscend950BF16QuantAllGatherFP8E4M3FN);
 static AutoRegister s_reg1(ALLGATHER_MATMUL_DEQUANT, INT8, &LaunchAllGatherMatmulDequantINT8);
 static AutoRegister s_reg2(ASCEND950_MXFP8_MATMUL_REDUCE_SCATTER, FP8E4M3FN, &LaunchAscend950MxFp8MatmulReduceScatterFP8E4M3FN);
@@ -221,3 +252,4 @@ static AutoRegister s_reg8(ASCEND950_FP8_MX_GROUPED_MATMUL_ALLTOALLV, FP16, &Lau
 static AutoRegister s_reg9(ASCEND950_FP4_MX_GROUPED_MATMUL_ALLTOALLV, FP16, &LaunchAscend950Fp4MxGroupedMatmulAllToAllVFP16);
 static AutoRegister s_reg10(ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL, FP16, &LaunchAscend950Fp4MxAllToAllVGroupedMatmulFP16);
 static AutoRegister s_reg11(ASCEND950_FP8_MX_ALLTOALLV_GROUPED_MATMUL, FP16, &LaunchAscend950Fp8MxAllToAllVGroupedMatmulFP16);
+static AutoRegister s_reg12(ASCEND950_DISPATCH_FFN_COMBINE, BF16, &LaunchAscend950DispatchFFNCombineBF16);

@@ -359,6 +359,76 @@ public:
 using Ascend950Fp8MxGroupedMatmulAllToAllVOperator = MxGroupedMatmulAllToAllVOperator<false, ASCEND950_FP8_MX_GROUPED_MATMUL_ALLTOALLV>;
 using Ascend950Fp4MxGroupedMatmulAllToAllVOperator = MxGroupedMatmulAllToAllVOperator<true, ASCEND950_FP4_MX_GROUPED_MATMUL_ALLTOALLV>;
 
+// ---------------------------------------------------------------------------------------------
+// The MXFP8 MoE FFN of one rank from routing to combine (reference examples/ascend950_dispatch_ffn_combine/
+// ascend950_dispatch_ffn_combine_host.h:15-194; files as examples/utils/gen_data_moe.py:460-616 writes them):
+//   in_routing_matrix_a_<r>.bin      bf16 [m,k] tokens            in_routing_expert_idx_<r>.bin  int32 [m,topK]
+//   in_gmm_matrix_b_<r>.bin          E4M3 [E,n,k] (W1 transposed) in_gmm_matrix_b_scale_<r>.bin  E8M0 [E,n,2*ceil(k/64)]
+//   in_gmm_matrix_b2_<r>.bin         E4M3 [E,k,n/2]               in_gmm_matrix_b2_scale_<r>.bin E8M0 [E,k,2*ceil(n/128)]
+//   in_gather_gate_weight_<r>.bin    fp32 [m,topK]                output_<r>.bin                 bf16 [m,k]
+// Pointer roles as the reference's main.cpp:203-210 reads them back: ptrA = tokens, ptrB = W1, ptrC = out,
+// custom[0] = W2, [1] = expert_idx, [2] = gate weights, [3] = W1 scales, [4] = W2 scales.  The buffers the
+// reference carves out of its workspace (:165-176) follow: [5] expanded_row_idx (row of each routed token after
+// the sort), [6] its inverse, [7] tokens per expert, [8] packed MXFP8 rows after dispatch, [9]/[10] the
+// quantised activation and its scales, [11] GMM2's output rows, [12] the routing sort's workspace.
+// One rank holds every expert here: the two all-to-all exchanges are the identity.
+class Ascend950DispatchFFNCombineOperator : public CatccosOperator {
+public:
+    void AllocateDeviceSpace(KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        const size_t m = t.m, k = t.k, n = t.n, h = n / 2, e = t.expertNum, topK = t.topK ? t.topK : 1, rows = m * topK;
+        const std::string r = R(rankId);
+        uint8_t *a = DeviceAlloc(m * k * 2), *idx = DeviceAlloc(rows * 4), *probs = DeviceAlloc(rows * 4);
+        {
+            // constant inputs of the perf mode: tokens 1.0, routes round-robin over the experts, equal gate weights
+            std::vector<uint16_t> ones(m * k, 0x3F80);
+            std::vector<int32_t> routes(rows);
+            std::vector<float> gate(rows, 1.0f / static_cast<float>(topK));
+            for (size_t i = 0; i < rows; i++) routes[i] = static_cast<int32_t>(i % e);
+            if (!dataFile.empty()) {
+                ReadFile(dataFile + "/in_routing_matrix_a_" + r + ".bin", ones.data(), m * k * 2);
+                ReadFile(dataFile + "/in_routing_expert_idx_" + r + ".bin", routes.data(), rows * 4);
+                ReadFile(dataFile + "/in_gather_gate_weight_" + r + ".bin", gate.data(), rows * 4);
+            }
+            CCH_CHECK(cch_memcpy_h2d(a, ones.data(), m * k * 2));
+            CCH_CHECK(cch_memcpy_h2d(idx, routes.data(), rows * 4));
+            CCH_CHECK(cch_memcpy_h2d(probs, gate.data(), rows * 4));
+        }
+        uint8_t *b = LoadOrFill(e * n * k, dataFile, "in_gmm_matrix_b_" + r + ".bin", 0x38);
+        uint8_t *b2 = LoadOrFill(e * k * h, dataFile, "in_gmm_matrix_b2_" + r + ".bin", 0x38);
+        uint8_t *sb = LoadOrFill(e * n * ScaleCols(k), dataFile, "in_gmm_matrix_b_scale_" + r + ".bin", 127);
+        uint8_t *sb2 = LoadOrFill(e * k * ScaleCols(h), dataFile, "in_gmm_matrix_b2_scale_" + r + ".bin", 127);
+        uint8_t *c = DeviceAlloc(m * k * 2);
+        CCH_CHECK(cch_memset(c, 0, m * k * 2));
+        const size_t wsBytes = static_cast<size_t>(cch_moe_init_routing_workspace_bytes(static_cast<int64_t>(rows), static_cast<int>(e)));
+        uint8_t *s2d = DeviceAlloc(rows * 4), *d2s = DeviceAlloc(rows * 4), *cnt = DeviceAlloc(e * 4);
+        uint8_t *packed = DeviceAlloc(rows * (k + ScaleCols(k))), *act = DeviceAlloc(rows * h), *actScale = DeviceAlloc(rows * ScaleCols(h));
+        uint8_t *y = DeviceAlloc(rows * k * 2), *ws = DeviceAlloc(wsBytes);
+        params.SetKernelParams(a, b, c, b2, idx, probs, sb, sb2, s2d, d2s, cnt, packed, act, actScale, y, ws);
+    }
+    void WriteResultFile(const KernelParams &params, const CocTilingParams &t, uint32_t rankId, std::string dataFile) override
+    {
+        DumpDevice(params.ptrC, static_cast<size_t>(t.m) * t.k * 2, dataFile + "/output_" + R(rankId) + ".bin");
+    }
+    size_t GetWorkspaceSize(const CocTilingParams &) override { return 0; }
+    CocCommType GetActualKernelType(const CocTilingParams &) override { return ASCEND950_DISPATCH_FFN_COMBINE; }
+    bool CheckCocTilingParams(uint32_t rankSize, const CocTilingParams &t) override
+    {
+        if (rankSize > 1) {
+            ERROR_LOG("Ascend950DispatchFFNCombine: this build runs one rank that holds every expert");
+            return false;
+        }
+        // the reference's own shape rule (ascend950_dispatch_ffn_combine_host.h:180-184)
+        if (t.k % 256 != 0 || t.n % 512 != 0) {
+            ERROR_LOG("MXFP8 FFN requires K %% 256 == 0 and N %% 512 == 0");
+            return false;
+        }
+        const uint32_t topK = t.topK ? t.topK : 1;
+        return t.m > 0 && t.k > 0 && t.n > 0 && t.expertNum > 0 && topK <= t.expertNum &&
+               static_cast<uint64_t>(t.m) * topK < (1ull << 31);
+    }
+};
+
 }  // namespace
 
 REGISTER_OPERATOR("MxQuantAllGather", MxQuantAllGatherOperator)
@@ -369,3 +439,4 @@ REGISTER_OPERATOR("Ascend950Fp4MxAllToAllVGroupedMatmul", Ascend950Fp4MxAllToAll
 REGISTER_OPERATOR("Ascend950Fp8MxAllToAllVGroupedMatmul", Ascend950Fp8MxAllToAllVGroupedMatmulOperator)
 REGISTER_OPERATOR("Ascend950Fp8MxGroupedMatmulAllToAllV", Ascend950Fp8MxGroupedMatmulAllToAllVOperator)
 REGISTER_OPERATOR("Ascend950Fp4MxGroupedMatmulAllToAllV", Ascend950Fp4MxGroupedMatmulAllToAllVOperator)
+REGISTER_OPERATOR("Ascend950DispatchFFNCombine", Ascend950DispatchFFNCombineOperator)

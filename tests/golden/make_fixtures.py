@@ -21,7 +21,7 @@ import sys
 OPS = [
     "ascend950_mx_quant_allgather", "allgather_matmul_dequant", "ascend950_mxfp8_matmul_reduce_scatter",
     "dispatch_gmm_dequant_swiglu", "ascend950_fp4_mx_alltoallv_grouped_matmul", "ascend950_fp8_mx_alltoallv_grouped_matmul",
-    "ascend950_fp8_mx_grouped_matmul_alltoallv", "ascend950_fp4_mx_grouped_matmul_alltoallv",
+    "ascend950_fp8_mx_grouped_matmul_alltoallv", "ascend950_fp4_mx_grouped_matmul_alltoallv", "ascend950_dispatch_ffn_combine",
 ]
 
 

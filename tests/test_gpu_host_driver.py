@@ -1,6 +1,7 @@
 """End-to-end through the C++ operator surface, the way the reference's run.sh scripts test an
 operator: write input .bin files, run the driver binary, compare the output files with the golden
 (here: the CPU oracle)."""
+import json
 import os
 import subprocess
 
@@ -192,3 +193,59 @@ def test_shape_list_walk(tmp_path):
     assert r.returncode == 0 and r.stdout.count("[PERF] Avg latency") == 2, r.stdout + r.stderr
     r = subprocess.run([DRIVER, "a5mxfp8mmrs", "--shapes", str(tmp_path / "missing.csv"), "-"], capture_output=True, text=True, timeout=60)
     assert r.returncode != 0
+
+
+@pytest.mark.parametrize("m,k,n,e,topk", [(4, 512, 1024, 16, 6), (300, 256, 512, 8, 2), (256, 7168, 1024, 16, 6)],
+                         ids=["m4-top6", "m300-top2", "reference-shape-256x7168x1024"])
+def test_dispatch_ffn_combine_files(tmp_path, m, k, n, e, topk):
+    """The reference's file set of the MXFP8 FFN example (ascend950_dispatch_ffn_combine_host.h:15-150, written the way
+    examples/utils/gen_data_moe.py:460-616 writes it: weights transposed, gate weights a softmax, routes distinct per
+    token) through the driver; the golden is that generator's chain restated with the oracle's routines.  The third case
+    is a line of the example's own shape list (scripts/test_shapes.csv) with its run.sh's 16 experts and top-6."""
+    rng = np.random.default_rng(m + e)
+    x = rand_bf16(rng, (m, k))
+    expert_idx = np.argsort(rng.random((m, e)), axis=1)[:, :topk].astype(np.int32)
+    logits = rng.standard_normal((m, topk)).astype(np.float32)
+    probs = (np.exp(logits) / np.exp(logits).sum(1, keepdims=True)).astype(np.float32)
+    h = n // 2
+    w1 = [orc.f32_to_bf16((rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)) for _ in range(e)]
+    w2 = [orc.f32_to_bf16((rng.standard_normal((h, k)) / np.sqrt(h)).astype(np.float32)) for _ in range(e)]
+    b1, sb1 = map(np.stack, zip(*[orc.mx_quant_b(w, orc.E4M3, orc.RNE, 1) for w in w1]))      # [E, n, k], scales [E, n, k/32]
+    b2, sb2 = map(np.stack, zip(*[orc.mx_quant_b(w, orc.E4M3, orc.RNE, 1) for w in w2]))      # [E, k, h], scales [E, k, h/32]
+    for name, arr in (("in_routing_matrix_a", x), ("in_routing_expert_idx", expert_idx), ("in_gather_gate_weight", probs),
+                      ("in_gmm_matrix_b", b1), ("in_gmm_matrix_b_scale", sb1), ("in_gmm_matrix_b2", b2), ("in_gmm_matrix_b2_scale", sb2)):
+        arr.tofile(tmp_path / f"{name}_0.bin")
+    drive(tmp_path, "a5moe", m, k, n, tmp_path, "--experts", e, "--topk", topk, "--iters", 1, "--warmup", 1)
+    rows = m * topk
+    _, s2d, cnt = orc.moe_init_routing(expert_idx, e)
+    packed = orc.mx_quant_scatter_packed(x, s2d, rows, topk, orc.E4M3)
+    _, c1 = orc.mx_gmm(packed[:, :k], packed[:, k:], b1, sb1, n, k, orc.E4M3, 1, group_sizes=cnt, want_bf16=True, blocked=True)
+    a2, sa2 = orc.mx_quant_rows(orc.swiglu_bf16(c1), orc.E4M3)
+    _, y = orc.mx_gmm(a2, sa2, b2, sb2, k, h, orc.E4M3, 1, group_sizes=cnt, want_bf16=True, blocked=True)
+    want = orc.bf16_to_f32(orc.moe_token_unpermute(y, s2d, probs, topk))
+    got = bf16_file(tmp_path / "output_0.bin", (m, k))
+    # two implementations of this chain agree to about 1 % of the tensor's rms: a bf16 step in GMM1's result moves a code
+    # of the quantised activation (tests/test_gpu_ffn_chain.py checks the stages one by one, to the bit where they are bytes)
+    rms = np.sqrt(np.mean(want ** 2))
+    assert np.sqrt(np.mean((got - want) ** 2)) <= 2e-2 * rms and np.abs(got - want).max() <= 0.12 * rms
+    # perf mode: constant inputs, nothing written
+    drive(tmp_path, "a5moe", m, k, n, "-", "--experts", e, "--topk", topk, "--iters", 2, "--warmup", 1)
+    # the reference's own shape rule and message (ascend950_dispatch_ffn_combine_host.h:180-184); one rank only
+    r = subprocess.run([DRIVER, "a5moe", "64", "7168", "1000", "-", "--experts", "8", "--topk", "2"], capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "MXFP8 FFN requires K % 256 == 0 and N % 512 == 0" in r.stdout
+    r = subprocess.run([DRIVER, "a5moe", "64", "256", "512", "-", "--experts", "8", "--topk", "2", "--ranks", "2"], capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "one rank" in r.stdout
+
+
+def test_dispatch_ffn_combine_reference_shape_list_perf_mode(tmp_path):
+    """Every line of the example's own shape list (tests/golden/reference_shapes.json, from its scripts/test_shapes.csv) with
+    its run.sh's 16 experts and top-6, on constant inputs: the driver's shape walk, all five launches on the tiled kernels."""
+    shapes = json.load(open(os.path.join(ROOT, "tests", "golden", "reference_shapes.json")))["ascend950_dispatch_ffn_combine"]
+    assert [256, 7168, 1024] in shapes and len(shapes) == 4
+    csv = tmp_path / "test_shapes.csv"
+    csv.write_text("M,K,N\n" + "".join("%d,%d,%d\n" % tuple(s) for s in shapes))
+    r = subprocess.run([DRIVER, "a5moe", "--shapes", str(csv), "-", "--experts", "16", "--topk", "6", "--iters", "3", "--warmup", "2"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.count("[PERF] Avg latency") == 4 and "4 shapes finished" in r.stdout, r.stdout + r.stderr
+    assert "[ERROR]" not in r.stdout and "generic" not in r.stderr, r.stdout + r.stderr
+    print(r.stdout)

@@ -19,6 +19,8 @@ EXPECT = {
     # this build has those launchers (keys (25 << 8) | 1, (26 << 8) | 1) and bf16 twins, which --list shows
     "a5fp8gmmata": ("Ascend950Fp8MxGroupedMatmulAllToAllV", 25, 27),
     "a5fp4gmmata": ("Ascend950Fp4MxGroupedMatmulAllToAllV", 26, 27),
+    # the MXFP8 FFN from routing to combine on one rank (bf16 in and out, as the reference's run.sh runs it)
+    "a5moe": ("Ascend950DispatchFFNCombine", 32, 27),
 }
 
 
@@ -47,7 +49,7 @@ def test_registry_and_dispatch_keys_match_reference():
     # (dtype FP16 = 1, launch_map.h:98-101)
     for short, ctype in (("a5fp8gmmata", 25), ("a5fp4gmmata", 26), ("a5fp8mxatavgmm", 27), ("a5fp4mxatavgmm", 28)):
         assert any(e[1:] == (ctype, 1, (ctype << 8) | 1) for e in seen[short])
-    assert sum(len(v) for v in seen.values()) == 12
+    assert sum(len(v) for v in seen.values()) == 13
 
 
 def test_unknown_kernel_and_bad_shape_fail_like_the_reference_main():
