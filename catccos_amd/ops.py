@@ -432,3 +432,29 @@ def mx_grouped_matmul_mapped(a, sa, b, sb, group_sizes, out_row_map, out, fmt="e
                                        _ptr(out), out.shape[0], 1 if out.dtype == torch.float16 else 0, e, t, n, k, fmt,
                                        int(trans_b), _stream()))
     return out
+
+
+def moe_ffn_mxfp8(x, expert_idx, probs, w1, sw1, w2, sw2, trans_b=1):
+    """The MXFP8 MoE FFN of one rank that holds every expert, routing to combine, five launches on the current stream
+    (the reference's Ascend950DispatchFFNCombine, examples/ascend950_dispatch_ffn_combine/ascend950_dispatch_ffn_combine_device.h:124-176):
+    routing sort -> MXFP8 quantise-and-scatter -> GMM1 + SwiGLU + MXFP8 quantise -> GMM2 -> weighted un-permute.
+
+    x bf16 [m, k]; expert_idx int32 [m, top_k]; probs float32 [m, top_k]; w1 / sw1 and w2 / sw2 E4M3 payload and E8M0 scales
+    of the experts' up ([k, n], gate columns first) and down ([n/2, k]) projections in the layout `trans_b` names
+    (1, as the reference's files hold them: [E, n, k] and [E, k, n/2]).  Returns bf16 [m, k]."""
+    _require_gpu(x, expert_idx, probs, w1, sw1, w2, sw2)
+    if x.dim() != 2 or x.dtype != torch.bfloat16:
+        raise ValueError("x must be a 2-D bfloat16 tensor")
+    if expert_idx.dim() != 2 or expert_idx.shape[0] != x.shape[0] or probs.shape != expert_idx.shape:
+        raise ValueError("expert_idx and probs must be [m, top_k]")
+    m, k = x.shape
+    top_k, e = expert_idx.shape[1], w1.shape[0]
+    _, s2d, cnt = moe_init_routing(expert_idx, e)
+    packed = torch.empty((m * top_k, packed_row_bytes(k)), dtype=torch.uint8, device=x.device)
+    mx_quant_scatter_packed(x, s2d, packed, top_k)
+    act, act_scales = mx_grouped_matmul_swiglu_packed(packed, k, w1, sw1, cnt, "e4m3", trans_b, "e4m3")
+    y = mx_grouped_matmul(act, act_scales, w2, sw2, cnt, "e4m3", trans_b)
+    if y.shape[1] != k:
+        raise ValueError("w2 must map back to the hidden size of x")
+    return moe_token_unpermute(y, s2d, probs, top_k)
+

@@ -41,6 +41,7 @@ _lib.define("gmm_dequant_swiglu(Tensor x, Tensor w, Tensor group_sizes, Tensor p
 _lib.define("mx_grouped_matmul(Tensor a, Tensor sa, Tensor b, Tensor sb, Tensor group_sizes, str fmt, int trans_b) -> Tensor")
 _lib.define("mx_grouped_matmul_swiglu_mx(Tensor a, Tensor sa, Tensor b, Tensor sb, Tensor group_sizes, str fmt, int trans_b, str out_fmt) -> (Tensor, Tensor)")
 _lib.define("gmm_dequant_swiglu_mx(Tensor x, Tensor w, Tensor group_sizes, Tensor per_tok, Tensor per_ch, int trans_b, str fmt) -> (Tensor, Tensor)")
+_lib.define("moe_ffn_mxfp8(Tensor x, Tensor expert_idx, Tensor probs, Tensor w1, Tensor sw1, Tensor w2, Tensor sw2, int trans_b) -> Tensor")
 
 
 def _init(rank_id, rank_size, local_mem_size, ip_port):
@@ -87,6 +88,7 @@ _lib.impl("mx_matmul", _guarded(ops.mx_matmul), "CUDA")
 _lib.impl("gmm_dequant_swiglu", _guarded(ops.gmm_dequant_swiglu), "CUDA")
 _lib.impl("mx_grouped_matmul", _guarded(ops.mx_grouped_matmul), "CUDA")
 _lib.impl("gmm_dequant_swiglu_mx", _guarded(ops.gmm_dequant_swiglu_mx), "CUDA")
+_lib.impl("moe_ffn_mxfp8", _guarded(ops.moe_ffn_mxfp8), "CUDA")
 _lib.impl("mx_grouped_matmul_swiglu_mx", _guarded(lambda a, sa, b, sb, gs, fmt, tb, ofmt: ops.mx_grouped_matmul_swiglu(a, sa, b, sb, gs, fmt, tb, out_fmt=ofmt)),
           "CUDA")
 
@@ -136,6 +138,7 @@ def _mx_gmm_meta(a, sa, b, sb, group_sizes, fmt, trans_b):
     return a.new_empty((a.shape[0], _mx_n(b.shape[1:], fmt, trans_b)), dtype=torch.bfloat16)
 
 
+_lib.impl("moe_ffn_mxfp8", lambda x, expert_idx, probs, w1, sw1, w2, sw2, trans_b: x.new_empty(x.shape), "Meta")
 _lib.impl("mx_quant", _mx_quant_meta, "Meta")
 _lib.impl("w8a8_matmul_dequant", _w8a8_meta, "Meta")
 _lib.impl("mx_matmul", _mx_matmul_meta, "Meta")

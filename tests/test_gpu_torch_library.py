@@ -52,5 +52,20 @@ def test_ops_need_init_then_match_the_oracle():
         torch.cuda.synchronize()
         want_p, want_s = orc.mx_quant_rows(act.view(torch.int16).cpu().numpy().view(np.uint16), orc.E4M3)
         assert np.array_equal(pq.cpu().numpy(), want_p) and np.array_equal(sq.cpu().numpy(), want_s)
+        # the whole MXFP8 FFN in one op equals the chain of the single calls, to the bit (same launches)
+        import catccos_amd as cc
+        m, topk, n1 = 100, 2, 512
+        idx = dev(np.argsort(rng.random((m, e)), axis=1)[:, :topk].astype(np.int32))
+        probs = torch.softmax(torch.randn(m, topk, device="cuda"), dim=-1)
+        w1 = [cc.mx_quant_b(torch.randn(k, n1, device="cuda").to(torch.bfloat16) / k ** 0.5, "e4m3", trans_b=1) for _ in range(e)]
+        w2 = [cc.mx_quant_b(torch.randn(n1 // 2, k, device="cuda").to(torch.bfloat16) / (n1 // 2) ** 0.5, "e4m3", trans_b=1) for _ in range(e)]
+        b1, s1, b2, s2 = (torch.stack([w[i] for w in ws]) for ws in (w1, w2) for i in (0, 1))
+        out = OPS.moe_ffn_mxfp8(xd[:m], idx, probs, b1, s1, b2, s2, 1)
+        _, s2d, cnt = cc.moe_init_routing(idx, e)
+        packed = torch.empty((m * topk, cc.packed_row_bytes(k)), dtype=torch.uint8, device="cuda")
+        cc.mx_quant_scatter_packed(xd[:m], s2d, packed, topk)
+        a2, sa2 = cc.mx_grouped_matmul_swiglu(packed[:, :k].contiguous(), packed[:, k:].contiguous(), b1, s1, cnt, "e4m3", 1, out_fmt="e4m3")
+        want = cc.moe_token_unpermute(cc.mx_grouped_matmul(a2, sa2, b2, s2, cnt, "e4m3", 1), s2d, probs, topk)
+        assert out.shape == (m, k) and torch.equal(out, want)
     finally:
         assert OPS.finalize() == 0

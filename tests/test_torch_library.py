@@ -66,6 +66,9 @@ def test_meta_shapes(initialised):
     pq, sq = OPS.mx_grouped_matmul_swiglu_mx(u8(m, k), u8(m, 32), u8(e, k, n), u8(e, 16, n, 2), torch.empty(e, dtype=torch.int32, device="meta"),
                                              "e4m3", 0, "e4m3")
     assert pq.shape == (m, n // 2) and sq.shape == (m, 2 * ((n // 2 + 63) // 64))
+    out = OPS.moe_ffn_mxfp8(torch.empty((m, k), dtype=torch.bfloat16, device="meta"), torch.empty((m, 2), dtype=torch.int32, device="meta"), torch.empty((m, 2), device="meta"),
+                            u8(e, n, k), u8(e, n, 32), u8(e, k, n // 2), u8(e, k, 2 * ((n // 2 + 63) // 64)), 1)
+    assert out.shape == (m, k) and out.dtype == torch.bfloat16
 
 
 def test_cpu_tensors_have_no_kernel(initialised):
