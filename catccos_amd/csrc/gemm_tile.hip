@@ -12,7 +12,18 @@
 //     wave alternates between a memory slot (LDS fragment reads, global -> LDS requests) and a
 //     matrix slot (MFMAs only), the slots are separated by workgroup barriers, and the second
 //     group runs one slot behind the first: while one wave of a SIMD issues matrix instructions
-//     its neighbour fetches, and the next slot they swap.  A K-step is four slots per wave:
+//     its neighbour fetches, and the next slot they swap.  A K-step is four slots per wave.
+//     B stored [K, N] (a step's panel is 128 K-rows, so its two 64-byte halves of K are separate rows):
+//       L0  read the first half of the step: B fragments and the A fragments of all four row blocks;
+//           request the second-half K-rows of B of step k+1
+//       C0  MFMAs of the first half (all row blocks)
+//       L1  read the second half into the same registers; request the first-half K-rows of B of step k+2
+//           (the other group read them one slot ago) and the scales
+//       C1  MFMAs of the second half; request this group's A rows of step k+2 between them
+//     so both memory slots read the same amount (48 KiB per group) and fit under a matrix slot, and a
+//     request has four to six slots to land.  B stored [N, K] (every panel row holds both halves, nothing
+//     of a stage is free before both are read) keeps the split by row blocks, which leaves its requests
+//     more time:
 //       L0  read all B fragments of the step and the A fragments of row blocks 0-1;
 //           request the A rows of row blocks 2-3 of step k+1
 //       C0  MFMAs of row blocks 0-1 (both 64-byte halves of the step)
@@ -20,7 +31,7 @@
 //           request B and the A rows of row blocks 0-1 of step k+2 - their place in the ring is the
 //           stage being computed, whose B panel and first A rows nobody reads any more
 //       C1  MFMAs of row blocks 2-3
-//     so a request has five slots (1.25 steps) to land before the barrier that publishes it.
+//     (five slots, 1.25 steps, from a request to the barrier that publishes it).
 //   * MX scales travel 16 bytes per row at a time (4 MXFP8 steps, 2 MXFP4 steps) into a pair of
 //     scale buffers: a per-step 4-byte fetch touches one L2 line per lane and costs as many
 //     line requests as the whole data panel.
@@ -221,6 +232,15 @@ __device__ uint64_t cch_prof[256 * 8 * 8];
 #define PROF_END(t, acc)
 #endif
 
+// Which split of a step the kernels of either B layout use (1: by halves of K, 0: by row blocks); the defaults
+// are what measured best, a measurement build can set the other.
+#ifndef CCH_KSPLIT_TB0
+#define CCH_KSPLIT_TB0 1
+#endif
+#ifndef CCH_KSPLIT_TB1
+#define CCH_KSPLIT_TB1 0
+#endif
+
 constexpr uint32_t NO_FETCH = 0xFFFFFFF0u;   // a lane offset past every descriptor: the lane fetches nothing
 
 // What one tile needs, all wave-uniform except the per-lane source offsets.
@@ -264,6 +284,8 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     constexpr int NC0 = 2;                          // A rows of row blocks 0-1 of the step after the next
     constexpr int NL1 = NJ / 2 + (MX ? 1 : 0);      // half of the B panel share, scales (or a request that fetches nothing)
     constexpr int NC1 = NJ / 2;                     // the other half of the B panel share
+    // The other split of a step's work over the two slot pairs (see `step`): by 64-byte halves of K instead of by row blocks.
+    constexpr bool KSPLIT = TB ? (CCH_KSPLIT_TB1 != 0) : (CCH_KSPLIT_TB0 != 0);
 
     __shared__ GroupTable tab;
     if (threadIdx.x == 0) build_group_table(tab, p.group_sizes, p.num_groups, p.T, BM);
@@ -327,7 +349,9 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     for (int j = 0; j < NT; j++) fr_bt[j] = lds_base + (uint32_t)RING_B_OFF + (rd_bt ^ ((uint32_t)j << (FP4K ? 4 : 5)));
     // wave-uniform LDS addresses of the first panel request of this wave (stage 0)
     const uint32_t lds_req_a = lds_base + (uint32_t)RING_OFF + (uint32_t)(wm * WM + wn * 16) * BKB;
-    const uint32_t lds_req_b = lds_base + (uint32_t)RING_B_OFF + (uint32_t)(wave * NJ) * 1024u;
+    // (K-half split, TB = 0: requests 0-1 of a wave land in the K-rows of the first 64-byte half, KiB 2*wave + j of the
+    // panel, requests 2-3 in those of the second half, KiB 16 + 2*wave + j - 2)
+    const uint32_t lds_req_b = lds_base + (uint32_t)RING_B_OFF + (uint32_t)(wave * ((KSPLIT && !TB) ? 2 : NJ)) * 1024u;
     const int ldb = TB ? lda : p.N / EPB;   // bytes between consecutive rows of B as stored
     const uint32_t b_bytes = (uint32_t)min((int64_t)p.N * lda, (int64_t)0x7FFFFFFF);   // one right-hand operand
     const uint32_t b_step = (uint32_t)(BKB * EPB) * (uint32_t)ldb;                      // TB = 0: bytes of B between K-steps
@@ -385,7 +409,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             const int col = SWIGLU ? ((brow >> 5) & 1) * p.n_out + (brow >> 6) * 32 + (brow & 31) : brow;   // relative to j0
             off_b[q] = (uint32_t)col * (uint32_t)lda + chunk;
         } else {
-            const int kr = (wave * NJ + q) * BRPI + lane / BCPR;
+            const int kr = ((KSPLIT ? (q >> 1) * 16 + wave * 2 + (q & 1) : wave * NJ + q)) * BRPI + lane / BCPR;
             const int tc = (lane % BCPR) ^ (FP4K ? (kr >> 1) & 7 : (kr & 7) << 1);
             // relative to j0 (FP4: a chunk is 32 columns, one whole gate or up block)
             const int col = !SWIGLU ? tc * 16 * EPB : FP4K ? (tc & 1) * p.n_out + (tc >> 1) * 32 : ((tc >> 1) & 1) * p.n_out + (tc >> 2) * 32 + (tc & 1) * 16;
@@ -511,7 +535,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             const uint32_t voff = ((j & 1) ? tl.ok1 : tl.ok0) ? off_b[j] : NO_FETCH;
             load16_to_lds_at<STG * PANEL_BYTES + j * 1024>(c.rs_b, voff, (uint32_t)tl.koff, lds_req_b);
         } else {
-            load16_to_lds_at<STG * PANEL_BYTES + j * 1024>(c.rs_b, off_b[j] + boff, 0u, lds_req_b);
+            load16_to_lds_at<STG * PANEL_BYTES + (KSPLIT ? (j >> 1) * 16 + (j & 1) : j) * 1024>(c.rs_b, off_b[j] + boff, 0u, lds_req_b);
         }
     };
     auto boff_of = [&](int kstep) {
@@ -627,9 +651,18 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             static_for<NJ>([&](auto q_c) { issue_a(cur, t0, IC<0>{}, q_c); });
             issue_scales(prep_scales(1, cur, 0));
             issue_params(cur, 0);
-            static_for<NJ>([&](auto j_c) { issue_b(cur, t1, boff_of(1), IC<1>{}, j_c); });
-            issue_a(cur, t1, IC<1>{}, IC<0>{});
-            issue_a(cur, t1, IC<1>{}, IC<1>{});
+            if constexpr (KSPLIT) {
+                // (slot L0 of step 0 requests the rest of step 1's B panel)
+                if constexpr (!TB) {
+                    issue_b(cur, t1, boff_of(1), IC<1>{}, IC<0>{});
+                    issue_b(cur, t1, boff_of(1), IC<1>{}, IC<1>{});
+                }
+                static_for<NJ>([&](auto q_c) { issue_a(cur, t1, IC<1>{}, q_c); });
+            } else {
+                static_for<NJ>([&](auto j_c) { issue_b(cur, t1, boff_of(1), IC<1>{}, j_c); });
+                issue_a(cur, t1, IC<1>{}, IC<0>{});
+                issue_a(cur, t1, IC<1>{}, IC<1>{});
+            }
             issue_scales(prep_scales(SPG == 2 && nk_tile > 2, cur, 1));
         }
         prep_scale_reads(0);
@@ -743,13 +776,14 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             if (!decltype(zero_c)::value) { asm volatile("" :: "v"(a)); return; }
 #endif
             constexpr bool ZERO = decltype(zero_c)::value != 0;
+            constexpr int fbi = KSPLIT ? 0 : ks;   // K-half split: the B fragments of the current half sit in fb[j][0]
             if constexpr (KIND == KIND_F8) {
 #pragma unroll
                 for (int j = 0; j < NT; j++) {
                     Acc c;
                     if (ZERO) c = (Acc)(0.0f);
                     else c = acc[ai][j];
-                    acc[ai][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, fb[j][ks], c, CBSZ, CBSZ, 2 * ks, (int)sc[0][ai], 2 * ks,
+                    acc[ai][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, fb[j][fbi], c, CBSZ, CBSZ, 2 * ks, (int)sc[0][ai], 2 * ks,
                                                                                  (int)sc[0][MT + j]);
                 }
             } else {
@@ -763,14 +797,14 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                         if constexpr (KIND == KIND_F4) {
                             // substep = 128 elements = scale dword ks; the low MFMA uses byte g, the high one byte 2+g
                             const v8i ah = (v8i){a[4 * half], a[4 * half + 1], a[4 * half + 2], a[4 * half + 3], 0, 0, 0, 0};
-                            const v8i bh = (v8i){fb[j][ks][4 * half], fb[j][ks][4 * half + 1], fb[j][ks][4 * half + 2], fb[j][ks][4 * half + 3], 0, 0, 0, 0};
+                            const v8i bh = (v8i){fb[j][fbi][4 * half], fb[j][fbi][4 * half + 1], fb[j][fbi][4 * half + 2], fb[j][fbi][4 * half + 3], 0, 0, 0, 0};
                             if (half == 0)
                                 acc[ai][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ah, bh, c, 4, 4, 0, (int)sc[ks][ai], 0, (int)sc[ks][MT + j]);
                             else
                                 acc[ai][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ah, bh, c, 4, 4, 2, (int)sc[ks][ai], 2, (int)sc[ks][MT + j]);
                         } else {
                             const v4i ah = (v4i){a[4 * half], a[4 * half + 1], a[4 * half + 2], a[4 * half + 3]};
-                            const v4i bh = (v4i){fb[j][ks][4 * half], fb[j][ks][4 * half + 1], fb[j][ks][4 * half + 2], fb[j][ks][4 * half + 3]};
+                            const v4i bh = (v4i){fb[j][fbi][4 * half], fb[j][fbi][4 * half + 1], fb[j][fbi][4 * half + 2], fb[j][fbi][4 * half + 3]};
                             acc[ai][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ah, bh, c, 0, 0, 0);
                         }
                     }
@@ -809,6 +843,112 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 #pragma unroll
                 for (int j = 0; j < NT; j++) asm volatile("" : "+v"(fr_bt[j]));
             }
+            if constexpr (KSPLIT) {
+                // K-half split.  L0 reads the first 64-byte half of the step (B fragments and the A fragments of
+                // all four row blocks), C0 multiplies it, L1 reads the second half into the same registers, C1
+                // multiplies that: the two memory slots read the same amount and both fit under a matrix slot.
+                // A stage is free once both halves are read, so the requests are: L0 the second-half K-rows of
+                // the next step's B panel (TB = 1: the whole panel, whose rows hold both halves), L1 the
+                // first-half K-rows of B two steps ahead (the other group read them one slot ago) and the scales,
+                // C1 the A rows two steps ahead (a group's A rows are read by that group alone).
+                constexpr int NB_L0 = TB ? NJ : NJ / 2, NB_L1 = TB ? 0 : NJ / 2;
+                constexpr int KL1 = NB_L1 + (MX ? 1 : 0), KC1 = NJ;
+                constexpr int K_PREV_L1 = KL1 + (MODE == 2 ? NPARAM : 0), K_THIS_L1 = KL1 + (MODE == 1 ? NPARAM : 0);
+                constexpr int NBLK = 2 * MTH;   // row blocks of this wave that hold rows of the group
+                // ------------------------------------------------------------------ L0
+                if constexpr (MTH > 0) {
+                    read_scales_raw();
+#pragma unroll
+                    for (int j = 0; j < NT; j++) fb[j][0] = frag_b(stg_c, 0, j);
+                    __builtin_amdgcn_sched_barrier(0);
+                    finish_scales(IC<MODE != 0>{}, kt);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int i = 0; i < NBLK; i++) fa[i & 1][i >> 1] = frag_a(stg_c, 0, i);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                {
+                    const TileCtx &nc = MODE == 2 ? nxt : cur;
+                    const int nk1 = MODE == 2 ? 0 : kt + 1;
+                    const Tail tl = tail_of(nk1);
+                    uint32_t nb = 0;
+                    if constexpr (!TB) nb = boff_of(nk1);
+                    if constexpr (TB) {
+                        issue_b(nc, tl, nb, IC<STG ^ 1>{}, IC<0>{});
+                        issue_b(nc, tl, nb, IC<STG ^ 1>{}, IC<1>{});
+                    }
+                    issue_b(nc, tl, nb, IC<STG ^ 1>{}, IC<2>{});
+                    issue_b(nc, tl, nb, IC<STG ^ 1>{}, IC<3>{});
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                { PROF_BEGIN(t_); CCH_WAIT_LGKM0(); PROF_END(t_, pf_l0); }
+                // TB = 0: the second-half K-rows of this step's B panel (requested in the previous step's L0) must have
+                // landed: younger are the previous step's L1 and C1, the stores and this L0
+                if constexpr (!TB) { PROF_BEGIN(t_); CCH_WAIT_VM(K_PREV_L1 + KC1 + STORES + NB_L0); PROF_END(t_, pf_wa); }
+                { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b0); }
+                // ------------------------------------------------------------------ C0
+                ScaleReq sreq;
+                if constexpr (MTH > 0) {
+                    static_for<NBLK>([&](auto i_c) {
+                        constexpr int i = decltype(i_c)::value;
+                        mfma_block(IC<FIRST>{}, IC<0>{}, i_c, fa[i & 1][i >> 1]);
+                    });
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                const Tail rq_tl = tail_of(rq_kt);
+                uint32_t rq_boff = 0;
+                if constexpr (!TB) rq_boff = boff_of(rq_kt);
+                if constexpr (MX) {
+                    if constexpr (MODE == 0) {
+                        sreq = prep_scales(((kt + 3) & (SPG - 1)) == 0 && kt + 3 < nk_tile, cur, (kt + 3) / SPG);
+                    } else if constexpr (MODE == 1) {
+                        nbase = gi;
+                        sreq = prep_scales(1, nxt, 0);
+                    } else {
+                        sreq = prep_scales(SPG == 2 && nk_tile > 2, nxt, 1);
+                    }
+                    asm volatile("" : "+s"(sreq.rs), "+v"(sreq.voff), "+s"(sreq.dst));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b1); }
+                // ------------------------------------------------------------------ L1
+                if constexpr (MTH > 0) {
+#pragma unroll
+                    for (int j = 0; j < NT; j++) fb[j][0] = frag_b(stg_c, 1, j);
+#pragma unroll
+                    for (int i = 0; i < NBLK; i++) fa[i & 1][i >> 1] = frag_a(stg_c, 1, i);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (!TB) {
+                    issue_b(rq, rq_tl, rq_boff, stg_c, IC<0>{});
+                    issue_b(rq, rq_tl, rq_boff, stg_c, IC<1>{});
+                }
+                issue_scales(sreq);
+                if constexpr (MODE == 1) issue_params(nxt, parity ^ 1);
+                __builtin_amdgcn_sched_barrier(0);
+                // what the next step's L0 reads of B must have landed.  TB = 0: its first-half K-rows and scales,
+                // requested in the previous step's L1; younger are that step's C1, the stores and this step's L0 and
+                // L1.  TB = 1: the whole panel, requested in this step's L0; younger is this L1.
+                { PROF_BEGIN(t_); CCH_WAIT_VM_LGKM0(TB ? K_THIS_L1 : KC1 + STORES + NB_L0 + K_THIS_L1); PROF_END(t_, pf_wb); }
+                { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b2); }
+                // ------------------------------------------------------------------ C1
+                static_for<NJ>([&](auto q_c) {
+                    constexpr int q = decltype(q_c)::value;
+                    if constexpr (q < NBLK) {
+                        mfma_block(IC<0>{}, IC<1>{}, q_c, fa[q & 1][q >> 1]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    issue_a(rq, rq_tl, stg_c, q_c);
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+                if constexpr (MODE == 2) prep_scale_reads(nbase);
+                else advance_scale_reads(gbase, kt);
+                __builtin_amdgcn_sched_barrier(0);
+                // this group's A rows of the next step (requested in the previous step's C1) must have landed:
+                // younger are the stores and this step's L0, L1 and C1
+                { PROF_BEGIN(t_); CCH_WAIT_VM(STORES + NB_L0 + K_THIS_L1 + KC1); PROF_END(t_, pf_wa); }
+                if constexpr (MODE != 2) { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b3); }
+            } else {
             // ------------------------------------------------------------------ L0
             if constexpr (MTH > 0) {
                 read_scales_raw();
@@ -918,6 +1058,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             else advance_scale_reads(gbase, kt);
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (MODE != 2) { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b3); }
+            }
             if constexpr (FIRST && MTH < 2) {
                 // row blocks that hold no row of the group are never stored; give them a value all the same
 #pragma unroll
