@@ -53,3 +53,37 @@ def test_captured_chain_replays_like_eager():
                 assert torch.equal(got, want), rep
     finally:
         cc.set_option("require_tiled_gemm", 0)
+
+
+def test_captured_ffn_follows_new_routing():
+    """The whole MXFP8 FFN (routing sort, quantise-and-scatter, both grouped matmuls, un-permute) in one graph: the
+    group sizes and row maps are device data that the graph's own kernels produce, so a replay follows new routes
+    and new tokens written into the captured input buffers; every replay equals the eager result bit for bit."""
+    torch.manual_seed(1)
+    m, k, n, e, topk = 200, 512, 1024, 8, 2
+    x = torch.randn(m, k, device="cuda").to(torch.bfloat16)
+    idx = torch.argsort(torch.rand(m, e, device="cuda"), dim=1)[:, :topk].to(torch.int32).contiguous()
+    probs = torch.softmax(torch.randn(m, topk, device="cuda"), dim=-1)
+    w1 = [cc.mx_quant_b(torch.randn(k, n, device="cuda").to(torch.bfloat16) / k ** 0.5, "e4m3", trans_b=1) for _ in range(e)]
+    w2 = [cc.mx_quant_b(torch.randn(n // 2, k, device="cuda").to(torch.bfloat16) / (n // 2) ** 0.5, "e4m3", trans_b=1) for _ in range(e)]
+    b1, s1, b2, s2 = (torch.stack([w[i] for w in ws]) for ws in (w1, w2) for i in (0, 1))
+    cc.set_option("require_tiled_gemm", 1)
+    try:
+        eager = cc.moe_ffn_mxfp8(x, idx, probs, b1, s1, b2, s2).clone()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = cc.moe_ffn_mxfp8(x, idx, probs, b1, s1, b2, s2)
+        for rep in range(4):
+            if rep == 2:
+                # other tokens, and routes that leave three experts empty
+                x.copy_((torch.randn(m, k, device="cuda") * 2).to(torch.bfloat16))
+                idx.copy_(torch.argsort(torch.rand(m, e - 3, device="cuda"), dim=1)[:, :topk].to(torch.int32))
+                eager = cc.moe_ffn_mxfp8(x, idx, probs, b1, s1, b2, s2).clone()
+            out.fill_(0)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), rep
+    finally:
+        cc.set_option("require_tiled_gemm", 0)
