@@ -636,6 +636,51 @@ def main():
                 "tflops_mxfp8_out": round(flop / (tq * 1e-3) / 1e12, 1),
                 "parity": {"bit_exact_vs_quantised_bf16_output": bool(torch.equal(pu, pv) and torch.equal(su, sv))}}
             del pu, su, pv, sv
+            # The MXFP8 FFN of one rank from routing to combine, at the largest shape of the reference example's own list
+            # (examples/ascend950_dispatch_ffn_combine/scripts/test_shapes.csv: 512 tokens, K 7168, N 4096) with its run.sh's
+            # 16 experts and top-6: seven launches (routing sort x3, quantise-and-scatter, GMM1 + SwiGLU + quantise, GMM2,
+            # un-permute), eager and as one HIP graph.  Weight bytes per pass: 16 x (29.4 + 14.7) MB + scales = 0.73 GB.
+            mf, ef, topf = 512, 16, 6
+            xf = torch.randn(mf, K, device=dev).to(torch.bfloat16)
+            idf = torch.argsort(torch.rand(mf, ef, device=dev), dim=1)[:, :topf].to(torch.int32).contiguous()
+            prf = torch.softmax(torch.randn(mf, topf, device=dev), dim=-1)
+            w1f = [cc.mx_quant_b((torch.randn(K, N, device=dev) / K ** 0.5).to(torch.bfloat16), "e4m3", trans_b=1) for _ in range(ef)]
+            w2f = [cc.mx_quant_b((torch.randn(N // 2, K, device=dev) / (N // 2) ** 0.5).to(torch.bfloat16), "e4m3", trans_b=1) for _ in range(ef)]
+            b1f, s1f, b2f, s2f = (torch.stack([w[i] for w in ws]) for ws in (w1f, w2f) for i in (0, 1))
+            del w1f, w2f
+            ffn = lambda: cc.moe_ffn_mxfp8(xf, idf, prf, b1f, s1f, b2f, s2f)   # noqa: E731
+            t_eager = queue_time_ms(ffn, 30, 60.0)
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                out_g = ffn()
+            t_graph = queue_time_ms(gr.replay, 30, 60.0)
+            ffn_flop = 2.0 * mf * topf * (K * N + (N // 2) * K)
+            wbytes = b1f.numel() + s1f.numel() + b2f.numel() + s2f.numel()
+            ent = {"us_eager": round(t_eager * 1e3, 1), "us_graph": round(t_graph * 1e3, 1), "tflops_graph": round(ffn_flop / (t_graph * 1e-3) / 1e12, 1),
+                   "weight_tb_s_graph": round(wbytes / (t_graph * 1e-3) / 1e12, 2),
+                   "workload": "%d tokens, top-%d of %d experts, K %d, N %d, weights [E,N,K] / [E,K,N/2] as the reference's files" % (mf, topf, ef, K, N)}
+            if cpu:
+                gr.replay()
+                torch.cuda.synchronize()
+                got = out_g.float().cpu().numpy()
+                xh = xf.view(torch.int16).cpu().numpy().view(np.uint16)
+                b1h, s1h, b2h, s2h = (v.cpu().numpy() for v in (b1f, s1f, b2f, s2f))
+                t0 = time.perf_counter()
+                _, s2d_h, cnt_h = orc.moe_init_routing(idf.cpu().numpy(), ef)
+                pk = orc.mx_quant_scatter_packed(xh, s2d_h, mf * topf, topf, orc.E4M3)
+                _, c1 = orc.mx_gmm(pk[:, :K], pk[:, K:], b1h, s1h, N, K, orc.E4M3, 1, group_sizes=cnt_h, want_bf16=True, blocked=True)
+                a2h, sa2h = orc.mx_quant_rows(orc.swiglu_bf16(c1), orc.E4M3)
+                _, yh = orc.mx_gmm(a2h, sa2h, b2h, s2h, K, N // 2, orc.E4M3, 1, group_sizes=cnt_h, want_bf16=True, blocked=True)
+                want = orc.bf16_to_f32(orc.moe_token_unpermute(yh, s2d_h, prf.cpu().numpy(), topf))
+                dt = time.perf_counter() - t0
+                ent["cpu_baseline"] = {"value": round(ffn_flop / dt / 1e12, 4), "unit": "TFLOP/s", "cores": orc.num_threads(), "kind": "port",
+                                       "sample": "the whole chain on the same inputs, %.1f s, cache-blocked CPU GEMMs" % dt}
+                rms = float(np.sqrt(np.mean(want ** 2)))
+                # two implementations of this chain differ where a bf16 step of GMM1 moves a code of the quantised activation
+                ent["parity"] = {"rms_err_over_rms": float(np.sqrt(np.mean((got - want) ** 2)) / rms), "max_err_over_rms": float(np.abs(got - want).max() / rms),
+                                 "rows_checked": mf, "stagewise_bit_exact_checks": "tests/test_gpu_ffn_chain.py"}
+            extra["mxfp8_ffn_chain_reference_shape"] = ent
+            del b1f, s1f, b2f, s2f, gr, out_g
             # Yardstick, not part of this build: the vendor library's dense FP8 GEMM (per-tensor scales, E4M3,
             # bf16 out) on the headline's shape as one group, and this kernel on the same bytes with unit scales.
             try:
