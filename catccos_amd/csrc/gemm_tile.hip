@@ -770,8 +770,9 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // The MFMAs of row block ai on the 64-byte substep ks: all column blocks on the low 32
         // bytes, then (int8 and FP4, which take two MFMAs per 64 bytes) all on the high 32 bytes.
         // With ZERO the accumulators start from zero instead of being read.
-        auto mfma_block = [&](auto zero_c, auto ks_c, auto ai_c, const v8i &a) {
-            constexpr int ks = decltype(ks_c)::value, ai = decltype(ai_c)::value;
+        // (int8 and FP4: `only_c` 0 or 1 issues the MFMAs of that 32-byte half alone, -1 both)
+        auto mfma_block = [&](auto zero_c, auto ks_c, auto ai_c, const v8i &a, auto only_c) {
+            constexpr int ks = decltype(ks_c)::value, ai = decltype(ai_c)::value, ONLY = decltype(only_c)::value;
 #ifdef CCH_V_NOMFMA
             if (!decltype(zero_c)::value) { asm volatile("" :: "v"(a)); return; }
 #endif
@@ -791,6 +792,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 for (int half = 0; half < 2; half++)
 #pragma unroll
                     for (int j = 0; j < NT; j++) {
+                        if (ONLY >= 0 && half != ONLY) continue;
                         Acc c;
                         if (ZERO && half == 0) c = (Acc)(0);
                         else c = acc[ai][j];
@@ -889,9 +891,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 // ------------------------------------------------------------------ C0
                 ScaleReq sreq;
                 if constexpr (MTH > 0) {
-                    static_for<NBLK>([&](auto i_c) {
-                        constexpr int i = decltype(i_c)::value;
-                        mfma_block(IC<FIRST>{}, IC<0>{}, i_c, fa[i & 1][i >> 1]);
+                    // (int8 and FP4 take two MFMAs per accumulator and half of K: all row blocks on the first 32 bytes, then
+                    // all on the second, so that an accumulator's two MFMAs are not neighbours in the pipe)
+                    static_for<(KIND == KIND_F8 ? 1 : 2)>([&](auto h_c) {
+                        static_for<NBLK>([&](auto i_c) {
+                            constexpr int i = decltype(i_c)::value;
+                            mfma_block(IC<FIRST>{}, IC<0>{}, i_c, fa[i & 1][i >> 1], IC<(KIND == KIND_F8 ? -1 : decltype(h_c)::value)>{});
+                        });
                     });
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -935,12 +941,18 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 static_for<NJ>([&](auto q_c) {
                     constexpr int q = decltype(q_c)::value;
                     if constexpr (q < NBLK) {
-                        mfma_block(IC<0>{}, IC<1>{}, q_c, fa[q & 1][q >> 1]);
+                        mfma_block(IC<0>{}, IC<1>{}, q_c, fa[q & 1][q >> 1], IC<(KIND == KIND_F8 ? -1 : 0)>{});
                         __builtin_amdgcn_sched_barrier(0);
                     }
                     issue_a(rq, rq_tl, stg_c, q_c);
                     __builtin_amdgcn_sched_barrier(0);
                 });
+                if constexpr (KIND != KIND_F8) {
+                    static_for<NBLK>([&](auto q_c) {
+                        constexpr int q = decltype(q_c)::value;
+                        mfma_block(IC<0>{}, IC<1>{}, q_c, fa[q & 1][q >> 1], IC<1>{});
+                    });
+                }
                 if constexpr (MODE == 2) prep_scale_reads(nbase);
                 else advance_scale_reads(gbase, kt);
                 __builtin_amdgcn_sched_barrier(0);
@@ -981,18 +993,18 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             Tail rq_tl;
             uint32_t rq_boff = 0;
             if constexpr (MTH > 0) {
-                mfma_block(IC<FIRST>{}, IC<0>{}, IC<0>{}, fa[0][0]);
+                mfma_block(IC<FIRST>{}, IC<0>{}, IC<0>{}, fa[0][0], IC<-1>{});
                 __builtin_amdgcn_sched_barrier(0);
                 rq_tl = tail_of(rq_kt);
                 if constexpr (!TB) rq_boff = boff_of(rq_kt);
                 issue_a(rq, rq_tl, stg_c, IC<0>{});
                 __builtin_amdgcn_sched_barrier(0);
-                mfma_block(IC<FIRST>{}, IC<0>{}, IC<1>{}, fa[1][0]);
+                mfma_block(IC<FIRST>{}, IC<0>{}, IC<1>{}, fa[1][0], IC<-1>{});
                 __builtin_amdgcn_sched_barrier(0);
                 issue_a(rq, rq_tl, stg_c, IC<1>{});
                 __builtin_amdgcn_sched_barrier(0);
-                mfma_block(IC<0>{}, IC<1>{}, IC<0>{}, fa[0][1]);
-                mfma_block(IC<0>{}, IC<1>{}, IC<1>{}, fa[1][1]);
+                mfma_block(IC<0>{}, IC<1>{}, IC<0>{}, fa[0][1], IC<-1>{});
+                mfma_block(IC<0>{}, IC<1>{}, IC<1>{}, fa[1][1], IC<-1>{});
             } else {
                 rq_tl = tail_of(rq_kt);
                 if constexpr (!TB) rq_boff = boff_of(rq_kt);
@@ -1038,16 +1050,16 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b2); }
             // ------------------------------------------------------------------ C1
             if constexpr (MTH > 1) {
-                mfma_block(IC<FIRST>{}, IC<0>{}, IC<2>{}, fa[0][0]);
+                mfma_block(IC<FIRST>{}, IC<0>{}, IC<2>{}, fa[0][0], IC<-1>{});
                 __builtin_amdgcn_sched_barrier(0);
                 issue_b(rq, rq_tl, rq_boff, stg_c, IC<2>{});
                 __builtin_amdgcn_sched_barrier(0);
-                mfma_block(IC<FIRST>{}, IC<0>{}, IC<3>{}, fa[1][0]);
+                mfma_block(IC<FIRST>{}, IC<0>{}, IC<3>{}, fa[1][0], IC<-1>{});
                 __builtin_amdgcn_sched_barrier(0);
                 issue_b(rq, rq_tl, rq_boff, stg_c, IC<3>{});
                 __builtin_amdgcn_sched_barrier(0);
-                mfma_block(IC<0>{}, IC<1>{}, IC<2>{}, fa[0][1]);
-                mfma_block(IC<0>{}, IC<1>{}, IC<3>{}, fa[1][1]);
+                mfma_block(IC<0>{}, IC<1>{}, IC<2>{}, fa[0][1], IC<-1>{});
+                mfma_block(IC<0>{}, IC<1>{}, IC<3>{}, fa[1][1], IC<-1>{});
             } else {
                 issue_b(rq, rq_tl, rq_boff, stg_c, IC<2>{});
                 issue_b(rq, rq_tl, rq_boff, stg_c, IC<3>{});
