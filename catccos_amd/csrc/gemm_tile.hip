@@ -130,12 +130,16 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 
 // Workgroup barrier that the compiler moves no memory access across (the intrinsic alone is not a
 // memory barrier to the optimiser) and that the instruction scheduler leaves where it is.
+#ifdef CCH_V_NOBARRIER
+#define CCH_BARRIER() __builtin_amdgcn_sched_barrier(0)
+#else
 #define CCH_BARRIER()                                  \
     do {                                               \
         __builtin_amdgcn_sched_barrier(0);             \
         asm volatile("s_barrier" ::: "memory");        \
         __builtin_amdgcn_sched_barrier(0);             \
     } while (0)
+#endif
 
 // 16 / 4 bytes per lane, global -> LDS without passing through registers, as raw buffer loads:
 // the descriptor holds the wave-uniform base, `voff` is the per-lane byte offset, `soff` a
@@ -221,7 +225,11 @@ __device__ __forceinline__ uint32_t swizzle_of_row(int row) { return (uint32_t)(
 //                    then the seven waits in program order);
 //   -DCCH_V_NOLOAD   no panel requests: matrix instructions and LDS reads alone (the MFMA-side ceiling);
 //   -DCCH_V_NOMFMA   no matrix instructions after a tile's first step: requests, LDS reads, waits and
-//                    barriers alone (the memory-side ceiling).
+//                    barriers alone (the memory-side ceiling);
+//   -DCCH_V_NOLDS    no fragment reads, -DCCH_V_NOBARRIER no workgroup barriers in the K loop, -DCCH_V_NOEPI no
+//                    epilogue, -DCCH_V_NOSCALE the unscaled form of the MXFP8 matrix instruction: with
+//                    CCH_V_NOLOAD they take the matrix side apart (what is left is MFMA issue, tile decode and
+//                    the kernel's start).
 // `python -m catccos_amd.build --only lib --define NAME --out DIR` builds one.
 #ifdef CCH_PROF
 __device__ uint64_t cch_prof[256 * 8 * 8];
@@ -682,12 +690,18 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 
         auto frag_a = [&](auto stg_c, int ks, int i) {
             constexpr int STG = decltype(stg_c)::value;
+#ifdef CCH_V_NOLDS
+            { v8i z; asm volatile("" : "=v"(z)); return z; }
+#endif
             const v4i lo = lds_read16_abs(fr_a[ks * 2] + (uint32_t)(STG * PANEL_BYTES + i * 32 * BKB));
             const v4i hi = lds_read16_abs(fr_a[ks * 2 + 1] + (uint32_t)(STG * PANEL_BYTES + i * 32 * BKB));
             return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         };
         auto frag_b = [&](auto stg_c, int ks, int j) {
             constexpr int STG = decltype(stg_c)::value;
+#ifdef CCH_V_NOLDS
+            { v8i z; asm volatile("" : "=v"(z)); return z; }
+#endif
             if constexpr (TB) {
                 const v4i lo = lds_read16_abs(fr_b[ks * 2] + (uint32_t)(STG * PANEL_BYTES + j * 32 * BKB));
                 const v4i hi = lds_read16_abs(fr_b[ks * 2 + 1] + (uint32_t)(STG * PANEL_BYTES + j * 32 * BKB));
@@ -784,8 +798,12 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                     Acc c;
                     if (ZERO) c = (Acc)(0.0f);
                     else c = acc[ai][j];
+#ifdef CCH_V_NOSCALE
+                    acc[ai][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, fb[j][fbi], c, CBSZ, CBSZ, 0, 0, 0, 0);
+#else
                     acc[ai][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, fb[j][fbi], c, CBSZ, CBSZ, 2 * ks, (int)sc[0][ai], 2 * ks,
                                                                                  (int)sc[0][MT + j]);
+#endif
                 }
             } else {
 #pragma unroll
@@ -1129,6 +1147,9 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // writes two adjacent bf16, then every lane reads back 16 contiguous bytes and stores
         // them.  Stores are raw buffer stores whose out-of-range lanes are dropped by the
         // bounds check.
+#ifdef CCH_V_NOEPI
+        if (p.T < 0)   // never: the accumulators stay live, nothing is stored
+#endif
         {
             const uint32_t epi = (uint32_t)(EPI_OFF + wave * EPI_WAVE);
             const uint32_t prm = (uint32_t)(PARAM_OFF + parity * PARAM_SET);
@@ -1145,110 +1166,145 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
 #pragma unroll
                 for (int j = 0; j < NT; j++) chs[j] = __uint_as_float(lds_read4(prm + 1024u + (uint32_t)(wn * WN + j * 32 + r) * 4u));
             }
+            // One pass = PASS_ROWS rows of a 32-row block: `produce` converts and writes them into the staging
+            // buffer, `readback` fetches this lane's 16 bytes (and the row's destination), `emit` stores them.
+            // The passes are software-pipelined: the values of pass n+1 are converted and written while the read
+            // of pass n is under way (one wave's LDS operations execute in order, so the later writes cannot
+            // overtake the earlier read), and only then is pass n stored.
+            auto produce = [&](auto i_c, auto ps_c, auto fp16_c) {
+                constexpr int i = decltype(i_c)::value, ps = decltype(ps_c)::value;
 #pragma unroll
-            for (int i = 0; i < MT; i++) {
+                for (int qq = 0; qq < PASS_ROWS / 8; qq++) {
+                    const int q = ps * (PASS_ROWS / 8) + qq;
+                    float tok[4];
+                    if (DEQ) {
+                        const v4i tv = lds_read16(prm + (uint32_t)(wm * WM + i * 32 + q * 8 + g * 4) * 4u);
 #pragma unroll
-                for (int ps = 0; ps < NPASS; ps++) {
+                        for (int xr = 0; xr < 4; xr++) tok[xr] = __int_as_float(tv[xr]);
+                    }
 #pragma unroll
-                    for (int qq = 0; qq < PASS_ROWS / 8; qq++) {
-                        const int q = ps * (PASS_ROWS / 8) + qq;
-                        float tok[4];
-                        if (DEQ) {
-                            const v4i tv = lds_read16(prm + (uint32_t)(wm * WM + i * 32 + q * 8 + g * 4) * 4u);
+                    for (int xr = 0; xr < 4; xr += 2)
 #pragma unroll
-                            for (int xr = 0; xr < 4; xr++) tok[xr] = __int_as_float(tv[xr]);
-                        }
+                        for (int j = 0; j < (SWIGLU ? 1 : NT); j++) {
+                            const int x = q * 4 + xr;
+                            float v[2];
 #pragma unroll
-                        for (int xr = 0; xr < 4; xr += 2)
-#pragma unroll
-                            for (int j = 0; j < (SWIGLU ? 1 : NT); j++) {
-                                const int x = q * 4 + xr;
-                                float v[2];
-#pragma unroll
-                                for (int d = 0; d < 2; d++) {
-                                    if (EPI == EPI_SWIGLU) {
-                                        // the up projection's result is a bf16 tile before the activation sees it
-                                        const float gate = (float)(__bf16)(float)acc[i][0][x + d];
-                                        const float up = (float)(__bf16)(float)acc[i][1][x + d];
-                                        v[d] = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;
-                                    } else if (SWIGLU) {
-                                        const float gate = (float)acc[i][0][x + d] * chs[0] * tok[xr + d];
-                                        const float up = (float)acc[i][1][x + d] * chs[1] * tok[xr + d];
-                                        // hardware exp2 and reciprocal: relative error ~1e-6, far inside the bf16 result
-                                        v[d] = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;
-                                    } else if (EPI == EPI_DEQUANT) {
-                                        v[d] = (float)acc[i][j][x + d] * tok[xr + d] * chs[j];
-                                    } else {
-                                        v[d] = (float)acc[i][j][x + d];
-                                    }
+                            for (int d = 0; d < 2; d++) {
+                                if (EPI == EPI_SWIGLU) {
+                                    // the up projection's result is a bf16 tile before the activation sees it
+                                    const float gate = (float)(__bf16)(float)acc[i][0][x + d];
+                                    const float up = (float)(__bf16)(float)acc[i][1][x + d];
+                                    v[d] = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;
+                                } else if (SWIGLU) {
+                                    const float gate = (float)acc[i][0][x + d] * chs[0] * tok[xr + d];
+                                    const float up = (float)acc[i][1][x + d] * chs[1] * tok[xr + d];
+                                    // hardware exp2 and reciprocal: relative error ~1e-6, far inside the bf16 result
+                                    v[d] = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;
+                                } else if (EPI == EPI_DEQUANT) {
+                                    v[d] = (float)acc[i][j][x + d] * tok[xr + d] * chs[j];
+                                } else {
+                                    v[d] = (float)acc[i][j][x + d];
                                 }
-                                // hardware RNE to bf16, both rows in one dword; then the neighbour's dword
-                                // and one byte permute: even lanes keep the low halves (row x), odd lanes
-                                // the high halves (row x+1), own column in its place
-                                const uint32_t pk_bf = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){v[0], v[1]}, bf16x2));
-                                const uint32_t pk_h = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){v[0], v[1]}, f16x2));
-                                const uint32_t pk = p.out_fp16 ? pk_h : pk_bf;   // wave-uniform choice of the output type
-                                const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, true);
-                                const uint32_t packed = __builtin_amdgcn_perm(nb, pk, odd ? 0x03020706u : 0x05040100u);
-                                const int lrow = qq * 8 + g * 4 + xr + (odd ? 1 : 0);
-                                const int lcol = j * 32 + (r & ~1);
-                                *reinterpret_cast<uint32_t *>(smem + epi + (uint32_t)(lrow * ROWB + lcol * 2)) = packed;
                             }
-                    }
-                    const int lrow = lane_e / CPR, chunk = lane_e % CPR;
-                    const v4i val = lds_read16(epi + (uint32_t)(lrow * ROWB + chunk * 16));
-                    const int row = wm * WM + i * 32 + ps * PASS_ROWS + lrow;  // relative to m0
-                    const int col = cur.j0 + wn * WN_OUT + chunk * 8;
-                    bool ok = (cur.m0 + row < cur.m_end) && (col + 8 <= p.n_out);
-                    uint32_t out_row = (uint32_t)row;
-                    if constexpr (EPI == EPI_PLAIN) {
-                        const int mapped = (int)lds_read4(prm + (uint32_t)row * 4u);
-                        ok = ok && (!has_map || (mapped >= 0 && mapped < (int)p.out_rows));   // dropped or out of range: not written
-                        out_row = has_map ? (uint32_t)mapped : out_row;
-                    }
-                    if constexpr (SWIGLU) {
-                        if (mx_out) {
-                            // The four lanes of a quad hold the 32 columns of one row that this wave owns:
-                            // one MX block.  Its maximum, shared exponent and codes as the row quantiser
-                            // makes them from the bf16 values.
-                            const uint32_t w[4] = {(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]};
-                            const uint32_t amax = block_amax_bits(w);
-                            uint32_t code[2], sbyte;
-                            int e;
-                            bool is_nan;
-                            if (p.mx_out_fmt == CCH_FMT_E2M1) {
-                                sbyte = shared_exp_byte<CCH_FMT_E2M1>(amax, e, is_nan);
-                                quant8_hw<CCH_FMT_E2M1>(w, e, is_nan, code);
-                            } else if (p.mx_out_fmt == CCH_FMT_E5M2) {
-                                sbyte = shared_exp_byte<CCH_FMT_E5M2>(amax, e, is_nan);
-                                quant8_hw<CCH_FMT_E5M2>(w, e, is_nan, code);
-                            } else {
-                                sbyte = shared_exp_byte<CCH_FMT_E4M3>(amax, e, is_nan);
-                                quant8_hw<CCH_FMT_E4M3>(w, e, is_nan, code);
-                            }
-                            const uint32_t elem = out_row * (uint32_t)p.n_out + (uint32_t)col;
-                            if (p.mx_out_fmt == CCH_FMT_E2M1)
-                                __builtin_amdgcn_raw_buffer_store_b32(code[0], rs_out, (int)(ok ? elem >> 1 : NO_FETCH), 0, 0);
-                            else
-                                __builtin_amdgcn_raw_buffer_store_b64((v2u){code[0], code[1]}, rs_out, (int)(ok ? elem : NO_FETCH), 0, 0);
-                            // the quad's first lane writes the block's scale, and behind the last block of a row
-                            // with an odd count of blocks the padding byte
-                            const __amdgpu_buffer_rsrc_t rs_sc_out = __builtin_amdgcn_make_buffer_rsrc(
-                                p.out_scales + (size_t)cur.m0 * p.mx_out_sld, 0, 0x7FFFFFFF, 0x00020000);
-                            const uint32_t blk = (uint32_t)col >> 5, soff = out_row * (uint32_t)p.mx_out_sld + blk;
-                            const bool first = ok && chunk == 0;
-                            __builtin_amdgcn_raw_buffer_store_b8((uint8_t)sbyte, rs_sc_out, (int)(first ? soff : NO_FETCH), 0, 0);
-                            if ((p.n_out & 32) != 0 && (int)blk == (p.n_out >> 5) - 1)
-                                __builtin_amdgcn_raw_buffer_store_b8((uint8_t)127, rs_sc_out, (int)(first ? soff + 1 : NO_FETCH), 0, 0);
-                            continue;
+                            // hardware RNE to bf16, both rows in one dword; then the neighbour's dword
+                            // and one byte permute: even lanes keep the low halves (row x), odd lanes
+                            // the high halves (row x+1), own column in its place
+                            uint32_t pk;
+                            if constexpr (decltype(fp16_c)::value) pk = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){v[0], v[1]}, f16x2));
+                            else pk = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){v[0], v[1]}, bf16x2));
+                            const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, true);
+                            const uint32_t packed = __builtin_amdgcn_perm(nb, pk, odd ? 0x03020706u : 0x05040100u);
+                            const int lrow = qq * 8 + g * 4 + xr + (odd ? 1 : 0);
+                            const int lcol = j * 32 + (r & ~1);
+                            *reinterpret_cast<uint32_t *>(smem + epi + (uint32_t)(lrow * ROWB + lcol * 2)) = packed;
                         }
-                    }
-                    const uint32_t off = ok ? (out_row * (uint32_t)p.n_out + (uint32_t)col) * 2u : NO_FETCH;
-                    const v4u sv = (v4u){(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]};
-                    if (p.nt_out) __builtin_amdgcn_raw_buffer_store_b128(sv, rs_out, (int)off, 0, 2);   // non-temporal
-                    else __builtin_amdgcn_raw_buffer_store_b128(sv, rs_out, (int)off, 0, 0);
                 }
-            }
+            };
+            struct PassData {
+                v4i val;
+                int mapped;
+            };
+            auto readback = [&](auto i_c, auto ps_c) {
+                constexpr int i = decltype(i_c)::value, ps = decltype(ps_c)::value;
+                PassData d;
+                const int lrow = lane_e / CPR, chunk = lane_e % CPR;
+                d.val = lds_read16(epi + (uint32_t)(lrow * ROWB + chunk * 16));
+                d.mapped = 0;
+                if constexpr (EPI == EPI_PLAIN) d.mapped = (int)lds_read4(prm + (uint32_t)(wm * WM + i * 32 + ps * PASS_ROWS + lrow) * 4u);
+                return d;
+            };
+            auto emit = [&](auto i_c, auto ps_c, const PassData &d) {
+                constexpr int i = decltype(i_c)::value, ps = decltype(ps_c)::value;
+                const v4i val = d.val;
+                const int lrow = lane_e / CPR, chunk = lane_e % CPR;
+                const int row = wm * WM + i * 32 + ps * PASS_ROWS + lrow;  // relative to m0
+                const int col = cur.j0 + wn * WN_OUT + chunk * 8;
+                bool ok = (cur.m0 + row < cur.m_end) & (col + 8 <= p.n_out);
+                uint32_t out_row = (uint32_t)row;
+                if constexpr (EPI == EPI_PLAIN) {
+                    // dropped or out of range: not written (without a map the destination is the row itself)
+                    ok = ok & (!has_map | ((d.mapped >= 0) & (d.mapped < (int)p.out_rows)));
+                    out_row = has_map ? (uint32_t)d.mapped : out_row;
+                }
+                if constexpr (SWIGLU) {
+                    if (mx_out) {
+                        // The four lanes of a quad hold the 32 columns of one row that this wave owns:
+                        // one MX block.  Its maximum, shared exponent and codes as the row quantiser
+                        // makes them from the bf16 values.
+                        const uint32_t w[4] = {(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]};
+                        const uint32_t amax = block_amax_bits(w);
+                        uint32_t code[2], sbyte;
+                        int e;
+                        bool is_nan;
+                        if (p.mx_out_fmt == CCH_FMT_E2M1) {
+                            sbyte = shared_exp_byte<CCH_FMT_E2M1>(amax, e, is_nan);
+                            quant8_hw<CCH_FMT_E2M1>(w, e, is_nan, code);
+                        } else if (p.mx_out_fmt == CCH_FMT_E5M2) {
+                            sbyte = shared_exp_byte<CCH_FMT_E5M2>(amax, e, is_nan);
+                            quant8_hw<CCH_FMT_E5M2>(w, e, is_nan, code);
+                        } else {
+                            sbyte = shared_exp_byte<CCH_FMT_E4M3>(amax, e, is_nan);
+                            quant8_hw<CCH_FMT_E4M3>(w, e, is_nan, code);
+                        }
+                        const uint32_t elem = out_row * (uint32_t)p.n_out + (uint32_t)col;
+                        if (p.mx_out_fmt == CCH_FMT_E2M1)
+                            __builtin_amdgcn_raw_buffer_store_b32(code[0], rs_out, (int)(ok ? elem >> 1 : NO_FETCH), 0, 0);
+                        else
+                            __builtin_amdgcn_raw_buffer_store_b64((v2u){code[0], code[1]}, rs_out, (int)(ok ? elem : NO_FETCH), 0, 0);
+                        // the quad's first lane writes the block's scale, and behind the last block of a row
+                        // with an odd count of blocks the padding byte
+                        const __amdgpu_buffer_rsrc_t rs_sc_out = __builtin_amdgcn_make_buffer_rsrc(
+                            p.out_scales + (size_t)cur.m0 * p.mx_out_sld, 0, 0x7FFFFFFF, 0x00020000);
+                        const uint32_t blk = (uint32_t)col >> 5, soff = out_row * (uint32_t)p.mx_out_sld + blk;
+                        const bool first = ok && chunk == 0;
+                        __builtin_amdgcn_raw_buffer_store_b8((uint8_t)sbyte, rs_sc_out, (int)(first ? soff : NO_FETCH), 0, 0);
+                        if ((p.n_out & 32) != 0 && (int)blk == (p.n_out >> 5) - 1)
+                            __builtin_amdgcn_raw_buffer_store_b8((uint8_t)127, rs_sc_out, (int)(first ? soff + 1 : NO_FETCH), 0, 0);
+                        return;
+                    }
+                }
+                const uint32_t off = ok ? (out_row * (uint32_t)p.n_out + (uint32_t)col) * 2u : NO_FETCH;
+                const v4u sv = (v4u){(uint32_t)val[0], (uint32_t)val[1], (uint32_t)val[2], (uint32_t)val[3]};
+                if (p.nt_out) __builtin_amdgcn_raw_buffer_store_b128(sv, rs_out, (int)off, 0, 2);   // non-temporal
+                else __builtin_amdgcn_raw_buffer_store_b128(sv, rs_out, (int)off, 0, 0);
+            };
+            constexpr int NP = MT * NPASS;
+            auto all_passes = [&](auto fp16_c) {
+                produce(IC<0>{}, IC<0>{}, fp16_c);
+                PassData pending = readback(IC<0>{}, IC<0>{});
+                static_for<NP - 1>([&](auto n_c) {
+                    constexpr int n = decltype(n_c)::value + 1;
+                    produce(IC<n / NPASS>{}, IC<n % NPASS>{}, fp16_c);
+                    __builtin_amdgcn_sched_barrier(0);   // the store's address arithmetic waits for the read: keep it behind the conversions
+                    emit(IC<(n - 1) / NPASS>{}, IC<(n - 1) % NPASS>{}, pending);
+                    pending = readback(IC<n / NPASS>{}, IC<n % NPASS>{});
+                });
+                emit(IC<(NP - 1) / NPASS>{}, IC<(NP - 1) % NPASS>{}, pending);
+            };
+            // the output type is a wave-uniform choice: one copy of the passes for each (the MX-quantised activation is
+            // made from bf16 values)
+            if (p.out_fp16) all_passes(IC<1>{});
+            else all_passes(IC<0>{});
         }
         if (wm == 1) CCH_BARRIER();
         cur = nxt;
