@@ -10,6 +10,7 @@ int launch_gemm_naive(const GemmProblem &p, int kind, int epi, hipStream_t strea
 int launch_gemm_tile(const GemmProblem &p, int kind, int epi, hipStream_t stream);
 const char *gemm_tile_unsupported(const GemmProblem &p, int kind, int epi);
 bool quant_set_option(const char *name, int value);   // mx_quant.hip
+extern std::atomic<int> g_route_three_launches;        // routing.hip
 
 static std::atomic<int> g_force_generic{0};
 static std::atomic<int> g_require_tiled{0};
@@ -77,6 +78,10 @@ int cch_set_option(const char *name, int value)
     }
     if (strcmp(name, "gemm_tile_order") == 0) {
         g_tile_order.store(value);
+        return CCH_OK;
+    }
+    if (strcmp(name, "routing_three_launches") == 0) {
+        g_route_three_launches.store(value);
         return CCH_OK;
     }
     if (quant_set_option(name, value)) return CCH_OK;

@@ -17,6 +17,8 @@ namespace cch {
 
 constexpr int ROUTE_CHUNK = 1024;       // rows per workgroup
 constexpr int ROUTE_MAX_EXPERTS = 1024;
+// cch_set_option("routing_three_launches", 1): the general path also where one workgroup would do (for tests)
+std::atomic<int> g_route_three_launches{0};
 
 // hist[e * nchunks + c] = rows of chunk c routed to expert e; dst_to_src of the chunk's positions
 // is preset to -1 (positions past the routed rows keep it).
@@ -157,6 +159,82 @@ __global__ __launch_bounds__(64 * ROUTE_WAVES) void route_place_kernel(const int
     }
 }
 
+// Few rows and experts (a decode step's routes): the whole sort in one workgroup and one launch.  Sixteen waves
+// walk their sixteenths of the rows in order, 64 at a time, exactly like the waves of the placement pass above;
+// the per-wave counts per expert meet in LDS, thread e scans expert e's counts over the waves, the experts'
+// totals are scanned across the workgroup, and a second walk over the rows (keys and lane sets kept in registers)
+// hands the positions out.  No workspace.
+constexpr int ONE_WAVES = 16, ONE_MAX_GROUPS = 8, ONE_MAX_EXPERTS = 256;
+constexpr int ONE_MAX_ROWS = ONE_WAVES * ONE_MAX_GROUPS * 64;   // 8192
+__global__ __launch_bounds__(64 * ONE_WAVES) void route_one_workgroup_kernel(const int32_t *__restrict__ expert_idx, int rows, int experts,
+                                                                            int bits, int groups, int32_t *__restrict__ dst_to_src,
+                                                                            int32_t *__restrict__ src_to_dst,
+                                                                            int32_t *__restrict__ expert_tokens, int cumsum)
+{
+    __shared__ int32_t cnt[ONE_WAVES][ONE_MAX_EXPERTS];
+    __shared__ int32_t part[ONE_MAX_EXPERTS];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    for (int e = threadIdx.x; e < ONE_WAVES * ONE_MAX_EXPERTS; e += 64 * ONE_WAVES) (&cnt[0][0])[e] = 0;
+    __syncthreads();
+    const int base = w * groups * 64;   // `groups` groups of 64 rows per wave
+    const uint64_t below = (1ull << lane) - 1ull;
+    int key[ONE_MAX_GROUPS];
+    uint64_t same[ONE_MAX_GROUPS];
+#pragma unroll
+    for (int g = 0; g < ONE_MAX_GROUPS; g++) {
+        key[g] = -1;
+        same[g] = 0;
+        if (g < groups) {
+            const int r = base + g * 64 + lane;
+            const int e = r < rows ? expert_idx[r] : -1;
+            const bool routed = e >= 0 && e < experts;
+            key[g] = routed ? e : -1;
+            same[g] = same_key_lanes(e, routed, bits);
+            if (routed && (same[g] & below) == 0) cnt[w][e] += __popcll(same[g]);   // first lane of its key
+        }
+    }
+    __syncthreads();
+    // thread e: expert e's counts over the waves -> exclusive running sums, total into part[e]
+    int total = 0;
+    if ((int)threadIdx.x < ONE_MAX_EXPERTS) {
+        const int e = threadIdx.x;
+#pragma unroll
+        for (int v = 0; v < ONE_WAVES; v++) {
+            const int c = cnt[v][e];
+            cnt[v][e] = total;
+            total += c;
+        }
+        part[e] = total;
+    }
+    __syncthreads();
+    // inclusive scan of the experts' totals (Hillis-Steele over 256 entries)
+    for (int off = 1; off < ONE_MAX_EXPERTS; off <<= 1) {
+        int add = 0;
+        if ((int)threadIdx.x < ONE_MAX_EXPERTS && (int)threadIdx.x >= off) add = part[threadIdx.x - off];
+        __syncthreads();
+        if ((int)threadIdx.x < ONE_MAX_EXPERTS) part[threadIdx.x] += add;
+        __syncthreads();
+    }
+    if ((int)threadIdx.x < experts) expert_tokens[threadIdx.x] = cumsum ? part[threadIdx.x] : total;
+    const int routed_rows = part[ONE_MAX_EXPERTS - 1];
+    // sorted positions past the routed rows hold no row
+    for (int i = routed_rows + (int)threadIdx.x; i < rows; i += 64 * ONE_WAVES) dst_to_src[i] = -1;
+#pragma unroll
+    for (int g = 0; g < ONE_MAX_GROUPS; g++) {
+        if (g < groups) {
+            const int r = base + g * 64 + lane;
+            const bool routed = key[g] >= 0;
+            int pos = -1;
+            if (routed) pos = (key[g] > 0 ? part[key[g] - 1] : 0) + cnt[w][key[g]] + __popcll(same[g] & below);
+            if (routed && (same[g] & below) == 0) cnt[w][key[g]] += __popcll(same[g]);
+            if (r < rows) {
+                src_to_dst[r] = pos;
+                if (pos >= 0) dst_to_src[pos] = r;
+            }
+        }
+    }
+}
+
 // Checks shared by the two entry points; fills nchunks.
 static int route_check(const char *who, const int32_t *expert_idx, int64_t rows, int num_experts, const int32_t *dst_to_src,
                        const int32_t *src_to_dst, const int32_t *expert_tokens, int64_t *nchunks)
@@ -173,9 +251,19 @@ static int route_check(const char *who, const int32_t *expert_idx, int64_t rows,
 
 // The three launches; hist holds nchunks * num_experts entries, every one of which the histogram
 // pass writes before the scan reads it (nothing has to start at zero).
+static bool route_fits_one_workgroup(int64_t rows, int num_experts) { return rows > 0 && rows <= ONE_MAX_ROWS && num_experts <= ONE_MAX_EXPERTS; }
+
 static int route_launch(const int32_t *expert_idx, int64_t rows, int num_experts, int64_t nchunks, int32_t *dst_to_src,
                         int32_t *src_to_dst, int32_t *expert_tokens, int cumsum, int32_t *hist, hipStream_t s)
 {
+    if (route_fits_one_workgroup(rows, num_experts) && !g_route_three_launches.load(std::memory_order_relaxed)) {
+        int bits = 0;
+        while ((1 << bits) < num_experts) bits++;
+        const int groups = (int)((rows + 64 * ONE_WAVES - 1) / (64 * ONE_WAVES));
+        hipLaunchKernelGGL(route_one_workgroup_kernel, dim3(1), dim3(64 * ONE_WAVES), 0, s, expert_idx, (int)rows, num_experts, bits, groups,
+                           dst_to_src, src_to_dst, expert_tokens, cumsum);
+        return launch_status("route kernel");
+    }
     hipLaunchKernelGGL(route_histogram_kernel, dim3((unsigned)nchunks), dim3(256), 0, s, expert_idx, (int)rows, num_experts,
                        (int)nchunks, hist, dst_to_src);
     hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, hist, num_experts, (int)nchunks, expert_tokens, cumsum);

@@ -281,7 +281,8 @@ int cch_moe_token_unpermute(const void *permuted_tokens, const int32_t *sorted_i
  *                  operator returns
  *   expert_tokens  int32 [num_experts]: entries per expert, or their running sum with cumsum != 0
  *   workspace      device memory of at least cch_moe_init_routing_workspace_bytes(rows, num_experts)
- * num_experts <= 1024. */
+ * num_experts <= 1024.  Up to 8192 rows and 256 experts the sort is one launch of one workgroup (the
+ * workspace is then not touched), three launches otherwise; the results are the same integers. */
 int64_t cch_moe_init_routing_workspace_bytes(int64_t rows, int num_experts);
 int cch_moe_init_routing(const int32_t *expert_idx, int64_t rows, int num_experts, int32_t *dst_to_src, int32_t *src_to_dst,
                          int32_t *expert_tokens, int cumsum, void *workspace, int64_t workspace_bytes, void *stream);

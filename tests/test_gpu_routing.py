@@ -28,6 +28,29 @@ def test_routing_exact(case, cumsum):
     assert np.array_equal(d2s.cpu().numpy(), wd)
 
 
+@pytest.mark.parametrize("case", [(1, 1), (63, 3), (64, 256), (1000, 16), (4097, 200), (8192, 256), (8192, 1), (8193, 256), (500, 257)])
+def test_routing_one_workgroup_equals_three_launches(case):
+    """Up to 8192 rows and 256 experts one workgroup does the whole sort in one launch; the general path (three launches,
+    `routing_three_launches`) and the oracle give the same integers, also just past either limit and with dropped routes."""
+    rows, e = case
+    rng = np.random.default_rng(rows * 7 + e)
+    idx = rng.integers(-1, e + 1, rows).astype(np.int32)      # -1 and e are dropped
+    want = orc.moe_init_routing(idx, e)
+    for cumsum in (False, True):
+        res = []
+        for three in (0, 1):
+            cc.set_option("routing_three_launches", three)
+            try:
+                res.append([t.cpu().numpy() for t in cc.moe_init_routing(torch.from_numpy(idx).cuda(), e, cumsum)])
+            finally:
+                cc.set_option("routing_three_launches", 0)
+        for a, b in zip(*res):
+            assert np.array_equal(a, b)
+        if not cumsum:
+            for a, w in zip(res[0], want):
+                assert np.array_equal(a, w)
+
+
 def test_routing_skewed_and_sorted_inputs():
     for idx in (np.zeros(5000, np.int32), np.arange(5000, dtype=np.int32) % 7, np.sort(np.arange(5000, dtype=np.int32) % 7)[::-1].copy()):
         d2s, s2d, cnt = cc.moe_init_routing(torch.from_numpy(idx).cuda(), 7)
