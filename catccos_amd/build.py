@@ -8,6 +8,7 @@ Outputs (git-ignored, shipped as built files):
     catccos_amd/libcatccos_hip.so      C ABI + HIP kernels   (include/catccos_hip.h)
     catccos_amd/libcatccos_host.so     C++ operator surface  (catccos_amd/csrc/host/)
     catccos_amd/catccos_run            command-line driver over the operator surface
+    catccos_amd/libcatccos_torch.so    torch.ops.catccos.* (C++ TORCH_LIBRARY, catccos_amd/csrc/torch/)
 """
 import argparse
 import concurrent.futures
@@ -23,6 +24,7 @@ OBJ = os.path.join(PKG, "build")
 LIB = os.path.join(PKG, "libcatccos_hip.so")
 HOST_LIB = os.path.join(PKG, "libcatccos_host.so")
 DRIVER = os.path.join(PKG, "catccos_run")
+TORCH_LIB = os.path.join(PKG, "libcatccos_torch.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
@@ -81,14 +83,32 @@ def build_host():
     return HOST_LIB
 
 
+def build_torch():
+    """torch.ops.catccos.* as a C++ TORCH_LIBRARY (catccos_amd/csrc/torch/torch_bindings.cpp): host code only, against
+    this interpreter's PyTorch and the HIP library above."""
+    import torch
+    from torch.utils import cpp_extension as ce
+    src = os.path.join(CSRC, "torch", "torch_bindings.cpp")
+    tlib = ce.library_paths()[0]
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+           # the platform macro the HIP runtime headers ask for, and PyTorch's switch for its ROCm headers
+           "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-I" + os.path.join(ROOT, "include"), "-I/opt/rocm/include"] + ["-isystem" + d for d in ce.include_paths()] + [
+           src, "-o", TORCH_LIB, "-L" + tlib, "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip", "-L" + PKG, "-lcatccos_hip",
+           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + tlib]
+    _run(cmd)
+    return TORCH_LIB
+
+
 def build_all(jobs=8):
     build_lib(jobs)
     build_host()
+    build_torch()
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", choices=["lib", "host"])
+    ap.add_argument("--only", choices=["lib", "host", "torch"])
     ap.add_argument("-j", type=int, default=8)
     ap.add_argument("--define", action="append", default=[], metavar="NAME", help="extra -D for the HIP sources (needs --out)")
     ap.add_argument("--out", metavar="DIR", help="directory for a library built with --define")
@@ -97,3 +117,5 @@ if __name__ == "__main__":
         print(build_lib(a.j, a.define, a.out))
     if a.only in (None, "host"):
         print(build_host())
+    if a.only in (None, "torch"):
+        print(build_torch())

@@ -22,127 +22,20 @@ empty tensors of the result shape.  There is no communication here, so `init` ac
 `rank_size == 1` only and makes no use of `local_mem_size` / `ip_port` (the symmetric heap they size is the
 part that was dropped).
 
-Importing this module registers the library; `import catccos_amd` does not import it.
+The operators are a C++ `TORCH_LIBRARY` (catccos_amd/csrc/torch/torch_bindings.cpp, built by
+`python -m catccos_amd.build` into catccos_amd/libcatccos_torch.so): C++ programs linking libtorch load that
+library directly; importing this module loads it into the Python process (`import catccos_amd` does not).
+Also there: `mx_grouped_matmul_swiglu_mx`, `gmm_dequant_swiglu_mx` (up projections with MX-quantised output) and
+`moe_ffn_mxfp8` (the MXFP8 MoE FFN of one rank, routing to combine).
 """
+import os
+
 import torch
 
-from . import ops
-from ._abi import FMT_E1M2, FMT_E2M1
+from . import _abi
 
-_state = {"initialized": False, "rank_id": -1, "rank_size": 0}
-
-_lib = torch.library.Library("catccos", "DEF")
-_lib.define("init(int rank_id, int rank_size, int local_mem_size, str ip_port) -> int")
-_lib.define("finalize() -> int")
-_lib.define("mx_quant(Tensor x, str fmt, int rounding) -> (Tensor, Tensor)")
-_lib.define("w8a8_matmul_dequant(Tensor a, Tensor b, Tensor per_tok, Tensor per_ch, int trans_b) -> Tensor")
-_lib.define("mx_matmul(Tensor a, Tensor sa, Tensor b, Tensor sb, str fmt, int trans_b) -> Tensor")
-_lib.define("gmm_dequant_swiglu(Tensor x, Tensor w, Tensor group_sizes, Tensor per_tok, Tensor per_ch, int trans_b) -> Tensor")
-_lib.define("mx_grouped_matmul(Tensor a, Tensor sa, Tensor b, Tensor sb, Tensor group_sizes, str fmt, int trans_b) -> Tensor")
-_lib.define("mx_grouped_matmul_swiglu_mx(Tensor a, Tensor sa, Tensor b, Tensor sb, Tensor group_sizes, str fmt, int trans_b, str out_fmt) -> (Tensor, Tensor)")
-_lib.define("gmm_dequant_swiglu_mx(Tensor x, Tensor w, Tensor group_sizes, Tensor per_tok, Tensor per_ch, int trans_b, str fmt) -> (Tensor, Tensor)")
-_lib.define("moe_ffn_mxfp8(Tensor x, Tensor expert_idx, Tensor probs, Tensor w1, Tensor sw1, Tensor w2, Tensor sw2, int trans_b) -> Tensor")
-
-
-def _init(rank_id, rank_size, local_mem_size, ip_port):
-    if _state["initialized"]:
-        return 0   # torch_bindings.cpp:88-90: a second init is a no-op
-    # the reference's argument checks and messages (torch_bindings.cpp:92-95)
-    torch._check(rank_id >= 0, lambda: "invalid rank_id: %d" % rank_id)
-    torch._check(rank_size > 0, lambda: "invalid rank_size: %d" % rank_size)
-    torch._check(local_mem_size > 0, lambda: "invalid local_mem_size: %d" % local_mem_size)
-    torch._check(len(ip_port) > 0, lambda: "ip_port is empty")
-    torch._check(rank_size == 1 and rank_id == 0,
-                 lambda: "catccos on one GPU has no peers: rank_size must be 1 and rank_id 0, got %d of %d" % (rank_id, rank_size))
-    _state.update(initialized=True, rank_id=rank_id, rank_size=rank_size)
-    return 0
-
-
-def _finalize():
-    if not _state["initialized"]:
-        return 0
-    if torch.cuda.is_available() and torch.cuda.is_initialized():
-        torch.cuda.current_stream().synchronize()   # the reference drains the stream before it lets go of its buffers
-    _state.update(initialized=False, rank_id=-1, rank_size=0)
-    return 0
-
-
-def _need_init():
-    torch._check(_state["initialized"], lambda: "catccos TORCH_LIBRARY not initialized, call torch.ops.catccos.init(...) first")
-
-
-def _guarded(fn):
-    def run(*args):
-        _need_init()
-        with torch.cuda.device(args[0].device):
-            return fn(*args)
-    return run
-
-
-# init / finalize take no tensors: one kernel for every backend, as in the reference
-_lib.impl("init", _init, "CompositeExplicitAutograd")
-_lib.impl("finalize", _finalize, "CompositeExplicitAutograd")
-_lib.impl("mx_quant", _guarded(ops.mx_quant), "CUDA")
-_lib.impl("w8a8_matmul_dequant", _guarded(ops.w8a8_matmul_dequant), "CUDA")
-_lib.impl("mx_matmul", _guarded(ops.mx_matmul), "CUDA")
-_lib.impl("gmm_dequant_swiglu", _guarded(ops.gmm_dequant_swiglu), "CUDA")
-_lib.impl("mx_grouped_matmul", _guarded(ops.mx_grouped_matmul), "CUDA")
-_lib.impl("gmm_dequant_swiglu_mx", _guarded(ops.gmm_dequant_swiglu_mx), "CUDA")
-_lib.impl("moe_ffn_mxfp8", _guarded(ops.moe_ffn_mxfp8), "CUDA")
-_lib.impl("mx_grouped_matmul_swiglu_mx", _guarded(lambda a, sa, b, sb, gs, fmt, tb, ofmt: ops.mx_grouped_matmul_swiglu(a, sa, b, sb, gs, fmt, tb, out_fmt=ofmt)),
-          "CUDA")
-
-
-# ---- Meta kernels: output shapes only (symbolic sizes pass through the arithmetic untouched)
-
-def _fp4(fmt):
-    return ops._fmt(fmt) in (FMT_E2M1, FMT_E1M2)
-
-
-def _mx_quant_meta(x, fmt, rounding):
-    m, k = x.shape
-    payload = x.new_empty((m, (k + 1) // 2 if _fp4(fmt) else k), dtype=torch.uint8)
-    return payload, x.new_empty((m, 2 * ((k + 63) // 64)), dtype=torch.uint8)
-
-
-def _w8a8_meta(a, b, per_tok, per_ch, trans_b):
-    return a.new_empty((a.shape[0], b.shape[0] if trans_b else b.shape[1]), dtype=torch.bfloat16)
-
-
-def _mx_n(b_shape, fmt, trans_b):
-    return b_shape[0] if trans_b else b_shape[1] * (2 if _fp4(fmt) else 1)
-
-
-def _mx_matmul_meta(a, sa, b, sb, fmt, trans_b):
-    return a.new_empty((a.shape[0], _mx_n(b.shape, fmt, trans_b)), dtype=torch.bfloat16)
-
-
-def _gmm_swiglu_meta(x, w, group_sizes, per_tok, per_ch, trans_b):
-    n = w.shape[1] if trans_b else w.shape[2]
-    return x.new_empty((x.shape[0], n // 2), dtype=torch.bfloat16)
-
-
-def _gmm_swiglu_mx_meta(x, w, group_sizes, per_tok, per_ch, trans_b, fmt):
-    h = (w.shape[1] if trans_b else w.shape[2]) // 2
-    payload = x.new_empty((x.shape[0], h // 2 if _fp4(fmt) else h), dtype=torch.uint8)
-    return payload, x.new_empty((x.shape[0], 2 * ((h + 63) // 64)), dtype=torch.uint8)
-
-
-def _mx_gmm_swiglu_mx_meta(a, sa, b, sb, group_sizes, fmt, trans_b, out_fmt):
-    h = _mx_n(b.shape[1:], fmt, trans_b) // 2
-    payload = a.new_empty((a.shape[0], h // 2 if _fp4(out_fmt) else h), dtype=torch.uint8)
-    return payload, a.new_empty((a.shape[0], 2 * ((h + 63) // 64)), dtype=torch.uint8)
-
-
-def _mx_gmm_meta(a, sa, b, sb, group_sizes, fmt, trans_b):
-    return a.new_empty((a.shape[0], _mx_n(b.shape[1:], fmt, trans_b)), dtype=torch.bfloat16)
-
-
-_lib.impl("moe_ffn_mxfp8", lambda x, expert_idx, probs, w1, sw1, w2, sw2, trans_b: x.new_empty(x.shape), "Meta")
-_lib.impl("mx_quant", _mx_quant_meta, "Meta")
-_lib.impl("w8a8_matmul_dequant", _w8a8_meta, "Meta")
-_lib.impl("mx_matmul", _mx_matmul_meta, "Meta")
-_lib.impl("gmm_dequant_swiglu", _gmm_swiglu_meta, "Meta")
-_lib.impl("mx_grouped_matmul", _mx_gmm_meta, "Meta")
-_lib.impl("gmm_dequant_swiglu_mx", _gmm_swiglu_mx_meta, "Meta")
-_lib.impl("mx_grouped_matmul_swiglu_mx", _mx_gmm_swiglu_mx_meta, "Meta")
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libcatccos_torch.so")
+if not os.path.exists(LIB_PATH):
+    raise ImportError("%s is missing: build it with `python -m catccos_amd.build`" % LIB_PATH)
+_abi.lib()                       # the HIP library first: a missing or unloadable one is reported by name
+torch.ops.load_library(LIB_PATH)

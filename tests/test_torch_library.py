@@ -4,7 +4,7 @@ torch_bindings_meta.cpp:18-35).  No GPU needed: Meta tensors carry shapes only."
 import pytest
 import torch
 
-import catccos_amd.torch_library  # noqa: F401  (registers the library)
+import catccos_amd.torch_library  # (loads the library)
 
 OPS = torch.ops.catccos
 
@@ -14,6 +14,18 @@ def initialised():
     assert OPS.init(0, 1, 1 << 20, "tcp://127.0.0.1:8666") == 0
     yield
     assert OPS.finalize() == 0
+
+
+def test_operators_come_from_the_cpp_library():
+    """The operators are a C++ TORCH_LIBRARY translation unit (catccos_amd/csrc/torch/torch_bindings.cpp), as the reference's
+    are (examples/torch_binding/src/torch_bindings.cpp:232-239): the Python module only loads the built library."""
+    import os
+    path = catccos_amd.torch_library.LIB_PATH
+    assert os.path.basename(path) == "libcatccos_torch.so" and os.path.exists(path)
+    assert any(os.path.samefile(path, p) for p in torch.ops.loaded_libraries)
+    assert torch._C._dispatch_has_kernel_for_dispatch_key("catccos::mx_quant", "CUDA")
+    assert torch._C._dispatch_has_kernel_for_dispatch_key("catccos::mx_quant", "Meta")
+    assert not torch._C._dispatch_has_kernel_for_dispatch_key("catccos::mx_quant", "CPU")
 
 
 def test_schemas_are_registered():
