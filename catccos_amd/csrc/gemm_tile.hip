@@ -296,7 +296,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     constexpr bool KSPLIT = TB ? (CCH_KSPLIT_TB1 != 0) : (CCH_KSPLIT_TB0 != 0);
 
     __shared__ GroupTable tab;
-    if (threadIdx.x == 0) build_group_table(tab, p.group_sizes, p.num_groups, p.T, BM);
+    if (threadIdx.x < 64) build_group_table_wave(tab, p.group_sizes, p.num_groups, p.T, BM);
     __syncthreads();
 
     const int lane = threadIdx.x & 63;
