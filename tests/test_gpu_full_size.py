@@ -134,3 +134,9 @@ def test_cfg5_mx_grouped_16384_tokens_32_experts(fmt, ofmt):
             assert torch.equal(one, out[r0:r0 + sz]), g
         r0 += sz
     assert r0 == t
+    # the result does not depend on the launch: forty more, queued back to back (as the bench queues them), equal the first to
+    # the bit - a stage of the ring read too early or a request counted wrongly would show as a launch that differs
+    same = torch.ones((), dtype=torch.bool, device="cuda")
+    for _ in range(40):
+        same &= torch.equal(cc.mx_grouped_matmul(a, sa, b, sb, gs, fmt, 0), out)
+    assert bool(same)
