@@ -595,3 +595,34 @@ def test_fp16_output_of_the_int8_and_dense_mx_operators(tiled):
     finally:
         cc.set_option("require_tiled_gemm", 0)
         cc.set_option("force_generic_gemm", 0)
+
+
+@pytest.mark.parametrize("sizes,t", [([-5, 300, -1, 2 ** 30, 7], 500), ([2 ** 31 - 1, 2 ** 31 - 1, 5], 300), ([0, 0, 0], 64), ([100] * 200, 9000)],
+                         ids=["negative-and-huge", "sum-overflows-int32", "all-empty", "200-groups-run-out-of-rows"])
+def test_group_sizes_are_clipped_the_same_way_on_both_paths(sizes, t):
+    """Group sizes below zero count as empty and the groups stop where the rows do (the reference's golden pads the
+    remainder with zeros, examples/utils/gen_data_fp4_mx_alltoallv_gmm.py:788-790): the tiled kernels (table built by
+    one wave with two scans) and the generic ones (one thread's running sum) agree to the bit on which rows belong
+    to which expert, and with the oracle fed the clipped sizes."""
+    rng = np.random.default_rng(len(sizes) + t)
+    e, k, n = len(sizes), 256, 256
+    gs_h = np.array(sizes, dtype=np.int64).astype(np.int32)
+    clipped, row = [], 0
+    for s in gs_h.tolist():
+        c = max(0, min(int(s), t - row))
+        clipped.append(c)
+        row += c
+    x = rng.integers(-127, 128, (t, k)).astype(np.int8)
+    w = rng.integers(-3, 4, (e, k, n)).astype(np.int8)
+    pt = rng.uniform(0.001, 0.02, t).astype(np.float32)
+    pc = rng.uniform(0.001, 0.02, (e, n)).astype(np.float32)
+    a, b = _both_paths(lambda: cc.gmm_dequant(dev(x), dev(w), dev(gs_h), dev(pt), dev(pc), 0))
+    assert np.array_equal(a, b)            # exact int32 sums, the same two fp32 products and one rounding on either path
+    want = np.zeros((t, n), np.float32)
+    r0 = 0
+    for g, c in enumerate(clipped):
+        if c:
+            want[r0:r0 + c] = orc.gemm_i8_dequant(x[r0:r0 + c], w[g], pt[r0:r0 + c], pc[g])
+        r0 += c
+    assert_close(a, want)
+    assert (a[r0:] == 0).all()
