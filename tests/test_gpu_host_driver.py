@@ -249,3 +249,18 @@ def test_dispatch_ffn_combine_reference_shape_list_perf_mode(tmp_path):
     assert r.returncode == 0 and r.stdout.count("[PERF] Avg latency") == 4 and "4 shapes finished" in r.stdout, r.stdout + r.stderr
     assert "[ERROR]" not in r.stdout and "generic" not in r.stderr, r.stdout + r.stderr
     print(r.stdout)
+
+
+def test_run_examples_walks_every_operator(tmp_path):
+    """`python -m catccos_amd.run_examples` (the counterpart of the reference's examples/run_all_examples.sh): every operator
+    over its reference shape list in perf mode, log patterns checked, summary line, exit status."""
+    import sys
+    r = subprocess.run([sys.executable, "-m", "catccos_amd.run_examples", "--iters", "2", "--warmup", "1", "--logs", str(tmp_path)],
+                       capture_output=True, text=True, timeout=600, cwd=ROOT)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "summary: 9 of 9 operators ran every shape of their lists" in r.stdout, r.stdout
+    assert r.stdout.count("a5moe") == 4 and r.stdout.count("a5mxfp8mmrs") == 6
+    # an operator that fails is reported and sets the exit status (a kernel name the driver does not know)
+    r = subprocess.run([sys.executable, "-c", "import catccos_amd.run_examples as m, sys; m.OPERATORS[:] = [('ascend950_mx_quant_allgather', 'nosuch', [])]; "
+                        "sys.argv = ['x']; sys.exit(m.main())"], capture_output=True, text=True, timeout=120, cwd=ROOT)
+    assert r.returncode == 1 and "FAILED" in r.stdout and "failed: ascend950_mx_quant_allgather" in r.stdout, r.stdout
