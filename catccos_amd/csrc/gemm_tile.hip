@@ -287,7 +287,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     constexpr int NPASS = 32 / PASS_ROWS;          // passes per 32-row MFMA tile
     constexpr int NSTORES = MT * NPASS;            // output stores per wave and tile (always issued; out-of-range lanes dropped)
     constexpr int NPARAM = DEQ ? 2 : 1;   // epilogue parameter requests per wave and tile
-    // requests per wave in the four slots of a step
+    // requests per wave in the four slots of a step, split by row blocks (the split by halves of K counts its own in `step`)
     constexpr int NL0 = 2;                          // A rows of row blocks 2-3 of the next step
     constexpr int NC0 = 2;                          // A rows of row blocks 0-1 of the step after the next
     constexpr int NL1 = NJ / 2 + (MX ? 1 : 0);      // half of the B panel share, scales (or a request that fetches nothing)
