@@ -297,7 +297,8 @@ int cch_moe_init_routing(const int32_t *expert_idx, int64_t rows, int num_expert
  *           over 1024 experts, or 8 Mi rows over 32); larger requests return CCH_EINVAL.
  *   sharing every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
  *           streams, two threads) race; calls in stream order do not.  Nothing in the array has to
- *           be cleared between calls (each call writes every entry it later reads). */
+ *           be cleared between calls (each call writes every entry it later reads).  Inputs that
+ *           one workgroup sorts (up to 8192 rows and 256 experts) do not touch the array at all. */
 #define CCH_ROUTING_NOALLOC_MAX_ENTRIES 262144
 int cch_moe_init_routing_noalloc(const int32_t *expert_idx, int64_t rows, int num_experts, int32_t *dst_to_src,
                                  int32_t *src_to_dst, int32_t *expert_tokens, int cumsum, void *stream);
