@@ -15,7 +15,6 @@ extern std::atomic<int> g_route_three_launches;        // routing.hip
 static std::atomic<int> g_force_generic{0};
 static std::atomic<int> g_require_tiled{0};
 static std::atomic<int> g_tile_order{-1};   // -1: chosen per problem
-static std::atomic<int> g_balance{0};
 static std::atomic<int> g_nt_out{-1};      // -1: chosen per problem
 
 static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
@@ -24,7 +23,6 @@ static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
     GemmProblem p = prob;
     const int order = g_tile_order.load();
     p.tile_order = order >= 0 ? order : 2;
-    p.balance_rounds = g_balance.load();
     const int nto = g_nt_out.load();
     p.nt_out = nto >= 0 ? nto : (kind == KIND_F4);
     const bool forced = g_force_generic.load() != 0;
@@ -70,10 +68,6 @@ int cch_set_option(const char *name, int value)
     }
     if (strcmp(name, "gemm_nt_output") == 0) {
         g_nt_out.store(value);
-        return CCH_OK;
-    }
-    if (strcmp(name, "gemm_balance_rounds") == 0) {
-        g_balance.store(value);
         return CCH_OK;
     }
     if (strcmp(name, "gemm_tile_order") == 0) {

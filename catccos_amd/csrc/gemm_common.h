@@ -46,7 +46,6 @@ struct GemmProblem {
     int64_t b_stride;        // bytes between experts in b
     int64_t sb_stride;       // bytes between experts in sb
     int nt_out;              // tiled kernels: output stores carry the non-temporal hint
-    int balance_rounds;      // tiled kernels: use only as many workgroups as the round count needs
     int tile_order;          // tiled kernels: 0 = row-major over (row tile, column tile); 1 = runs of consecutive tiles per XCD;
                              // 2 = a block of 4 row tiles x 8 column tiles per XCD where the shape allows (else 1 for groups, 0 without)
 };
@@ -78,49 +77,6 @@ __device__ inline void build_group_table(GroupTable &tab, const int32_t *group_s
     tile += (T - row + bm - 1) / bm;
     tab.row_start[num_groups + 1] = T;
     tab.tile_start[num_groups + 1] = tile;
-}
-
-// The same table built by one wave (all 64 lanes of the caller's first wave): lane l loads the size of group
-// g0 + l, so the loads of 64 groups are one request instead of a chain of dependent ones, and two wave scans give
-// the row and tile prefixes.  The running row after group g is min(T, sum of the non-negative sizes so far): once
-// the rows are used up every later group is empty, before that nothing is clipped.
-__device__ inline void build_group_table_wave(GroupTable &tab, const int32_t *group_sizes, int num_groups, int T, int bm)
-{
-    const int lane = threadIdx.x & 63;
-    long long raw_before = 0;   // sum of the non-negative sizes of the groups before this batch of 64
-    int tile_before = 0;
-    for (int g0 = 0; g0 < num_groups; g0 += 64) {
-        const int g = g0 + lane;
-        long long sz = 0;
-        if (g < num_groups) sz = group_sizes ? (long long)max(group_sizes[g], 0) : (long long)T;
-        long long incl = sz;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const long long up = __shfl_up(incl, off, 64);
-            if (lane >= off) incl += up;
-        }
-        const int row_lo = (int)min((long long)T, raw_before + incl - sz), row_hi = (int)min((long long)T, raw_before + incl);
-        const int tiles = (row_hi - row_lo + bm - 1) / bm;
-        int tincl = tiles;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int up = __shfl_up(tincl, off, 64);
-            if (lane >= off) tincl += up;
-        }
-        if (g < num_groups) {
-            tab.row_start[g] = row_lo;
-            tab.tile_start[g] = tile_before + tincl - tiles;
-        }
-        raw_before += __shfl(incl, 63, 64);
-        tile_before += __shfl(tincl, 63, 64);
-    }
-    if (lane == 0) {
-        const int row = (int)min((long long)T, raw_before);
-        tab.row_start[num_groups] = row;  // pseudo group: rows that belong to no expert
-        tab.tile_start[num_groups] = tile_before;
-        tab.row_start[num_groups + 1] = T;
-        tab.tile_start[num_groups + 1] = tile_before + (T - row + bm - 1) / bm;
-    }
 }
 
 // Group that owns global tile-row `tr` (largest g with tile_start[g] <= tr and a non-empty range).

@@ -1,0 +1,7 @@
+// Instantiates the tiled GEMM template: MXFP8 kernels with the SwiGLU epilogue, B stored [K, N].
+#include "gemm_tile_kernel.h"
+
+namespace cch {
+template int launch_tile_t<KIND_F8, EPI_SWIGLU, CCH_FMT_E4M3, 0>(const GemmProblem &, hipStream_t);
+template int launch_tile_t<KIND_F8, EPI_SWIGLU, CCH_FMT_E5M2, 0>(const GemmProblem &, hipStream_t);
+}  // namespace cch

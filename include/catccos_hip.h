@@ -339,9 +339,7 @@ int cch_dyn_quant_i8_rows_smooth(const void *x, const int32_t *src_rows, const f
  * over (row tile, column tile), 1 = each XCD takes a run of consecutive tiles of every round (whole
  * row tiles next to each other: fewer token and weight panels per L2), 2 = each XCD takes a block of
  * 4 row tiles x 8 column tiles of every round (where 8, 16, 32 or 64 column tiles and 256 workgroups
- * allow it; else 1 for grouped problems and 0 for dense ones), -1 (default) = 2; "gemm_balance_rounds" = 1 lets only as many workgroups take tiles as
- * the number of rounds needs (640 tiles on 256 CUs are three rounds: 216 workgroups do them in the
- * same three, with fewer CUs competing for L2 and memory), 0 (default) uses every CU;
+ * allow it; else 1 for grouped problems and 0 for dense ones), -1 (default) = 2;
  * "gemm_nt_output" = 1 / 0 gives or denies the output stores the non-temporal hint, -1 (default) gives it to the MXFP4 kernels, where it measured
  * 3-4 % faster (no difference for the others); "quant_integer_encoder" = 1 runs the E4M3
  * round-to-nearest-even quantiser through the integer encoder instead of the hardware conversion (an

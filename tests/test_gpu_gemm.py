@@ -525,10 +525,8 @@ def test_grouped_tile_order_covers_every_tile_once():
     outs = {}
     cc.set_option("require_tiled_gemm", 1)
     try:
-        for order in (0, 1, 2, -1, 3, 4):
-            # 3: the default order again, with a balanced count of workgroups taking tiles instead of every CU
+        for order in (0, 1, 2, -1, 4):
             # 4: the default order with non-temporal output stores
-            cc.set_option("gemm_balance_rounds", 1 if order == 3 else 0)
             cc.set_option("gemm_nt_output", 1 if order == 4 else 0 if order == 0 else -1)
             cc.set_option("gemm_tile_order", -1 if order >= 3 else order)
             # the output starts as NaN: a tile that no workgroup computes would keep it
@@ -537,13 +535,52 @@ def test_grouped_tile_order_covers_every_tile_once():
             outs[order] = out_f32(out)
     finally:
         cc.set_option("gemm_tile_order", -1)
-        cc.set_option("gemm_balance_rounds", 0)
         cc.set_option("gemm_nt_output", -1)
         cc.set_option("require_tiled_gemm", 0)
     assert not np.isnan(outs[1]).any()
-    for order in (1, 2, -1, 3, 4):
+    for order in (1, 2, -1, 4):
         assert np.array_equal(outs[0], outs[order]), order
     assert_close(outs[1], gold, "per-XCD tile order")
+
+
+@pytest.mark.parametrize("e,t,seed", [(70, 9000, 1), (200, 20000, 2), (256, 12000, 3), (5, 1300, 4)])
+def test_group_table_of_many_groups_covers_every_tile_once(e, t, seed):
+    """The tiled kernels build their table of row ranges and row tiles with wave-wide prefix sums, 64 groups per batch:
+    with more groups than one batch, empty ones, groups of one row, of exactly one and of several row tiles and rows that
+    belong to no group, every output element must be written exactly once (the output starts as NaN and is written
+    through an identity row map, which leaves rows of no group alone), the same bits under every tile order, and agree
+    with the oracle."""
+    rng = np.random.default_rng(seed)
+    k, n = 128, 4096
+    gs = rng.integers(0, 2 * t // e, e).astype(np.int32)
+    gs[rng.integers(0, e, max(e // 8, 1))] = 0
+    gs[rng.integers(0, e)] = 256
+    gs[rng.integers(0, e)] = 64
+    gs[rng.integers(0, e)] = 1
+    while gs.sum() > t - 5:
+        gs[int(gs.argmax())] //= 2
+    pa, sa = orc.mx_quant_rows(rand_bf16(rng, (t, k), 1.0), orc.E4M3)
+    pbs, sbs = zip(*[orc.mx_quant_b(rand_bf16(rng, (k, n), 1.0), orc.E4M3, orc.RNE, 0) for _ in range(e)])
+    pb, sb = np.stack(pbs), np.stack(sbs)
+    ident = np.arange(t, dtype=np.int32)
+    outs = {}
+    cc.set_option("require_tiled_gemm", 1)
+    try:
+        for order in (0, 1, 2):
+            cc.set_option("gemm_tile_order", order)
+            out = torch.full((t, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+            cc.mx_grouped_matmul_mapped(dev(pa), dev(sa), dev(pb), dev(sb), dev(gs), dev(ident), out, "e4m3", 0)
+            outs[order] = out_f32(out)
+    finally:
+        cc.set_option("gemm_tile_order", -1)
+        cc.set_option("require_tiled_gemm", 0)
+    used = int(gs.sum())
+    for order in (0, 1, 2):
+        assert not np.isnan(outs[order][:used]).any(), order
+        assert np.isnan(outs[order][used:]).all(), order   # rows of no group are not written through a row map
+        assert np.array_equal(outs[0][:used], outs[order][:used]), order
+    gold = orc.mx_gmm(pa, sa, pb, sb, n, k, orc.E4M3, 0, group_sizes=gs)
+    assert_close(outs[2][:used], gold[:used], ("many groups", e, t))
 
 
 # ---------------------------------------------------------------- half-precision output
