@@ -92,6 +92,9 @@ def parity_record(got, gold):
             "within_1e-2": bool(m["max_rel_floor1"] <= 1e-2 and m["max_rel_floor_rms"] <= 1e-2)}
 
 
+LAST_WARM = {"launches": 0, "ms": 0.0}   # what the last event_time_ms() call ran untimed
+
+
 def event_time_ms(fn, steps, warmup, warm_ms=0.0):
     """Wall time per step, average launch duration over the timed region and per-launch durations of fn()
     on the current stream, the latter two by HIP events.
@@ -102,13 +105,17 @@ def event_time_ms(fn, steps, warmup, warm_ms=0.0):
     """
     import torch
     t0 = time.perf_counter()
+    launches = 0
     for _ in range(warmup):
         fn()
+    launches += warmup
     torch.cuda.synchronize()
     while (time.perf_counter() - t0) * 1e3 < warm_ms:
         for _ in range(10):
             fn()
+        launches += 10
         torch.cuda.synchronize()
+    LAST_WARM["launches"], LAST_WARM["ms"] = launches, (time.perf_counter() - t0) * 1e3
     # the timed region: exactly `steps` launches queued back to back between one pair of events
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
@@ -298,6 +305,7 @@ def main():
 
         # `warmup` launches as asked for, then more of the same until the shader clock has settled (see event_time_ms)
         wall_ms, kernel_ms, per_ms = event_time_ms(step, args.steps, args.warmup, warm_ms=100.0)
+        warm_run = dict(LAST_WARM)
         flop = 2.0 * T * N * K
         value = flop / (wall_ms * 1e-3) / 1e12
         achieved = flop / (kernel_ms * 1e-3) / 1e12
@@ -328,6 +336,10 @@ def main():
             "n_gpus": 1,
             "steps": args.steps,
             "warmup": args.warmup,
+            # the untimed part is the `warmup` launches asked for plus more of the same until 100 ms have passed (the shader
+            # clock settles after about 50 ms of load): what actually ran before the timed region
+            "warmup_launches_run": warm_run["launches"],
+            "warm_ms": round(warm_run["ms"], 1),
             "ms_per_step": round(wall_ms, 4),
             "higher_is_better": True,
             "scaling": "weak",
@@ -338,6 +350,8 @@ def main():
                        "n": N, "trans_b": TRANS_B, "group_sizes": gs_host.tolist()},
             "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(achieved / FP8_PEAK_TFLOPS, 4), "traffic": GMM_TRAFFIC_BYTES,
+                         # (a constant of this script, from the counter runs summarised in that file: not measured by this run)
+                         "traffic_source": "profiles/gemm_tile_mxfp8_grouped_cfg5_e4m3.md",
                          "kernel": "gemm_tile_kernel<KIND_F8, EPI_PLAIN, E4M3, TB=0, UA=0>", "algorithmic_flop_per_launch": flop,
                          "kernel_ms_min": round(float(np.min(per_ms)), 4), "kernel_ms_median": round(float(np.median(per_ms)), 4),
                          "kernel_ms_mean": round(kernel_ms, 4), "kernel_ms_mean_single_launches": round(float(np.mean(per_ms)), 4), **clk},

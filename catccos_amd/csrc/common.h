@@ -12,6 +12,8 @@ namespace cch {
 
 // Records a message for cch_last_error() and returns `code`.
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// Empties the calling thread's message (a call that succeeds without a note leaves none behind).
+void clear_error();
 
 #define CCH_HIP(call)                                                                              \
     do {                                                                                           \

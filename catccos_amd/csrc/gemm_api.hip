@@ -16,13 +16,17 @@ static std::atomic<int> g_force_generic{0};
 static std::atomic<int> g_require_tiled{0};
 static std::atomic<int> g_tile_order{-1};   // -1: chosen per problem
 static std::atomic<int> g_nt_out{-1};      // -1: chosen per problem
+static std::atomic<int> g_i8_fp16_step{0};
 
 static int run(const GemmProblem &prob, int kind, int epi, hipStream_t stream)
 {
+    // the message of this thread describes this call only: a fall-back note of an earlier call must not outlive it
+    clear_error();
     if (prob.T == 0 || prob.n_out == 0) return CCH_OK;
     GemmProblem p = prob;
     const int order = g_tile_order.load();
     p.tile_order = order >= 0 ? order : 2;
+    p.i8_fp16_step = g_i8_fp16_step.load() != 0;
     const int nto = g_nt_out.load();
     p.nt_out = nto >= 0 ? nto : (kind == KIND_F4);
     const bool forced = g_force_generic.load() != 0;
@@ -68,6 +72,10 @@ int cch_set_option(const char *name, int value)
     }
     if (strcmp(name, "gemm_nt_output") == 0) {
         g_nt_out.store(value);
+        return CCH_OK;
+    }
+    if (strcmp(name, "i8_epilogue_fp16_step") == 0) {
+        g_i8_fp16_step.store(value);
         return CCH_OK;
     }
     if (strcmp(name, "gemm_tile_order") == 0) {

@@ -30,6 +30,12 @@ struct GemmProblem {
     const int32_t *out_row_map;  // device int32[T] or nullptr: row of `out` that receives row i (negative: dropped)
     int64_t out_rows;        // rows of `out` when out_row_map is given
     int out_fp16;            // output elements are IEEE half instead of bf16 (both rounded to nearest even)
+    int i8_fp16_step;        // int8 epilogues: acc * per_channel is rounded to IEEE half (nearest even) before the per-token
+                             // factor, as the reference's device does - its matrix unit's output stage writes the per-channel
+                             // product as fp16 and the vector epilogue widens it again
+                             // (include/catccos/epilogue/block/block_epilogue_per_token_dequant_swiglu.hpp:348-361; the golden
+                             // generator's option, examples/utils/gen_data_dispatch_gmm_dequant_swiglu.py:309-310).  0 keeps
+                             // fp32 throughout, the golden generator's default path.
     int mx_out;              // SwiGLU epilogue only: 1 = the activation leaves MX-quantised along its rows (what the
                              // row quantiser would make of the bf16 output): payload [T, n_out] codes of format
                              // mx_out_fmt at `out` (FP4: two per byte), E8M0 scales [T, mx_out_sld] at `out_scales`

@@ -71,8 +71,8 @@ __global__ __launch_bounds__(256) void gemm_naive_kernel(GemmProblem p)
     __shared__ GroupTable tab;
     if (threadIdx.x == 0) build_group_table(tab, p.group_sizes, p.num_groups, p.T, 1);
     __syncthreads();
-    const int col = blockIdx.x * 256 + threadIdx.x;
-    const int row = blockIdx.y;
+    const int col = blockIdx.y * 256 + threadIdx.x;
+    const int row = blockIdx.x;   // rows on the grid's x axis: it takes 2^31 - 1 of them
     if (col >= p.n_out) return;
     const int e = find_group(tab, p.num_groups, row);  // bm = 1: tile rows are rows
     size_t out_row = (size_t)row;
@@ -91,11 +91,25 @@ __global__ __launch_bounds__(256) void gemm_naive_kernel(GemmProblem p)
         } else if (EPI == EPI_DEQUANT_SWIGLU) {
             float g = dot_column<KIND>(p, row, e, col) * p.per_ch[(size_t)e * p.N + col];
             float u = dot_column<KIND>(p, row, e, col + p.n_out) * p.per_ch[(size_t)e * p.N + col + p.n_out];
+            if (p.i8_fp16_step) {
+                // the reference's device hands the per-channel product on as IEEE half (gemm_common.h); the fp32 product
+                // is rounded first, as the golden's two casts do (no fused product-and-convert instruction)
+                asm volatile("" : "+v"(g), "+v"(u));
+                g = (float)(_Float16)g;
+                u = (float)(_Float16)u;
+            }
             g *= p.per_tok[row];
             u *= p.per_tok[row];
             v = g * (1.0f / (1.0f + expf(-g))) * u;
         } else if (EPI == EPI_DEQUANT) {
-            v = dot_column<KIND>(p, row, e, col) * p.per_tok[row] * p.per_ch[(size_t)e * p.N + col];
+            const float a = dot_column<KIND>(p, row, e, col);
+            if (p.i8_fp16_step) {
+                float prod = a * p.per_ch[(size_t)e * p.N + col];
+                asm volatile("" : "+v"(prod));
+                v = (float)(_Float16)prod * p.per_tok[row];
+            } else {
+                v = a * p.per_tok[row] * p.per_ch[(size_t)e * p.N + col];
+            }
         } else {
             v = dot_column<KIND>(p, row, e, col);
         }
@@ -113,8 +127,8 @@ __global__ __launch_bounds__(256) void gemm_naive_swiglu_mx_kernel(GemmProblem p
     __shared__ GroupTable tab;
     if (threadIdx.x == 0) build_group_table(tab, p.group_sizes, p.num_groups, p.T, 1);
     __syncthreads();
-    const int col = blockIdx.x * 256 + threadIdx.x;
-    const int row = blockIdx.y;
+    const int col = blockIdx.y * 256 + threadIdx.x;
+    const int row = blockIdx.x;
     const bool live = col < p.n_out;
     const int e = find_group(tab, p.num_groups, row);
     float v = 0.0f;
@@ -122,6 +136,11 @@ __global__ __launch_bounds__(256) void gemm_naive_swiglu_mx_kernel(GemmProblem p
         if (KIND == KIND_I8) {
             float g = dot_column<KIND>(p, row, e, col) * p.per_ch[(size_t)e * p.N + col];
             float u = dot_column<KIND>(p, row, e, col + p.n_out) * p.per_ch[(size_t)e * p.N + col + p.n_out];
+            if (p.i8_fp16_step) {
+                asm volatile("" : "+v"(g), "+v"(u));
+                g = (float)(_Float16)g;
+                u = (float)(_Float16)u;
+            }
             g *= p.per_tok[row];
             u *= p.per_tok[row];
             v = g * (1.0f / (1.0f + expf(-g))) * u;
@@ -159,8 +178,8 @@ template <int KIND, int EPI>
 static int launch_naive_t(const GemmProblem &p, hipStream_t stream)
 {
     if (p.T == 0 || p.n_out == 0) return CCH_OK;
-    if (p.T > 65535) return fail(CCH_ENOSUP, "generic GEMM path takes at most 65535 rows per call (got %d)", p.T);
-    dim3 grid((unsigned)((p.n_out + 255) / 256), (unsigned)p.T);
+    if ((p.n_out + 255) / 256 > 65535) return fail(CCH_ENOSUP, "generic GEMM path takes at most 65535 * 256 output columns per call (got %d)", p.n_out);
+    dim3 grid((unsigned)p.T, (unsigned)((p.n_out + 255) / 256));
     hipLaunchKernelGGL((gemm_naive_kernel<KIND, EPI>), grid, dim3(256), 0, stream, p);
     return launch_status("gemm_naive_kernel");
 }
@@ -170,8 +189,8 @@ int launch_gemm_naive(const GemmProblem &p, int kind, int epi, hipStream_t strea
     if (p.mx_out) {
         if (epi != EPI_DEQUANT_SWIGLU && epi != EPI_SWIGLU) return fail(CCH_ENOSUP, "MX-quantised output exists for the SwiGLU epilogues only");
         if (p.T == 0 || p.n_out == 0) return CCH_OK;
-        if (p.T > 65535) return fail(CCH_ENOSUP, "generic GEMM path takes at most 65535 rows per call (got %d)", p.T);
-        dim3 grid((unsigned)((p.n_out + 255) / 256), (unsigned)p.T);
+        if ((p.n_out + 255) / 256 > 65535) return fail(CCH_ENOSUP, "generic GEMM path takes at most 65535 * 256 output columns per call (got %d)", p.n_out);
+        dim3 grid((unsigned)p.T, (unsigned)((p.n_out + 255) / 256));
 #define CCH_NAIVE_MX_OUT(K)                                                                                                                        \
     do {                                                                                                                                           \
         if (p.mx_out_fmt == CCH_FMT_E4M3) hipLaunchKernelGGL((gemm_naive_swiglu_mx_kernel<K, CCH_FMT_E4M3>), grid, dim3(256), 0, stream, p);      \

@@ -355,7 +355,11 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     constexpr int CPR = ROWB / 16;                 // 16-byte chunks per staged row
     constexpr int PASS_ROWS = 64 / CPR;            // rows staged per pass: 1 KiB, one read-back instruction
     constexpr int NPASS = 32 / PASS_ROWS;          // passes per 32-row MFMA tile
-    constexpr int NSTORES = MT * NPASS;            // output stores per wave and tile (always issued; out-of-range lanes dropped)
+    // Output stores per wave and tile that the first step's request counts allow for: one per pass, always issued
+    // (out-of-range lanes are dropped by the bounds check).  The MX-quantised activation issues two or three per pass
+    // (payload, scale byte, padding byte); requests complete in order, so the waits that count NSTORES younger stores
+    // are then merely stricter than they need to be.
+    constexpr int NSTORES = MT * NPASS;
     constexpr int NPARAM = DEQ ? 2 : 1;   // epilogue parameter requests per wave and tile
     // requests per wave in the four slots of a step, split by row blocks (the split by halves of K counts its own in `step`)
     constexpr int NL0 = 2;                          // A rows of row blocks 2-3 of the next step
@@ -498,6 +502,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     const int nk_tile = ksteps;
 #ifdef CCH_PROF
     uint64_t pf_wa = 0, pf_wb = 0, pf_b0 = 0, pf_b1 = 0, pf_b2 = 0, pf_b3 = 0, pf_l0 = 0;
+    uint64_t pf_dec = 0;   // clocks in the decode of the next tile
     int pf_nt = 0;
     const uint64_t pf_start = __builtin_readcyclecounter();
 #endif
@@ -517,8 +522,8 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             // Workgroup w of a round runs on XCD w % 8.  Each XCD takes a block of 4 row tiles x 8
             // column tiles of the round (256 / n_tiles row tiles by n_tiles column tiles): a weight
             // panel then has up to four users in one L2 and a token panel eight.
-            const int x = w & 7, i = w >> 3, cb = n_tiles >> 3;
-            place = ((x / cb) * 4 + (i >> 3)) * n_tiles + (x % cb) * 8 + (i & 7);
+            const int x = w & 7, i = w >> 3, lcb = __builtin_ctz(n_tiles >> 3);   // 1, 2, 4 or 8 blocks of 8 column tiles
+            place = ((x >> lcb) * 4 + (i >> 3)) * n_tiles + (x & ((1 << lcb) - 1)) * 8 + (i & 7);
         } else if (whole_round && (p.tile_order == 1 || (p.tile_order == 2 && p.group_sizes != nullptr && p.num_groups > 1)) && (G & 7) == 0) {
             // Each XCD takes a run of nwg / 8 consecutive tiles of the round (whole row tiles next
             // to each other), so that its L2 fetches one or two A panels and the B panels of one or
@@ -1166,7 +1171,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                     step(IC<0>{}, IC<0>{}, nblk_c, IC<0>{}, kt);
                     step(IC<0>{}, IC<0>{}, nblk_c, IC<1>{}, kt + 1);
                 }
-                decode(t + nwg, nxt);
+                { PROF_BEGIN(t_); decode(t + nwg, nxt); PROF_END(t_, pf_dec); }
                 step(IC<1>{}, IC<0>{}, nblk_c, IC<0>{}, nk - 2);
             } else {
                 decode(t + nwg, nxt);
@@ -1175,7 +1180,7 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             step(IC<2>{}, IC<0>{}, nblk_c, IC<1>{}, nk - 1);
         };
 #ifdef CCH_PROF
-        const uint64_t pf_k0 = __builtin_readcyclecounter(), pf_w0 = wall_clock64();
+        const uint64_t pf_k0 = __builtin_readcyclecounter();
 #endif
         const int nblk = uniform(min(max((((cur.rows + 31) >> 5) + 1 - wm) >> 1, 1), MT));
         if (nblk == 4) k_loop(IC<4>{});
@@ -1217,8 +1222,10 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             // The passes are software-pipelined: the values of pass n+1 are converted and written while the read
             // of pass n is under way (one wave's LDS operations execute in order, so the later writes cannot
             // overtake the earlier read), and only then is pass n stored.
-            auto produce = [&](auto i_c, auto ps_c, auto fp16_c) {
+            auto produce = [&](auto i_c, auto ps_c, auto fp16_c, auto half_step_c) {
                 constexpr int i = decltype(i_c)::value, ps = decltype(ps_c)::value;
+                // int8 epilogues: the per-channel product passes through IEEE half first (GemmProblem::i8_fp16_step)
+                constexpr bool HALF_STEP = decltype(half_step_c)::value != 0;
 #pragma unroll
                 for (int qq = 0; qq < PASS_ROWS / 8; qq++) {
                     const int q = ps * (PASS_ROWS / 8) + qq;
@@ -1242,12 +1249,27 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                                     const float up = (float)(__bf16)(float)acc[i][1][x + d];
                                     v[d] = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;
                                 } else if (SWIGLU) {
-                                    const float gate = (float)acc[i][0][x + d] * chs[0] * tok[xr + d];
-                                    const float up = (float)acc[i][1][x + d] * chs[1] * tok[xr + d];
+                                    float gate = (float)acc[i][0][x + d] * chs[0], up = (float)acc[i][1][x + d] * chs[1];
+                                    if constexpr (HALF_STEP) {
+                                        // (the fp32 product is rounded before the half conversion sees it, as the golden's
+                                        // two casts do: the compiler would otherwise fuse product and conversion into one
+                                        // mixed-precision instruction with a single rounding)
+                                        asm volatile("" : "+v"(gate), "+v"(up));
+                                        gate = (float)(_Float16)gate;
+                                        up = (float)(_Float16)up;
+                                    }
+                                    gate *= tok[xr + d];
+                                    up *= tok[xr + d];
                                     // hardware exp2 and reciprocal: relative error ~1e-6, far inside the bf16 result
                                     v[d] = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;
                                 } else if (EPI == EPI_DEQUANT) {
-                                    v[d] = (float)acc[i][j][x + d] * tok[xr + d] * chs[j];
+                                    if constexpr (HALF_STEP) {
+                                        float prod = (float)acc[i][j][x + d] * chs[j];
+                                        asm volatile("" : "+v"(prod));   // (see the SwiGLU branch)
+                                        v[d] = (float)(_Float16)prod * tok[xr + d];
+                                    } else {
+                                        v[d] = (float)acc[i][j][x + d] * tok[xr + d] * chs[j];
+                                    }
                                 } else {
                                     v[d] = (float)acc[i][j][x + d];
                                 }
@@ -1335,12 +1357,12 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 else __builtin_amdgcn_raw_buffer_store_b128(sv, rs_out, (int)off, 0, 0);
             };
             constexpr int NP = MT * NPASS;
-            auto all_passes = [&](auto fp16_c) {
-                produce(IC<0>{}, IC<0>{}, fp16_c);
+            auto all_passes = [&](auto fp16_c, auto half_step_c) {
+                produce(IC<0>{}, IC<0>{}, fp16_c, half_step_c);
                 PassData pending = readback(IC<0>{}, IC<0>{});
                 static_for<NP - 1>([&](auto n_c) {
                     constexpr int n = decltype(n_c)::value + 1;
-                    produce(IC<n / NPASS>{}, IC<n % NPASS>{}, fp16_c);
+                    produce(IC<n / NPASS>{}, IC<n % NPASS>{}, fp16_c, half_step_c);
                     __builtin_amdgcn_sched_barrier(0);   // the store's address arithmetic waits for the read: keep it behind the conversions
                     emit(IC<(n - 1) / NPASS>{}, IC<(n - 1) % NPASS>{}, pending);
                     pending = readback(IC<n / NPASS>{}, IC<n % NPASS>{});
@@ -1349,14 +1371,24 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             };
             // the output type is a wave-uniform choice: one copy of the passes for each (the MX-quantised activation is
             // made from bf16 values)
-            if (p.out_fp16) all_passes(IC<1>{});
-            else all_passes(IC<0>{});
+            if constexpr (DEQ) {
+                if (p.i8_fp16_step) {
+                    if (p.out_fp16) all_passes(IC<1>{}, IC<1>{});
+                    else all_passes(IC<0>{}, IC<1>{});
+                } else {
+                    if (p.out_fp16) all_passes(IC<1>{}, IC<0>{});
+                    else all_passes(IC<0>{}, IC<0>{});
+                }
+            } else {
+                if (p.out_fp16) all_passes(IC<1>{}, IC<0>{});
+                else all_passes(IC<0>{}, IC<0>{});
+            }
         }
 #ifdef CCH_PROF
         if (lane == 0 && (wave & 3) == 0 && blockIdx.x < 256 && pf_nt < PROF_TILES) {
             uint64_t *o = cch_prof_tiles + (((size_t)blockIdx.x * 2 + wm) * PROF_TILES + pf_nt) * 6;
             o[0] = (uint64_t)(uint32_t)t | ((uint64_t)(uint32_t)cur.rows << 32) | ((uint64_t)(uint32_t)cur.e << 48);
-            o[1] = pf_k0; o[2] = pf_k1; o[3] = __builtin_readcyclecounter(); o[4] = pf_w0; o[5] = pf_entry;
+            o[1] = pf_k0; o[2] = pf_k1; o[3] = __builtin_readcyclecounter(); o[4] = pf_dec; o[5] = pf_entry;
         }
         pf_nt++;
 #endif

@@ -16,6 +16,8 @@ int fail(int code, const char *fmt, ...)
     va_end(ap);
     return code;
 }
+
+void clear_error() { g_err[0] = '\0'; }
 }  // namespace cch
 
 using cch::fail;

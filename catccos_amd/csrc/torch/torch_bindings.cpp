@@ -19,7 +19,9 @@
 #include <torch/library.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cctype>
+#include <initializer_list>
 #include <mutex>
 #include <string>
 #include <tuple>
@@ -29,7 +31,8 @@
 namespace {
 
 struct CatccosTorchState {
-    bool initialized = false;
+    std::atomic<bool> initialized{false};   // read without the lock by every operator
+    std::atomic<bool> launched{false};      // some operator of this library has put work on a stream
     int64_t rank_id = -1, rank_size = 0;
     std::mutex mu;
 };
@@ -42,7 +45,26 @@ CatccosTorchState &State()
 
 void NeedInit()
 {
-    TORCH_CHECK(State().initialized, "catccos TORCH_LIBRARY not initialized, call torch.ops.catccos.init(...) first");
+    TORCH_CHECK(State().initialized.load(std::memory_order_acquire), "catccos TORCH_LIBRARY not initialized, call torch.ops.catccos.init(...) first");
+}
+
+// Every tensor argument of a device kernel must live on the GPU of the first one.  The dispatcher picks the GPU
+// kernel as soon as one argument is a GPU tensor; a host tensor among the others (group sizes often live on the
+// host) would hand a host address to a kernel (the reference checks the same, torch_bindings.cpp:140-144).  Called
+// before anything is allocated or launched.
+struct NamedTensor {
+    const char *name;
+    const at::Tensor &t;
+};
+void SameDevice(const char *op, std::initializer_list<NamedTensor> args)
+{
+    const NamedTensor &first = *args.begin();
+    for (const NamedTensor &a : args) {
+        TORCH_CHECK(a.t.defined(), "catccos::", op, ": ", a.name, " is undefined");
+        TORCH_CHECK(a.t.is_cuda(), "catccos::", op, ": ", a.name, " must be a GPU tensor, got one on ", a.t.device());
+        TORCH_CHECK(a.t.device() == first.t.device(), "catccos::", op, ": ", a.name, " is on ", a.t.device(), " but ", first.name, " is on ",
+                    first.t.device());
+    }
 }
 
 int FormatCode(const std::string &name)
@@ -62,7 +84,11 @@ int64_t ScaleCols(int64_t k) { return 2 * ((k + 63) / 64); }   // E8M0 bytes per
 
 // (a ROCm build of PyTorch presents its HIP devices and streams under the names of the GPU key: the stream of a
 // tensor's device is asked for through that front)
-void *StreamOf(const at::Tensor &t) { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream(); }
+void *StreamOf(const at::Tensor &t)
+{
+    State().launched.store(true, std::memory_order_release);
+    return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream();
+}
 
 void Check(int rc, const char *what) { TORCH_CHECK(rc == CCH_OK, "catccos::", what, ": ", cch_last_error()); }
 
@@ -75,16 +101,16 @@ int64_t Init(int64_t rank_id, int64_t rank_size, int64_t local_mem_size, std::st
 {
     auto &st = State();
     std::lock_guard<std::mutex> lock(st.mu);
-    if (st.initialized) return 0;
+    if (st.initialized.load()) return 0;
     TORCH_CHECK(rank_id >= 0, "invalid rank_id: ", rank_id);
     TORCH_CHECK(rank_size > 0, "invalid rank_size: ", rank_size);
     TORCH_CHECK(local_mem_size > 0, "invalid local_mem_size: ", local_mem_size);
     TORCH_CHECK(!ip_port.empty(), "ip_port is empty");
     TORCH_CHECK(rank_size == 1 && rank_id == 0, "catccos on one GPU has no peers: rank_size must be 1 and rank_id 0, got ", rank_id, " of ",
                 rank_size);
-    st.initialized = true;
     st.rank_id = rank_id;
     st.rank_size = rank_size;
+    st.initialized.store(true, std::memory_order_release);
     return 0;
 }
 
@@ -92,12 +118,12 @@ int64_t Finalize()
 {
     auto &st = State();
     std::lock_guard<std::mutex> lock(st.mu);
-    if (!st.initialized) return 0;
-    // the reference drains its stream before it lets go of its buffers; a process that never touched the GPU
-    // has nothing to drain (and must not initialise it here)
-    int devices = 0;
-    if (hipGetDeviceCount(&devices) == hipSuccess && devices > 0) (void)hipStreamSynchronize(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
-    st.initialized = false;
+    if (!st.initialized.load()) return 0;
+    // the reference drains its stream before it lets go of its buffers; a process in which no operator of this
+    // library ever launched (only init / finalize or Meta-shape calls) has nothing to drain and must not create a
+    // GPU context here
+    if (st.launched.load(std::memory_order_acquire)) (void)hipStreamSynchronize(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
+    st.initialized.store(false, std::memory_order_release);
     st.rank_id = -1;
     st.rank_size = 0;
     return 0;
@@ -166,6 +192,7 @@ std::tuple<at::Tensor, at::Tensor> MxQuant(const at::Tensor &x_in, std::string f
     const int fmt = FormatCode(fmt_name);
     TORCH_CHECK(x_in.dim() == 2 && (x_in.scalar_type() == at::kBFloat16 || x_in.scalar_type() == at::kHalf),
                 "mx_quant expects a 2-D bfloat16 (or float16) tensor");
+    SameDevice("mx_quant", {{"x", x_in}});
     c10::DeviceGuard guard(x_in.device());
     const at::Tensor x = x_in.contiguous();
     const int64_t m = x.size(0), k = x.size(1);
@@ -182,6 +209,7 @@ at::Tensor W8A8MatmulDequant(const at::Tensor &a_in, const at::Tensor &b_in, con
     NeedInit();
     TORCH_CHECK(a_in.dim() == 2 && a_in.scalar_type() == at::kChar, "a must be a 2-D int8 tensor");
     TORCH_CHECK(b_in.dim() == 2 && b_in.scalar_type() == at::kChar, "b must be a 2-D int8 tensor");
+    SameDevice("w8a8_matmul_dequant", {{"a", a_in}, {"b", b_in}, {"per_tok", per_tok_in}, {"per_ch", per_ch_in}});
     c10::DeviceGuard guard(a_in.device());
     const at::Tensor a = a_in.contiguous(), b = b_in.contiguous();
     const int64_t m = a.size(0), k = a.size(1), n = trans_b ? b.size(0) : b.size(1);
@@ -198,6 +226,7 @@ at::Tensor W8A8MatmulDequant(const at::Tensor &a_in, const at::Tensor &b_in, con
 at::Tensor MxMatmul(const at::Tensor &a_in, const at::Tensor &sa_in, const at::Tensor &b_in, const at::Tensor &sb_in, std::string fmt_name, int64_t trans_b)
 {
     NeedInit();
+    SameDevice("mx_matmul", {{"a", a_in}, {"sa", sa_in}, {"b", b_in}, {"sb", sb_in}});
     c10::DeviceGuard guard(a_in.device());
     const at::Tensor a = a_in.contiguous(), sa = sa_in.contiguous(), b = b_in.contiguous(), sb = sb_in.contiguous();
     const MxShape s = MxShapes(a, sa, b, sb, fmt_name, trans_b, false);
@@ -212,6 +241,7 @@ at::Tensor GmmDequantSwiglu(const at::Tensor &x_in, const at::Tensor &w_in, cons
                             const at::Tensor &per_ch_in, int64_t trans_b)
 {
     NeedInit();
+    SameDevice("gmm_dequant_swiglu", {{"x", x_in}, {"w", w_in}, {"group_sizes", gs_in}, {"per_tok", per_tok_in}, {"per_ch", per_ch_in}});
     c10::DeviceGuard guard(x_in.device());
     const at::Tensor x = x_in.contiguous(), w = w_in.contiguous(), gs = gs_in.contiguous();
     const at::Tensor per_tok = per_tok_in.contiguous().to(at::kFloat), per_ch = per_ch_in.contiguous().to(at::kFloat);
@@ -228,6 +258,7 @@ std::tuple<at::Tensor, at::Tensor> GmmDequantSwigluMx(const at::Tensor &x_in, co
 {
     NeedInit();
     const int fmt = FormatCode(fmt_name);
+    SameDevice("gmm_dequant_swiglu_mx", {{"x", x_in}, {"w", w_in}, {"group_sizes", gs_in}, {"per_tok", per_tok_in}, {"per_ch", per_ch_in}});
     c10::DeviceGuard guard(x_in.device());
     const at::Tensor x = x_in.contiguous(), w = w_in.contiguous(), gs = gs_in.contiguous();
     const at::Tensor per_tok = per_tok_in.contiguous().to(at::kFloat), per_ch = per_ch_in.contiguous().to(at::kFloat);
@@ -245,6 +276,7 @@ at::Tensor MxGroupedMatmul(const at::Tensor &a_in, const at::Tensor &sa_in, cons
                            std::string fmt_name, int64_t trans_b)
 {
     NeedInit();
+    SameDevice("mx_grouped_matmul", {{"a", a_in}, {"sa", sa_in}, {"b", b_in}, {"sb", sb_in}, {"group_sizes", gs_in}});
     c10::DeviceGuard guard(a_in.device());
     const at::Tensor a = a_in.contiguous(), sa = sa_in.contiguous(), b = b_in.contiguous(), sb = sb_in.contiguous(), gs = gs_in.contiguous();
     const MxShape s = MxShapes(a, sa, b, sb, fmt_name, trans_b, true);
@@ -261,6 +293,7 @@ std::tuple<at::Tensor, at::Tensor> MxGroupedMatmulSwigluMx(const at::Tensor &a_i
 {
     NeedInit();
     const int ofmt = FormatCode(out_fmt_name);
+    SameDevice("mx_grouped_matmul_swiglu_mx", {{"a", a_in}, {"sa", sa_in}, {"b", b_in}, {"sb", sb_in}, {"group_sizes", gs_in}});
     c10::DeviceGuard guard(a_in.device());
     const at::Tensor a = a_in.contiguous(), sa = sa_in.contiguous(), b = b_in.contiguous(), sb = sb_in.contiguous(), gs = gs_in.contiguous();
     const MxShape s = MxShapes(a, sa, b, sb, fmt_name, trans_b, true);
@@ -286,6 +319,7 @@ at::Tensor MoeFfnMxfp8(const at::Tensor &x_in, const at::Tensor &expert_idx_in, 
                 "expert_idx must be an int32 [m, top_k] tensor");
     TORCH_CHECK(probs_in.sizes() == expert_idx_in.sizes() && probs_in.scalar_type() == at::kFloat, "probs must be a float32 [m, top_k] tensor");
     TORCH_CHECK(w1_in.dim() == 3 && w2_in.dim() == 3 && w1_in.size(0) == w2_in.size(0), "w1 and w2 must hold one matrix per expert");
+    SameDevice("moe_ffn_mxfp8", {{"x", x_in}, {"expert_idx", expert_idx_in}, {"probs", probs_in}, {"w1", w1_in}, {"sw1", sw1_in}, {"w2", w2_in}, {"sw2", sw2_in}});
     c10::DeviceGuard guard(x_in.device());
     const at::Tensor x = x_in.contiguous(), idx = expert_idx_in.contiguous(), probs = probs_in.contiguous();
     const at::Tensor w1 = w1_in.contiguous(), sw1 = sw1_in.contiguous(), w2 = w2_in.contiguous(), sw2 = sw2_in.contiguous();

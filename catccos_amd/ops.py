@@ -68,10 +68,14 @@ def packed_row_bytes(k, fmt="e4m3"):
     return ((k + 1) // 2 if _fmt(fmt) in _FP4 else k) + scale_cols(k)
 
 
-def mx_quant_scatter_packed(x, expanded_row_idx, packed_out, top_k, fmt="e4m3", rounding=ROUND_RNE):
+def mx_quant_scatter_packed(x, expanded_row_idx, packed_out, top_k, fmt="e4m3", rounding=ROUND_RNE, check_routes=False):
     """Quantises every row of x (bf16 [tokens, K]) once and writes [payload | scales] to rows
     expanded_row_idx[t * top_k + r] of packed_out (uint8 [rows, packed_row_bytes(K)]), skipping
-    negative entries and entries at or past `rows`.  Rows that no route names keep their contents.  Returns packed_out."""
+    negative entries and entries at or past `rows`.  Rows that no route names keep their contents.  Returns packed_out.
+
+    An entry at or past `rows` is a caller's error that the kernel turns into a dropped token (it cannot report from the
+    device, and the reference treats it as the caller's error too).  check_routes=True looks at the whole table first and
+    raises ValueError for such an entry: a debugging aid, it waits for the stream."""
     fmt = _fmt(fmt)
     _require_gpu(x, expanded_row_idx, packed_out)
     if x.dim() != 2 or x.dtype != torch.bfloat16:
@@ -83,7 +87,9 @@ def mx_quant_scatter_packed(x, expanded_row_idx, packed_out, top_k, fmt="e4m3", 
     if packed_out.dim() != 2 or packed_out.dtype != torch.uint8 or packed_out.shape[1] != row_bytes or not packed_out.is_contiguous():
         raise ValueError("packed_out must be a contiguous uint8 [rows, %d] tensor" % row_bytes)
     # the kernel skips entries at or past packed_out's rows (like negative ones): no pass over the table
-    # here, which would stall the stream
+    # here, which would stall the stream, unless the caller asks for it
+    if check_routes and expanded_row_idx.numel() and int(expanded_row_idx.max()) >= packed_out.shape[0]:
+        raise ValueError("expanded_row_idx names row %d but packed_out has %d rows" % (int(expanded_row_idx.max()), packed_out.shape[0]))
     x = x.contiguous()
     idx = expanded_row_idx.contiguous()
     check(_abi.lib().cch_mx_quant_scatter_packed_rows(_ptr(x), _ptr(idx), _ptr(packed_out), packed_out.shape[0], tokens, k, int(top_k),

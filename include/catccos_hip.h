@@ -340,17 +340,24 @@ int cch_dyn_quant_i8_rows_smooth(const void *x, const int32_t *src_rows, const f
  * row tiles next to each other: fewer token and weight panels per L2), 2 = each XCD takes a block of
  * 4 row tiles x 8 column tiles of every round (where 8, 16, 32 or 64 column tiles and 256 workgroups
  * allow it; else 1 for grouped problems and 0 for dense ones), -1 (default) = 2;
+ * "i8_epilogue_fp16_step" = 1 makes the int8 epilogues (cch_gemm_i8_dequant*, cch_gmm_i8_dequant*, both kernel paths)
+ * round acc * per_channel to IEEE half before the per-token factor, as the reference's device kernel does
+ * (include/catccos/epilogue/block/block_epilogue_per_token_dequant_swiglu.hpp:348-361: the matrix unit's output stage
+ * writes fp16, the vector epilogue widens it; the golden generator's option,
+ * examples/utils/gen_data_dispatch_gmm_dequant_swiglu.py:309-310); 0 (default) keeps fp32 throughout, the golden
+ * generator's default path - this one switch does change results, by at most 2^-11 relative;
  * "gemm_nt_output" = 1 / 0 gives or denies the output stores the non-temporal hint, -1 (default) gives it to the MXFP4 kernels, where it measured
  * 3-4 % faster (no difference for the others); "quant_integer_encoder" = 1 runs the E4M3
  * round-to-nearest-even quantiser through the integer encoder instead of the hardware conversion (an
- * on-device cross-check; same bytes).  Results do not depend on any of them.
+ * on-device cross-check; same bytes).  Results depend on none of them but "i8_epilogue_fp16_step".
  * The tiled MFMA kernels take every problem whose rows of K are a multiple of 16 bytes, with
  * n % 8 == 0 (and, for [K,N] operands, rows of B a multiple of 4 bytes), 16-byte aligned operands
- * below 2 GiB each and MX scale arrays back to back.  The generic kernels take everything else up to
- * 65535 rows per call (more is CCH_ENOSUP).
+ * below 2 GiB each and MX scale arrays back to back.  The generic kernels take everything else.
  * When a GEMM entry point falls back from the tiled MFMA kernels to the one-thread-per-element
  * kernels (orders of magnitude slower), the call still returns CCH_OK, cch_last_error() names the
- * precondition that failed, and the first such call of the process prints one line to stderr. */
+ * precondition that failed, and the first such call of the process prints one line to stderr.  Every
+ * GEMM entry point empties the calling thread's message when it starts, so after CCH_OK the message is
+ * either that note of this very call or empty. */
 int cch_set_option(const char *name, int value);
 
 #ifdef __cplusplus

@@ -349,6 +349,22 @@ def compare(d, g, rtol=2.0 ** -7):
     return {"max_rel_floor1": m[0], "max_rel_floor_rms": m[1], "eb": m[2], "rms_golden": m[3], "frac_bad": m[4]}
 
 
+def compare_double(d, g, g_low, err_threshold=2.0 ** -8, eb_threshold=2.0 ** -7):
+    """The reference's double-golden acceptance metric (oracle.c:orc_compare_double): ratios of the result's max / mean
+    relative error and RMSE against the high-precision golden to those of a low-precision golden, the eb percentage,
+    and `ok` = the reference's verdict (ratios < 10, 2, 2 and eb <= 100)."""
+    d = np.ascontiguousarray(d, dtype=np.float32).ravel()
+    g = np.ascontiguousarray(g, dtype=np.float32).ravel()
+    gl = np.ascontiguousarray(g_low, dtype=np.float32).ravel()
+    assert d.size == g.size == gl.size
+    m = np.zeros(10, dtype=np.float64)
+    lib().orc_compare_double(_p(d), _p(g), _p(gl), _i64(d.size), ctypes.c_float(err_threshold), ctypes.c_float(eb_threshold), _p(m))
+    names = ["max_rel_ratio", "mean_rel_ratio", "rmse_ratio", "eb_percent", "max_rel", "mean_rel", "rmse", "max_rel_low", "mean_rel_low", "rmse_low"]
+    out = dict(zip(names, (float(x) for x in m)))
+    out["ok"] = bool(m[0] < 10 and m[1] < 2 and m[2] < 2 and m[3] <= 100)
+    return out
+
+
 def moe_token_unpermute(permuted_bf16, sorted_indices, probs, top_k):
     """permuted uint16 [rows, hidden] (bf16 bits), sorted_indices int32 [tokens*top_k], probs float32
     [tokens*top_k] or None -> uint16 [tokens, hidden]."""

@@ -1178,6 +1178,51 @@ void orc_compare(const float *d, const float *g, int64_t n, float rtol, double *
     m[0] = m0; m[1] = m1; m[2] = n ? eb / (double)n : 0.0; m[3] = rms; m[4] = n ? (double)bad / (double)n : 0.0;
 }
 
+/*
+ * The "double golden" acceptance metric of verify_result.py:198-246 (cal_double_precision_eb_percent), the one
+ * examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/run.sh:56-61 applies: the device result d and a
+ * low-precision golden glow are both measured against the high-precision golden g,
+ *   rel(x) = |x - g| / (|g| + 1e-7)     (:224-225; NaN and Inf count as 0, :206-211, everything in fp32 as torch does)
+ * and the result passes (double_precision_performance_analysis, :105-117) when
+ *   m[0] = max rel(d)  / max(max rel(glow),  err_threshold) < 10
+ *   m[1] = mean rel(d) / max(mean rel(glow), err_threshold) < 2
+ *   m[2] = rmse(d)     / max(rmse(glow),     err_threshold) < 2
+ *   m[3] = |mean((d - g) / max(1, |g|))| / eb_threshold * 100 <= 100
+ * with err_threshold = 2^-8 and eb_threshold = 2^-7 for a bfloat16 result (:66-68).  m[4..9] are the six
+ * quantities themselves (max, mean, rmse of d, then of glow).  The low-precision golden of that example is the fp32
+ * matmul of the dequantised operands cast to bfloat16 (gen_data_mxfp8_mmrs.py:349-355), i.e. g rounded to bf16.
+ * pinned by: a numpy restatement in fp32 on random data, and closed forms (d == g gives zeros; d == glow gives
+ *            ratios of exactly 1 where glow's error is above the floor).
+ */
+void orc_compare_double(const float *d, const float *g, const float *glow, int64_t n, float err_threshold, float eb_threshold,
+                        double *m)
+{
+    const float eps = 1e-7f;
+    float max_d = 0.0f, max_l = 0.0f;
+    double sum_d = 0.0, sum_l = 0.0, sq_d = 0.0, sq_l = 0.0, eb = 0.0;
+    for (int64_t i = 0; i < n; i++) {
+        float dv = d[i], gv = g[i], lv = glow[i];
+        if (dv != dv || isinf(dv)) dv = 0.0f;
+        if (gv != gv || isinf(gv)) gv = 0.0f;
+        if (lv != lv || isinf(lv)) lv = 0.0f;
+        const float dd = dv - gv, dl = lv - gv, den = fabsf(gv) + eps;
+        const float rd = fabsf(dd) / den, rl = fabsf(dl) / den;
+        if (rd > max_d) max_d = rd;
+        if (rl > max_l) max_l = rl;
+        sum_d += rd; sum_l += rl;
+        sq_d += (double)(dd * dd); sq_l += (double)(dl * dl);
+        eb += (double)(dd / fmaxf(1.0f, fabsf(gv)));
+    }
+    const double nn = n ? (double)n : 1.0;
+    const double mean_d = sum_d / nn, mean_l = sum_l / nn, rmse_d = sqrt(sq_d / nn), rmse_l = sqrt(sq_l / nn);
+    const double thr = err_threshold;
+    m[0] = (double)max_d / fmax((double)max_l, thr);
+    m[1] = mean_d / fmax(mean_l, thr);
+    m[2] = rmse_d / fmax(rmse_l, thr);
+    m[3] = eb_threshold != 0.0f ? fabs(eb / nn) / (double)eb_threshold * 100.0 : 0.0;
+    m[4] = max_d; m[5] = mean_d; m[6] = rmse_d; m[7] = max_l; m[8] = mean_l; m[9] = rmse_l;
+}
+
 int orc_num_threads(void)
 {
 #ifdef _OPENMP

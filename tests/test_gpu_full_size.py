@@ -1,7 +1,7 @@
-"""The five configurations at their full sizes on the tiled kernels: a sample of at least 512 output rows
-against the oracle's cache-blocked routine (the gate of the small-shape tests; for the grouped ones the
-sample holds the first and the last row of every group and the first row of its last, ragged tile), plus a property that holds at any size and needs
-no oracle - an exact power-of-two scaling (bf16 rounding commutes with a factor of two) or the equality
+"""The five configurations at their full sizes on the tiled kernels: every output row against the oracle's
+cache-blocked routine (the gate of the small-shape tests; the routine is pinned bit for bit to the row-at-a-time
+golden and does a configuration in a second or two on the box's cores), plus a property that holds at any size and
+needs no oracle - an exact power-of-two scaling (bf16 rounding commutes with a factor of two) or the equality
 of the grouped result with per-expert dense calls (same accumulation order along K for every element).
 Inputs are drawn on the GPU and quantised by the library's own quantisers, which have bit-exact parity
 tests of their own."""
@@ -27,21 +27,6 @@ def zipf_groups(rng, t, e):
     return gs
 
 
-def sample_rows(rng, group_sizes, want):
-    """First and last row of every non-empty group, first row of its last 256-row tile, then random rows."""
-    used = int(np.sum(group_sizes))
-    must, r0 = [], 0
-    for g in group_sizes:
-        g = int(g)
-        if g > 0:
-            must += [r0, r0 + g - 1, r0 + ((g - 1) // 256) * 256]
-        r0 += g
-    must = np.unique(np.array(must, dtype=np.int64))
-    rest = np.setdiff1d(np.arange(used, dtype=np.int64), must)
-    more = rng.choice(rest, max(0, min(rest.size, want - must.size)), replace=False)
-    return np.sort(np.concatenate([must, more]))
-
-
 def close(got, want, what):
     m = orc.compare(got, want)
     assert m["max_rel_floor1"] <= TOL and m["max_rel_floor_rms"] <= TOL, (what, m)
@@ -63,9 +48,8 @@ def test_cfg2_w8a8_dequant_8192x4096x8192():
     pt = torch.rand(m, device="cuda") * 0.019 + 0.001
     pc = torch.rand(n, device="cuda") * 0.019 + 0.001
     out = cc.w8a8_matmul_dequant(a, b, pt, pc, 0)
-    rows = np.sort(rng.choice(m, 1024, replace=False)).astype(np.int64)
-    gold = orc.gemm_i8_dequant(a.cpu().numpy(), b.cpu().numpy(), pt.cpu().numpy(), pc.cpu().numpy(), 0, rows=rows, blocked=True)
-    close(out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), gold, "cfg2 sample")
+    gold = orc.gemm_i8_dequant(a.cpu().numpy(), b.cpu().numpy(), pt.cpu().numpy(), pc.cpu().numpy(), 0, blocked=True)
+    close(out.float().cpu().numpy(), gold, "cfg2, every row")
     out2 = cc.w8a8_matmul_dequant(a, b, pt * 2, pc, 0)
     assert torch.equal(out2.float(), out.float() * 2)          # exact: per-token scale times two
 
@@ -77,9 +61,18 @@ def test_cfg3_mxfp8_dense_4096x2048x7168():
     a, sa = cc.mx_quant(torch.randn(m, k, device="cuda").to(torch.bfloat16), "e4m3")
     b, sb = cc.mx_quant_b(torch.randn(k, n, device="cuda").to(torch.bfloat16), "e4m3", trans_b=0)
     out = cc.mx_matmul(a, sa, b, sb, "e4m3", 0)
-    rows = np.sort(rng.choice(m, 1024, replace=False)).astype(np.int64)
-    gold = orc.mx_gmm(a.cpu().numpy(), sa.cpu().numpy(), b.cpu().numpy()[None], sb.cpu().numpy()[None], n, k, orc.E4M3, 0, rows=rows, blocked=True)
-    close(out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), gold, "cfg3 sample")
+    gold = orc.mx_gmm(a.cpu().numpy(), sa.cpu().numpy(), b.cpu().numpy()[None], sb.cpu().numpy()[None], n, k, orc.E4M3, 0, blocked=True)
+    got = out.float().cpu().numpy()
+    close(got, gold, "cfg3, every row")
+    # the reference's own acceptance metric for this operator (double golden: verify_result.py:198-246 as called at
+    # examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/run.sh:56-61; the low-precision golden is the fp32 golden
+    # cast to bf16): mean relative error and RMSE within 2x of that cast's, bias within 2^-7 over every element, the
+    # largest relative error within 10x over the elements that are not cancellations to (almost) nothing
+    low = orc.bf16_to_f32(orc.f32_to_bf16(gold))
+    dg = orc.compare_double(got, gold, low)
+    assert dg["mean_rel_ratio"] < 2 and dg["rmse_ratio"] < 2 and dg["eb_percent"] <= 100, dg
+    keep = np.abs(gold) >= 2.0 ** -7 * np.sqrt(np.mean(gold.astype(np.float64) ** 2))
+    assert orc.compare_double(got[keep], gold[keep], low[keep])["max_rel_ratio"] < 10
     out2 = cc.mx_matmul(a, sa + 1, b, sb, "e4m3", 0)           # every A block scale doubled
     assert torch.equal(out2.float(), out.float() * 2)
 
@@ -95,9 +88,8 @@ def test_cfg4_moe_w8a8_swiglu_8192_tokens_16_experts():
     pt = torch.rand(t, device="cuda") * 0.019 + 0.001
     pc = torch.rand(e, n, device="cuda") * 0.019 + 0.001
     out = cc.gmm_dequant_swiglu(x, w, gs, pt, pc, 0)
-    rows = sample_rows(rng, gs_h, 768)
-    gold = orc.gmm_i8_dequant_swiglu(x.cpu().numpy(), w.cpu().numpy(), gs_h, pt.cpu().numpy(), pc.cpu().numpy(), rows=rows, blocked=True)
-    close(out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), gold, "cfg4 sample")
+    gold = orc.gmm_i8_dequant_swiglu(x.cpu().numpy(), w.cpu().numpy(), gs_h, pt.cpu().numpy(), pc.cpu().numpy(), blocked=True)
+    close(out.float().cpu().numpy(), gold, "cfg4, every row")
     # every expert on its own, as a one-group call over its rows, gives the same bits
     r0 = 0
     for g in range(e):
@@ -122,9 +114,8 @@ def test_cfg5_mx_grouped_16384_tokens_32_experts(fmt, ofmt):
     for g in range(e):
         b[g], sb[g] = cc.mx_quant_b((torch.randn(k, n, device="cuda") * 0.02).to(torch.bfloat16), fmt, trans_b=0)
     out = cc.mx_grouped_matmul(a, sa, b, sb, gs, fmt, 0)
-    rows = sample_rows(rng, gs_h, 768)
-    gold = orc.mx_gmm(a.cpu().numpy(), sa.cpu().numpy(), b.cpu().numpy(), sb.cpu().numpy(), n, k, ofmt, 0, group_sizes=gs_h, rows=rows, blocked=True)
-    close(out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), gold, fmt + " sample")
+    gold = orc.mx_gmm(a.cpu().numpy(), sa.cpu().numpy(), b.cpu().numpy(), sb.cpu().numpy(), n, k, ofmt, 0, group_sizes=gs_h, blocked=True)
+    close(out.float().cpu().numpy(), gold, fmt + ", every row")
     # per-expert dense calls equal the grouped result bit for bit; empty groups contribute nothing
     r0 = 0
     for g in range(e):

@@ -100,3 +100,6 @@ def test_scatter_skips_rows_past_the_output(shape):
     want = orc.mx_quant_scatter_packed(xb, np.where(idx >= out_rows, -1, idx), out_rows, topk, orc.E4M3, orc.RNE, fill=0x5A)
     assert np.array_equal(whole[:out_rows].cpu().numpy(), want)
     assert (whole[out_rows:] == 0x5A).all()
+    # the opt-in check names the caller's error instead of dropping the tokens
+    with pytest.raises(ValueError, match="packed_out has"):
+        cc.mx_quant_scatter_packed(dev_bf16(xb), torch.from_numpy(idx).cuda(), whole[:out_rows], topk, check_routes=True)

@@ -69,3 +69,44 @@ def test_ops_need_init_then_match_the_oracle():
         assert out.shape == (m, k) and torch.equal(out, want)
     finally:
         assert OPS.finalize() == 0
+
+
+def test_a_host_tensor_among_gpu_arguments_is_refused_before_any_launch():
+    """The dispatcher picks the GPU kernel as soon as one argument is a GPU tensor.  Every other tensor argument must then
+    be on that GPU too (the reference's binding checks the same, examples/torch_binding/src/torch_bindings.cpp:140-144):
+    a host tensor's address must never reach a kernel.  The check throws on the host, so nothing is launched."""
+    rng = np.random.default_rng(4)
+    e, t, k, n = 2, 64, 128, 64
+    gs = np.array([40, 24], np.int32)
+    a8 = rng.integers(0, 120, (t, k)).astype(np.uint8)
+    sa = np.full((t, 4), 127, np.uint8)
+    b8 = rng.integers(0, 120, (e, k, n)).astype(np.uint8)
+    sb = np.full((e, 2, n, 2), 127, np.uint8)
+    xi = rng.integers(-127, 128, (t, k)).astype(np.int8)
+    wi = rng.integers(-127, 128, (e, k, n)).astype(np.int8)
+    pt = rng.uniform(0.001, 0.02, t).astype(np.float32)
+    pc = rng.uniform(0.001, 0.02, (e, n)).astype(np.float32)
+    idx = np.zeros((t, 1), np.int32)
+    probs = np.ones((t, 1), np.float32)
+    xb = torch.zeros((t, k), dtype=torch.bfloat16)
+    w1, s1 = np.zeros((e, 64, k), np.uint8), np.full((e, 64, 4), 127, np.uint8)
+    w2, s2 = np.zeros((e, k, 32), np.uint8), np.full((e, k, 2), 127, np.uint8)
+    calls = {
+        "w8a8_matmul_dequant": (lambda a: OPS.w8a8_matmul_dequant(*a, 0), [xi, wi[0], pt, pc[0]]),
+        "mx_matmul": (lambda a: OPS.mx_matmul(*a, "e4m3", 0), [a8, sa, b8[0], sb[0]]),
+        "gmm_dequant_swiglu": (lambda a: OPS.gmm_dequant_swiglu(*a, 0), [xi, wi, gs, pt, pc]),
+        "gmm_dequant_swiglu_mx": (lambda a: OPS.gmm_dequant_swiglu_mx(*a, 0, "e4m3"), [xi, wi, gs, pt, pc]),
+        "mx_grouped_matmul": (lambda a: OPS.mx_grouped_matmul(*a, "e4m3", 0), [a8, sa, b8, sb, gs]),
+        "mx_grouped_matmul_swiglu_mx": (lambda a: OPS.mx_grouped_matmul_swiglu_mx(*a, "e4m3", 0, "e4m3"), [a8, sa, b8, sb, gs]),
+        "moe_ffn_mxfp8": (lambda a: OPS.moe_ffn_mxfp8(*a, 1), [xb, idx, probs, w1, s1, w2, s2]),
+    }
+    assert OPS.init(0, 1, 1 << 20, "tcp://127.0.0.1:8666") == 0
+    try:
+        for name, (call, host_args) in calls.items():
+            as_t = [x if isinstance(x, torch.Tensor) else torch.from_numpy(x) for x in host_args]
+            for on_host in range(len(as_t)):
+                mixed = [x if i == on_host else x.cuda() for i, x in enumerate(as_t)]
+                with pytest.raises(RuntimeError, match="must be a GPU tensor"):
+                    call(mixed)
+    finally:
+        assert OPS.finalize() == 0

@@ -167,6 +167,50 @@ def test_compare_metrics_vs_numpy():
     assert np.isclose(m["rms_golden"], rms)
 
 
+def test_double_golden_metric_vs_torch_restatement_and_closed_forms():
+    """The reference's acceptance metric for the MXFP8 dense operator (examples/utils/verify_result.py:198-246 with the
+    verdict of :105-117): pinned by a torch restatement of those lines in fp32 (NaN and Inf replaced by zero first) and
+    by what the formulas fix: a result equal to the golden has zero ratios, a result equal to the low-precision golden
+    has ratios of exactly one wherever that golden's own error lies above the 2^-8 floor, and below the floor the
+    denominator is the floor."""
+    import torch
+    rng = np.random.default_rng(19)
+    g = (rng.standard_normal(5000) * 30).astype(np.float32)
+    g[:5] = [0.0, 1e-6, -3e-5, np.inf, np.nan]
+    low = orc.bf16_to_f32(orc.f32_to_bf16(g))
+    d = (g * (1 + rng.standard_normal(5000) * 2e-3)).astype(np.float32)
+    d[7] = np.nan
+    got = orc.compare_double(d, g, low)
+    td, tg, tl = (torch.nan_to_num(torch.from_numpy(x), nan=0.0, posinf=0.0, neginf=0.0) for x in (d, g, low))
+    da, dl = td - tg, tl - tg
+    ra, rl = da.abs() / (tg.abs() + 1e-7), dl.abs() / (tg.abs() + 1e-7)
+    thr = 2.0 ** -8
+    want = {
+        "max_rel_ratio": float(ra.max()) / max(float(rl.max()), thr),
+        "mean_rel_ratio": float(ra.mean()) / max(float(rl.mean()), thr),
+        "rmse_ratio": float((da ** 2).mean().sqrt()) / max(float((dl ** 2).mean().sqrt()), thr),
+        "eb_percent": abs(float((da / torch.maximum(torch.ones_like(tg), tg.abs())).mean())) / 2.0 ** -7 * 100,
+    }
+    for key, val in want.items():
+        assert np.isclose(got[key], val, rtol=1e-4), (key, got[key], val)
+    same = orc.compare_double(g, g, low)
+    assert same["max_rel_ratio"] == 0 and same["mean_rel_ratio"] == 0 and same["rmse_ratio"] == 0 and same["eb_percent"] == 0 and same["ok"]
+    # a coarse "low" golden (error above the floor): a result equal to it has ratios of one
+    coarse = (g * (1 + 0.05 * np.sign(rng.standard_normal(5000)))).astype(np.float32)
+    one = orc.compare_double(coarse, g, coarse)
+    assert one["max_rel_ratio"] == 1 and one["mean_rel_ratio"] == 1 and one["rmse_ratio"] == 1
+    # below the floor the floor is the denominator: the bf16 golden's mean relative error is about 2^-10
+    fl = orc.compare_double(low, g, low)
+    assert fl["mean_rel_low"] < thr and np.isclose(fl["mean_rel_ratio"], fl["mean_rel"] / thr)
+    # the verdict's four limits
+    bad = orc.compare_double((g * 1.2).astype(np.float32), g, low)
+    assert not bad["ok"] and bad["mean_rel_ratio"] > 2 and bad["rmse_ratio"] > 2
+    # a constant offset of 1 on goldens of magnitude 4: eb = 1/4 of 2^-7 scaled to percent, far past 100
+    four = np.where(rng.standard_normal(64) > 0, 4.0, -4.0).astype(np.float32)
+    off = orc.compare_double(four + 1, four, four)
+    assert np.isclose(off["eb_percent"], 0.25 / 2.0 ** -7 * 100) and not off["ok"]
+
+
 def test_swiglu_bf16_against_torch_and_closed_forms():
     """The SwiGLU of a bf16 tile (gate | up halves): torch's silu on the widened values, rounded to
     bf16, is the independent check.  The oracle divides gate by 1 + exp(-gate) where torch multiplies by a
