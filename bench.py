@@ -139,6 +139,69 @@ def event_time_ms(fn, steps, warmup, warm_ms=0.0):
     return wall, region, per
 
 
+def measurement_build_clocks(ksteps, group_sizes=None):
+    """With a measurement build of the library (`--lib`, built with -DCCH_PROF): what the tiled GEMM kernel's last launch
+    noted down - per wave the shader clocks spent in each wait and barrier of the K loops, per workgroup the clocks from
+    kernel entry to the first K-step, and per tile its rows, its group and the clocks of its K loop and its epilogue,
+    summarised by rows (in classes of 64) and, for whole tiles, by the rows of their group and by their place in the
+    workgroup's sequence.  {} with the shipped library, which has none of this."""
+    import collections
+    import ctypes
+    import numpy as np
+    from catccos_amd import _abi
+    lib = _abi.lib()
+    try:
+        rd, rdt, rde = lib.cch_prof_read, lib.cch_prof_read_tiles, lib.cch_prof_read_entry
+    except AttributeError:
+        return {}
+    for f in (rd, rdt, rde):
+        f.argtypes = [ctypes.c_void_p]
+    pt = 12   # PROF_TILES of the kernel
+    wbuf, tbuf, ebuf = (ctypes.c_uint64 * (256 * 64))(), (ctypes.c_uint64 * (256 * 2 * pt * 6))(), (ctypes.c_uint64 * (256 * 8))()
+    if rd(wbuf) != 0 or rdt(tbuf) != 0 or rde(ebuf) != 0:
+        return {}
+    out = {}
+    wd = np.frombuffer(wbuf, dtype=np.uint64).reshape(256, 8, 8).astype(np.float64)
+    names = ["total", "lgkm_wait_L0", "barrier_after_L0", "vm_wait_a", "barrier_after_C0", "vm_wait_b", "barrier_after_L1", "barrier_after_C1"]
+    out["shader_cycles_per_wave"] = {g: {n: int(v) for n, v in zip(names, wd[:, sl, :].mean(axis=(0, 1)))}
+                                     for g, sl in (("waves_0_3", slice(0, 4)), ("waves_4_7", slice(4, 8)))}
+    en = np.frombuffer(ebuf, dtype=np.uint64).reshape(256, 8).astype(np.int64)
+    en = en[en[:, 5] > 0]
+    st = (en[:, 1:6] - en[:, 0:5]).mean(axis=0)
+    out["kernel_entry_cycles"] = dict(zip(["group_table", "per_lane_set_up", "first_decode", "first_requests_issued", "wait_and_barrier"],
+                                          (int(v) for v in st)), total=int((en[:, 5] - en[:, 0]).mean()))
+    d = np.frombuffer(tbuf, dtype=np.uint64).reshape(256, 2, pt, 6)
+    recs = []
+    for w in range(256):
+        for i in range(pt):
+            v, k0, k1, e1, dec, ent = (int(x) for x in d[w, 0, i])
+            if k1 == 0 or (i > 0 and k0 <= int(d[w, 0, i - 1][1])):
+                break
+            recs.append({"wg": w, "idx": i, "rows": (v >> 32) & 0xFFFF, "group": v >> 48, "kloop": k1 - k0, "epi": e1 - k1, "dec": dec, "span": e1 - ent})
+    out["tiles_noted"] = len(recs)
+    by_wg = collections.defaultdict(list)
+    for r in recs:
+        by_wg[r["wg"]].append(r)
+    out["decode_of_next_tile_cycles_per_tile"] = int(np.mean([max(r["dec"] for r in rs) / len(rs) for rs in by_wg.values()]))
+    span = np.array([max(r["span"] for r in rs) for rs in by_wg.values()])
+    out["entry_to_last_epilogue_cycles_per_workgroup"] = {"mean": int(span.mean()), "min": int(span.min()), "max": int(span.max())}
+    by_rows = collections.defaultdict(list)
+    for r in recs:
+        by_rows[(r["rows"] + 63) // 64].append(r)
+    out["k_loop_cycles_by_rows_div_64"] = {
+        str(c): {"tiles": len(rs), "mean": int(np.mean([r["kloop"] for r in rs])), "min": int(min(r["kloop"] for r in rs)), "max": int(max(r["kloop"] for r in rs)),
+                 "per_step": int(np.mean([r["kloop"] for r in rs]) / ksteps), "epilogue_mean": int(np.mean([r["epi"] for r in rs]))}
+        for c, rs in sorted(by_rows.items())}
+    whole = [r for r in recs if r["rows"] == 256]
+    if group_sizes is not None and len(group_sizes) > 1:
+        out["whole_tiles_by_rows_of_their_group"] = [
+            {"group_rows": int(group_sizes[g]), "tiles": len(ks), "k_loop_mean": int(np.mean(ks))}
+            for g in np.argsort(group_sizes) for ks in [[r["kloop"] for r in whole if r["group"] == g]] if ks]
+    out["whole_tiles_by_place_in_the_workgroups_sequence"] = [
+        {"place": i, "tiles": len(ks), "k_loop_mean": int(np.mean(ks))} for i in range(pt) for ks in [[r["kloop"] for r in whole if r["idx"] == i]] if ks]
+    return out
+
+
 def clock_under_load(fn, seconds=1.5):
     """Shader clock and power as rocm-smi reports them while fn() runs back to back: the figure that prices
     the published peak (quoted at the 2.4 GHz boost clock) for this kernel.  Returns {} where rocm-smi is
@@ -239,6 +302,8 @@ def main():
     ap.add_argument("--no-clock", action="store_true", help="skip the 1.5 s of back-to-back launches under which rocm-smi is asked for the clock")
     ap.add_argument("--set-option", action="append", default=[], metavar="NAME=VALUE",
                     help="library switch for an A/B run, e.g. gemm_tile_order=0 (cch_set_option)")
+    ap.add_argument("--groups", metavar="E:ROWS", help="the headline kernel on E equal groups of ROWS rows each (E * ROWS tokens) instead of the "
+                    "Zipf-sized groups: how the time follows the tiles and the weight bytes per tile (profiles/)")
     ap.add_argument("--lib", metavar="PATH", help="another build of libcatccos_hip.so (a measurement build, see catccos_amd/build.py)")
     ap.add_argument("--only", choices=["copy", "quant", "cfg2", "cfg3", "cfg4", "cfg5"], help="profiling aid: run only a 512 MiB device copy "
                     "(counter calibration), only the config-1 MX quantiser, or only one of the other configurations' GEMMs; "
@@ -282,6 +347,10 @@ def main():
         name, _, val = kv.partition("=")
         cc.set_option(name, int(val))
     gs_host = zipf_groups(rng, T, E)
+    if args.groups:
+        E, rows_each = (int(v) for v in args.groups.split(":"))
+        T = E * rows_each
+        gs_host = np.full(E, rows_each, dtype=np.int32)
     gs = torch.from_numpy(gs_host).to(dev)
     only_cfg = args.only if args.only in ("cfg2", "cfg3", "cfg4", "cfg5") else None
     flop = 2.0 * T * N * K
@@ -311,23 +380,10 @@ def main():
         achieved = flop / (kernel_ms * 1e-3) / 1e12
 
         clk = clock_under_load(step) if not args.no_clock else {}
-        # an instrumented build of the library (--lib, built with -DCCH_PROF) counts the shader cycles every wave spends in the
-        # waits and barriers of the K loop: mean per wave of the last launch, first and second wave group apart
-        try:
-            import ctypes
-            from catccos_amd import _abi as abi_p
-            rd = abi_p.lib().cch_prof_read
-            rd.argtypes = [ctypes.c_void_p]
-            step()
-            torch.cuda.synchronize()
-            buf = (ctypes.c_uint64 * (256 * 64))()
-            if rd(buf) == 0:
-                d = np.frombuffer(buf, dtype=np.uint64).reshape(256, 8, 8).astype(np.float64)
-                names = ["total", "lgkm_wait_L0", "barrier_after_L0", "vm_wait_C0", "barrier_after_C0", "vm_wait_L1", "barrier_after_L1", "barrier_after_C1"]
-                clk["shader_cycles_per_wave"] = {g: {n: int(v) for n, v in zip(names, d[:, sl, :].mean(axis=(0, 1)))}
-                                                 for g, sl in (("waves_0_3", slice(0, 4)), ("waves_4_7", slice(4, 8)))}
-        except AttributeError:
-            pass
+        # an instrumented build of the library (--lib, built with -DCCH_PROF) notes clocks per wave, workgroup and tile
+        step()
+        torch.cuda.synchronize()
+        clk.update(measurement_build_clocks((K + 127) // 128, gs_host))
         # size-independent sanity of the timed result: sampled rows against the oracle happen in the CPU leg below
         result = {
             "metric": "MXFP8 GMM TFLOP/s (% MFMA peak); MX-quant HBM GB/s (% of peak)",
@@ -346,7 +402,7 @@ def main():
             "vs_baseline": None,
             "dtype": "mxfp8 (e4m3 x e4m3, e8m0 scales, f32 accumulate, bf16 out)",
             "data": "synthetic",
-            "config": {"workload": "MXFP8 grouped matmul, config-5 shapes with E4M3 payload", "experts": E, "tokens": T, "k": K,
+            "config": {"workload": "MXFP8 grouped matmul, config-5 shapes with E4M3 payload" + (" but equal groups (--groups)" if args.groups else ""), "experts": E, "tokens": T, "k": K,
                        "n": N, "trans_b": TRANS_B, "group_sizes": gs_host.tolist()},
             "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(achieved / FP8_PEAK_TFLOPS, 4), "traffic": GMM_TRAFFIC_BYTES,
@@ -459,6 +515,7 @@ def main():
             t2 = [queue_time_ms(lambda: cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, TRANS_B), 30, 60.0)]
             extra["w8a8_dequant_cfg2"] = {"tops": round(2.0 * m2 * n2 * k2 / (np.mean(t2) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t2)) * 1e3, 1)}
             extra["w8a8_dequant_cfg2"]["frac_of_int8_peak"] = round(extra["w8a8_dequant_cfg2"]["tops"] / FP8_PEAK_TFLOPS, 4)
+            extra["w8a8_dequant_cfg2"].update(measurement_build_clocks(k2 // 128))
             if cpu:
                 o2 = cc.w8a8_matmul_dequant(a2, b2, pt2, pc2, TRANS_B).float().cpu().numpy()
                 a2h, b2h, pt2h, pc2h = a2.cpu().numpy(), b2.cpu().numpy(), pt2.cpu().numpy(), pc2.cpu().numpy()
@@ -476,6 +533,7 @@ def main():
             t3 = [queue_time_ms(lambda: cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", TRANS_B), 30, 60.0)]
             extra["mxfp8_dense_cfg3"] = {"tflops": round(2.0 * m3 * n3 * k3 / (np.mean(t3) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t3)) * 1e3, 1)}
             extra["mxfp8_dense_cfg3"]["frac_of_fp8_peak"] = round(extra["mxfp8_dense_cfg3"]["tflops"] / FP8_PEAK_TFLOPS, 4)
+            extra["mxfp8_dense_cfg3"].update(measurement_build_clocks(k3 // 128))
             if cpu:
                 o3 = cc.mx_matmul(a3, sa3, b3, sb3, "e4m3", TRANS_B).float().cpu().numpy()
                 h3 = [t.cpu().numpy() for t in (a3, sa3, b3, sb3)]
@@ -495,6 +553,7 @@ def main():
             tt4 = [queue_time_ms(lambda: cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), 30, 60.0)]
             extra["moe_w8a8_swiglu_cfg4"] = {"tops": round(2.0 * t4 * n4 * k4 / (np.mean(tt4) * 1e-3) / 1e12, 1), "us": round(float(np.mean(tt4)) * 1e3, 1)}
             extra["moe_w8a8_swiglu_cfg4"]["frac_of_int8_peak"] = round(extra["moe_w8a8_swiglu_cfg4"]["tops"] / FP8_PEAK_TFLOPS, 4)
+            extra["moe_w8a8_swiglu_cfg4"].update(measurement_build_clocks(k4 // 128, gs4.cpu().numpy()))
             # the same with the activation leaving as MXFP8 from the epilogue, against the two-kernel chain it replaces
             tf4 = queue_time_ms(lambda: cc.gmm_dequant_swiglu_mx(x4, w4, gs4, pt4, pc4, TRANS_B, "e4m3"), 30, 60.0)
             tc4 = queue_time_ms(lambda: cc.mx_quant(cc.gmm_dequant_swiglu(x4, w4, gs4, pt4, pc4, TRANS_B), "e4m3"), 30, 60.0)
@@ -627,6 +686,7 @@ def main():
             t5 = [queue_time_ms(lambda: cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", TRANS_B), 30, 60.0)]
             extra["mxfp4_grouped_cfg5"] = {"tflops": round(flop / (np.mean(t5) * 1e-3) / 1e12, 1), "us": round(float(np.mean(t5)) * 1e3, 1)}
             extra["mxfp4_grouped_cfg5"]["frac_of_fp4_peak"] = round(extra["mxfp4_grouped_cfg5"]["tflops"] / FP4_PEAK_TFLOPS, 4)
+            extra["mxfp4_grouped_cfg5"].update(measurement_build_clocks(K // 256, gs_host))
             if cpu:
                 o5 = cc.mx_grouped_matmul(a5, sa5, b5, sb5, gs, "e2m1", TRANS_B).float().cpu().numpy()
                 h5 = [t.cpu().numpy() for t in (a5, sa5, b5, sb5)]

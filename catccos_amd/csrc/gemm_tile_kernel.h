@@ -369,6 +369,9 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     // How a step's work is split over the two slot pairs (see `step`): by 64-byte halves of K for [K, N] operands, by row
     // blocks for [N, K] ones.
     constexpr bool KSPLIT = !TB;
+    // MXFP4 [K, N] kernels whose scale rows all start on 4-byte boundaries read the scale dword of a step's second half
+    // in the step's second memory slot (see `step`)
+    constexpr bool SPLIT_SC = KIND == KIND_F4 && KSPLIT && !UA;
 
 #ifdef CCH_PROF
     const uint64_t pf_entry = __builtin_readcyclecounter();
@@ -825,10 +828,12 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
         // Lane group g uses byte g and byte 2 + g of a step's dword: one byte permute brings them to
         // bytes 0 and 2, where the matrix instruction's byte selector finds them.
         uint32_t raw_lo[NSC][MT + NT], raw_hi[NSC][MT + NT];
-        auto read_scales_raw = [&]() {
+        // (d0_c .. d1_c: the dwords of the step to handle, all of them or, where the step's two halves fetch their
+        // scales apart, one each)
+        auto read_scales_raw = [&](auto d0_c, auto d1_c) {
             if constexpr (MX) {
 #pragma unroll
-                for (int d = 0; d < SCALE_DW; d++) {
+                for (int d = decltype(d0_c)::value; d < decltype(d1_c)::value; d++) {
 #pragma unroll
                     for (int s = 0; s < MT; s++) {
                         raw_lo[d][s] = lds_read4_abs(va_sa + d * 4 + s * 512);
@@ -849,12 +854,12 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 }
             }
         };
-        auto finish_scales = [&](auto last_c, int kt) {
+        auto finish_scales = [&](auto last_c, int kt, auto d0_c, auto d1_c) {
             if constexpr (MX) {
                 constexpr bool LAST = decltype(last_c)::value != 0;
                 const int nblk = (p.K + 31) >> 5;
 #pragma unroll
-                for (int d = 0; d < SCALE_DW; d++) {
+                for (int d = decltype(d0_c)::value; d < decltype(d1_c)::value; d++) {
                     uint32_t keep = 0xFFFFFFFFu;
                     if constexpr (LAST) {
                         // blocks of this dword that lie inside K; this lane's two are g and 2 + g
@@ -951,10 +956,17 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
             // Scale group n of a tile is requested three steps before its first step (a reader of the
             // group before it needs its first bytes one step early); group 0 comes with the tile's
             // first step, and MXFP4's group 1 (steps 2-3) with its second.  Prepared in C0 for L1.
+            // SPLIT_SC: two steps before its first step instead, i.e. in the first step of the group before it (the
+            // request lands in the buffer of the group before that one, whose second dwords the other wave group
+            // still reads in the L1 of its last step, one slot after this group's; nothing is read a step early here,
+            // as all scale rows start on 4-byte boundaries).  A request issued in a step's L1 has landed when the
+            // next step's L1 ends, one step before the group's first L0.
             auto next_scale_request = [&]() {
                 ScaleReq sreq{};
                 if constexpr (MX) {
-                    if constexpr (MODE == 0) {
+                    if constexpr (MODE == 0 && SPLIT_SC) {
+                        sreq = prep_scales(((kt + 2) & (SPG - 1)) == 0 && kt >= SPG && kt + 2 < nk_tile, cur, (kt + 2) / SPG);
+                    } else if constexpr (MODE == 0) {
                         sreq = prep_scales(((kt + 3) & (SPG - 1)) == 0 && kt + 3 < nk_tile, cur, (kt + 3) / SPG);
                     } else if constexpr (MODE == 1) {
                         nbase = gi;
@@ -977,12 +989,17 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 constexpr int NB_L0 = NJ / 2, NB_L1 = NJ / 2;
                 constexpr int KL1 = NB_L1 + (MX ? 1 : 0), KC1 = NJ;
                 constexpr int K_PREV_L1 = KL1 + (MODE == 2 ? NPARAM : 0), K_THIS_L1 = KL1 + (MODE == 1 ? NPARAM : 0);
+                // MXFP4 has a scale dword for either half of the step: the second one is read and prepared in L1, with the
+                // half it scales, so that the two memory slots stay alike (SPLIT_SC).  That read comes two slots later
+                // than one in L0, which the scale requests allow for (next_scale_request); a tile's last step reads both
+                // in L0, because the requests for the next tile's scales follow in its L1.
+                constexpr int SC_L0 = SPLIT_SC && MODE != 2 ? 1 : SCALE_DW;
                 // ------------------------------------------------------------------ L0
-                read_scales_raw();
+                read_scales_raw(IC<0>{}, IC<SC_L0>{});
 #pragma unroll
                 for (int j = 0; j < NT; j++) fb[j][0] = frag_b(stg_c, 0, j);
                 __builtin_amdgcn_sched_barrier(0);
-                finish_scales(IC<MODE != 0>{}, kt);
+                finish_scales(IC<MODE != 0>{}, kt, IC<0>{}, IC<SC_L0>{});
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int i = 0; i < NBLK; i++) fa[i & 1][i >> 1] = frag_a(stg_c, 0, i);
@@ -1017,8 +1034,12 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 __builtin_amdgcn_sched_barrier(0);
                 { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b1); }
                 // ------------------------------------------------------------------ L1
+                read_scales_raw(IC<SC_L0>{}, IC<SCALE_DW>{});
 #pragma unroll
                 for (int j = 0; j < NT; j++) fb[j][0] = frag_b(stg_c, 1, j);
+                __builtin_amdgcn_sched_barrier(0);
+                finish_scales(IC<MODE != 0>{}, kt, IC<SC_L0>{}, IC<SCALE_DW>{});
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int i = 0; i < NBLK; i++) fa[i & 1][i >> 1] = frag_a(stg_c, 1, i);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1060,13 +1081,13 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 constexpr int THIS_L1 = MODE == 1 ? NL1 + NPARAM : NL1;
                 constexpr int NB0 = NBLK < 2 ? NBLK : 2, NB1 = NBLK - NB0;   // row blocks of either slot pair
                 // ------------------------------------------------------------------ L0
-                read_scales_raw();
+                read_scales_raw(IC<0>{}, IC<SCALE_DW>{});
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++)
 #pragma unroll
                     for (int j = 0; j < NT; j++) fb[j][ks] = frag_b(stg_c, ks, j);
                 __builtin_amdgcn_sched_barrier(0);
-                finish_scales(IC<MODE != 0>{}, kt);   // while the B fragments arrive; its inputs die before the A fragments need registers
+                finish_scales(IC<MODE != 0>{}, kt, IC<0>{}, IC<SCALE_DW>{});   // while the B fragments arrive; its inputs die before the A fragments need registers
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++)
