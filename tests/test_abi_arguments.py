@@ -95,6 +95,11 @@ def test_routing_and_unpermute_arguments():
     rejected(L.cch_moe_token_unpermute(P, P, None, P, 8, 4, 64, 9, None), "top_k")
     rejected(L.cch_moe_token_unpermute(P, P, None, P, -1, 4, 64, 2, None), "negative")
     rejected(L.cch_set_option(b"no_such_option", 1), "unknown option")
+    rejected(L.cch_set_option(b"gemm_balance_rounds", 1), "unknown option")   # a switch that no longer exists
+    # the switches the header documents are all known (set to their defaults: nothing changes)
+    for name, default in ((b"force_generic_gemm", 0), (b"require_tiled_gemm", 0), (b"gemm_tile_order", -1), (b"gemm_nt_output", -1),
+                          (b"i8_epilogue_fp16_step", 0), (b"quant_integer_encoder", 0), (b"routing_three_launches", 0)):
+        assert L.cch_set_option(name, default) == _abi.OK, name
 
 
 def test_empty_problems_succeed_without_a_device():

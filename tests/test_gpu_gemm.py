@@ -598,6 +598,20 @@ def test_fall_back_note_describes_the_call_that_fell_back_only():
     torch.cuda.synchronize()
 
 
+def test_generic_kernels_take_more_than_65535_rows():
+    """The one-thread-per-element kernels put the rows on the grid's x axis: a problem the tiled kernels do not take
+    (K no multiple of 16 bytes) runs at any row count (the reference takes such shapes; an earlier form of the generic
+    path stopped at 65535 rows)."""
+    rng = np.random.default_rng(41)
+    t, k, n = 70000, 40, 8
+    a = rng.integers(-127, 128, (t, k)).astype(np.int8)
+    b = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    pt = rng.uniform(0.001, 0.02, t).astype(np.float32)
+    pc = rng.uniform(0.001, 0.02, n).astype(np.float32)
+    got = out_f32(cc.w8a8_matmul_dequant(dev(a), dev(b), dev(pt), dev(pc), 0))
+    assert_close(got, orc.gemm_i8_dequant(a, b, pt, pc), "generic path, 70000 rows")
+
+
 # ---------------------------------------------------------------- tile order
 
 def test_grouped_tile_order_covers_every_tile_once():
