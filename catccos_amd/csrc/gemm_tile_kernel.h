@@ -1021,16 +1021,29 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 // ------------------------------------------------------------------ C0
                 // (int8 and FP4 take two MFMAs per accumulator and half of K: all row blocks on the first 32 bytes, then
                 // all on the second, so that an accumulator's two MFMAs are not neighbours in the pipe)
+                // (what the coming slots need is worked out between the matrix instructions, in the issue cycles that
+                // the wave has to spare while the pipe is busy: behind the last one it would hold up the barrier, and
+                // with it the other group's first matrix instruction, past the moment the pipe falls free)
+                Tail rq_tl{};
+                uint32_t rq_boff = 0;
+                ScaleReq sreq{};
                 static_for<(KIND == KIND_F8 ? 1 : 2)>([&](auto h_c) {
                     static_for<NBLK>([&](auto i_c) {
-                        constexpr int i = decltype(i_c)::value;
-                        mfma_block(IC<FIRST>{}, IC<0>{}, i_c, fa[i & 1][i >> 1], IC<(KIND == KIND_F8 ? -1 : decltype(h_c)::value)>{});
+                        constexpr int i = decltype(i_c)::value, h = decltype(h_c)::value;
+                        mfma_block(IC<FIRST>{}, IC<0>{}, i_c, fa[i & 1][i >> 1], IC<(KIND == KIND_F8 ? -1 : h)>{});
+                        if constexpr (h == 0 && i == 0) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            rq_tl = tail_of(rq_kt);
+                            rq_boff = boff_of(rq_kt);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        if constexpr (h == 0 && i == (NBLK > 1 ? 1 : 0)) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            sreq = next_scale_request();
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
                     });
                 });
-                __builtin_amdgcn_sched_barrier(0);
-                const Tail rq_tl = tail_of(rq_kt);
-                const uint32_t rq_boff = boff_of(rq_kt);
-                const ScaleReq sreq = next_scale_request();
                 __builtin_amdgcn_sched_barrier(0);
                 { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b1); }
                 // ------------------------------------------------------------------ L1
@@ -1053,10 +1066,16 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                 { PROF_BEGIN(t_); CCH_WAIT_VM_LGKM0(KC1 + STORES + NB_L0 + K_THIS_L1); PROF_END(t_, pf_wb); }
                 { PROF_BEGIN(t_); CCH_BARRIER(); PROF_END(t_, pf_b2); }
                 // ------------------------------------------------------------------ C1
+                // (the scale read addresses of the next step move on behind the first matrix instructions, not behind the last)
                 static_for<NJ>([&](auto q_c) {
                     constexpr int q = decltype(q_c)::value;
                     if constexpr (q < NBLK) {
                         mfma_block(IC<0>{}, IC<1>{}, q_c, fa[q & 1][q >> 1], IC<(KIND == KIND_F8 ? -1 : 0)>{});
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    if constexpr (q == 0) {
+                        if constexpr (MODE == 2) prep_scale_reads(nbase);
+                        else advance_scale_reads(gbase, kt);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                     issue_a(rq, rq_tl, stg_c, q_c);
@@ -1068,8 +1087,6 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
                         mfma_block(IC<0>{}, IC<1>{}, q_c, fa[q & 1][q >> 1], IC<1>{});
                     });
                 }
-                if constexpr (MODE == 2) prep_scale_reads(nbase);
-                else advance_scale_reads(gbase, kt);
                 __builtin_amdgcn_sched_barrier(0);
                 // this group's A rows of the next step (requested in the previous step's C1) must have landed:
                 // younger are the stores and this step's L0, L1 and C1
