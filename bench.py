@@ -28,9 +28,9 @@ FP8_PEAK_TFLOPS = 5000.0   # MI355X dense FP8 / INT8 MFMA, published
 FP4_PEAK_TFLOPS = 10100.0  # MI355X dense FP4 MFMA, published
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 # Bytes per launch of the headline kernel between the L2s and the fabric (Infinity Cache and HBM behind it), from two
-# rocprofv3 --pmc runs of this script (FETCH_SIZE 1 135 866 KiB x 2.000, WRITE_SIZE 131 072 KiB x 1.000; the factors are
+# rocprofv3 --pmc runs of this script (FETCH_SIZE 1 128 767 KiB x 2.000, WRITE_SIZE 131 072 KiB x 1.000; the factors are
 # what the same counters read for a 512 MiB device copy, `--only copy`).  Algorithmic bytes: 1 224 212 480.
-GMM_TRAFFIC_BYTES = 2460471296
+GMM_TRAFFIC_BYTES = 2445932544
 
 
 def zipf_groups(rng, t, e):
