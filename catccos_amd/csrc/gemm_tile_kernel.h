@@ -377,7 +377,16 @@ __global__ __launch_bounds__(TILE_THREADS) void gemm_tile_kernel(GemmProblem p)
     const uint64_t pf_entry = __builtin_readcyclecounter();
 #endif
     __shared__ GroupTable tab;
-    if (threadIdx.x < 64) build_group_table_dpp(tab, p.group_sizes, p.num_groups, p.T);
+    if (p.group_sizes == nullptr && p.num_groups == 1) {
+        // a dense problem: one group of all rows, no rows past it
+        if (threadIdx.x == 0) {
+            const int tiles = (p.T + BM - 1) / BM;
+            tab.row_start[0] = 0; tab.row_start[1] = p.T; tab.row_start[2] = p.T;
+            tab.tile_start[0] = 0; tab.tile_start[1] = tiles; tab.tile_start[2] = tiles;
+        }
+    } else if (threadIdx.x < 64) {
+        build_group_table_dpp(tab, p.group_sizes, p.num_groups, p.T);
+    }
     __syncthreads();
 
 #ifdef CCH_PROF
