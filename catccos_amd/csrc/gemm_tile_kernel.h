@@ -17,7 +17,10 @@
 //   * A wave alternates between a memory slot (LDS fragment reads, global -> LDS requests) and a
 //     matrix slot (MFMAs only), the slots are separated by workgroup barriers, and the second
 //     group runs one slot behind the first: while one wave of a SIMD issues matrix instructions
-//     its neighbour fetches, and the next slot they swap.  A K-step is four slots per wave.
+//     its neighbour fetches, and the next slot they swap.  A K-step is four slots per wave.  A wave issues in
+//     order: a matrix slot holds nothing that can wait (no LDS read, no wait for data), and what it prepares for
+//     the coming slots sits between its first matrix instructions, so that the wave is at the slot's barrier
+//     before the matrix pipe falls free and the other group's first instruction finds it so.
 //     B stored [K, N] (a step's panel is 128 K-rows, so its two 64-byte halves of K are separate rows):
 //       L0  read the first half of the step: B fragments and the A fragments of the wave's row blocks;
 //           request the second-half K-rows of B of step k+1
