@@ -480,7 +480,7 @@ def _both_paths(fn):
     return outs
 
 
-@pytest.mark.parametrize("seed", range(32))
+@pytest.mark.parametrize("seed", range(96))
 def test_tiled_matches_generic_on_random_groups(seed):
     """Random expert counts, group sizes (empty, one-row, many-tile groups, rows of no group), K-step
     counts, widths and both weight layouts: the tiled kernels against the one-thread-per-output
